@@ -1,0 +1,217 @@
+"""The cache manager: which pages and which state slot every live request holds.
+
+Layers are put in groups by what their mixers keep (`CacheNeed`): layers that
+keep all keys and values of a given (kv_heads, head_dim) share a group, layers
+that keep a window of them form another, and so on. A group has a page pool of
+its own and, per request, one block table that serves all its layers: page p of
+a group exists once in each of the group's layers' planes. A request's pages
+go back to the pool when it ends, and, in a windowed group, as soon as every
+position a page covers lies behind the window. Mixers that keep a state of
+fixed size get one slot per live request, the same slot number in all such
+groups; it is handed out at admission and taken back when the request ends.
+
+The reference has one homogeneous pool with reference counts for a prefix
+index (src/qwen3_from_scratch/inference/block_manager.py:26-138); the
+arithmetic of `pages_missing` is its `can_allocate` (:90-95). There is no
+prefix index here.
+"""
+
+from dataclasses import dataclass, field
+
+from .pages import OutOfPages, PagePool
+
+
+@dataclass
+class _Group:
+    kv_heads: int
+    head_dim: int
+    window: int
+    planes: list
+    pool: PagePool
+
+
+@dataclass
+class _StateGroup:
+    shape: tuple
+    dtype: object
+    planes: list
+
+
+@dataclass
+class _Held:
+    length: int = 0                      # tokens whose keys are in the cache
+    reserved: int = 0                    # tokens beyond `length` that pages are held for
+    tables: list = field(default_factory=list)   # per group: page of each block, -1 once given back
+    slot: int = -1
+
+
+class CacheManager:
+    def __init__(self, needs, page_size, num_pages, max_requests):
+        """`needs`: one CacheNeed (or None) per cache plane of the model.
+        `num_pages`: pages in every group's pool. `max_requests`: state slots."""
+        if page_size <= 0:
+            raise ValueError("page_size must be positive")
+        self.page_size = page_size
+        self.max_requests = max_requests
+        self.groups = []
+        self.state_groups = []
+        self.group_of_plane = []
+        self.state_group_of_plane = []
+        for plane, need in enumerate(needs):
+            g = s = -1
+            if need is not None and need.paged:
+                key = (need.kv_heads, need.head_dim, need.window)
+                for i, grp in enumerate(self.groups):
+                    if (grp.kv_heads, grp.head_dim, grp.window) == key:
+                        g = i
+                if g < 0:
+                    self.groups.append(_Group(*key, planes=[], pool=PagePool(num_pages)))
+                    g = len(self.groups) - 1
+                self.groups[g].planes.append(plane)
+            if need is not None and need.has_state:
+                key = (tuple(need.state_shape), need.state_dtype)
+                for i, grp in enumerate(self.state_groups):
+                    if (grp.shape, grp.dtype) == key:
+                        s = i
+                if s < 0:
+                    self.state_groups.append(_StateGroup(*key, planes=[]))
+                    s = len(self.state_groups) - 1
+                self.state_groups[s].planes.append(plane)
+            self.group_of_plane.append(g)
+            self.state_group_of_plane.append(s)
+        self._slots = list(range(max_requests - 1, -1, -1))
+        self._requests = {}
+        self.fresh_slots = []     # slots handed out since the storage last cleared them
+
+    # ---- requests ----
+    def has(self, request_id):
+        return request_id in self._requests
+
+    def live(self):
+        return list(self._requests)
+
+    def length(self, request_id):
+        return self._requests[request_id].length
+
+    def slot(self, request_id):
+        return self._requests[request_id].slot
+
+    def admit(self, request_id):
+        if request_id in self._requests:
+            raise KeyError("request %r is already live" % (request_id,))
+        if not self._slots:
+            raise OutOfPages("all %d request slots are taken" % self.max_requests)
+        held = _Held(tables=[[] for _ in self.groups], slot=self._slots.pop())
+        self._requests[request_id] = held
+        self.fresh_slots.append(held.slot)
+        return held.slot
+
+    # ---- growth ----
+    def _blocks_for(self, tokens):
+        return -(-tokens // self.page_size)
+
+    def pages_missing(self, request_id, new_tokens):
+        """Per group, the pages still to be taken before `new_tokens` more can be written."""
+        held = self._requests.get(request_id)
+        length = held.length if held else 0
+        target = self._blocks_for(length + new_tokens)
+        return [target - (len(held.tables[g]) if held else 0) for g in range(len(self.groups))]
+
+    def can_grow(self, request_id, new_tokens, spare=None):
+        """True if every group's pool can cover `new_tokens` more for the request.
+        `spare`, if given, is a per-group count of pages already promised to
+        others in this step; it is updated when the answer is True."""
+        if request_id not in self._requests and not self._slots:
+            return False
+        missing = self.pages_missing(request_id, new_tokens)
+        taken = spare if spare is not None else [0] * len(self.groups)
+        for g, grp in enumerate(self.groups):
+            if max(0, missing[g]) + taken[g] > grp.pool.num_free:
+                return False
+        if spare is not None:
+            for g in range(len(self.groups)):
+                spare[g] += max(0, missing[g])
+        return True
+
+    def reserve(self, request_id, new_tokens):
+        """Take the pages that positions length .. length + new_tokens - 1 need.
+        Either all groups get theirs or nothing changes."""
+        held = self._requests[request_id]
+        missing = self.pages_missing(request_id, new_tokens)
+        for g, grp in enumerate(self.groups):
+            if missing[g] > grp.pool.num_free:
+                raise OutOfPages(
+                    "request %r needs %d more pages of group %d, %d are free"
+                    % (request_id, missing[g], g, grp.pool.num_free))
+        for g, grp in enumerate(self.groups):
+            for _ in range(max(0, missing[g])):
+                held.tables[g].append(grp.pool.take())
+        held.reserved = max(held.reserved, new_tokens)
+
+    def commit(self, request_id, new_tokens):
+        """The step wrote `new_tokens` more positions. Pages of windowed groups
+        that no later query can see are given back."""
+        held = self._requests[request_id]
+        if new_tokens > held.reserved:
+            raise RuntimeError("commit of %d tokens, only %d reserved" % (new_tokens, held.reserved))
+        held.length += new_tokens
+        held.reserved = 0
+        for g, grp in enumerate(self.groups):
+            if grp.window <= 0:
+                continue
+            # the next query sits at position >= length and sees keys > its position - window
+            first_needed = held.length - grp.window + 1
+            dead_blocks = max(0, first_needed) // self.page_size
+            table = held.tables[g]
+            for b in range(min(dead_blocks, len(table))):
+                if table[b] >= 0:
+                    grp.pool.give(table[b])
+                    table[b] = -1
+
+    def release(self, request_id):
+        """The request has ended: everything it holds goes back."""
+        held = self._requests.pop(request_id)
+        for g, grp in enumerate(self.groups):
+            for page in held.tables[g]:
+                if page >= 0:
+                    grp.pool.give(page)
+        self._slots.append(held.slot)
+
+    # ---- views ----
+    def block_table(self, request_id, group):
+        return self._requests[request_id].tables[group]
+
+    def num_free(self, group=0):
+        return self.groups[group].pool.num_free
+
+    def num_pages(self, group=0):
+        return self.groups[group].pool.num_pages
+
+    def capacity_tokens(self):
+        """Tokens one request can hold at most (bounded by the smallest pool)."""
+        if not self.groups:
+            return 1 << 62
+        return min(g.pool.num_pages for g in self.groups) * self.page_size
+
+    def audit(self):
+        """Every page is free or held by exactly one request; slots likewise."""
+        for g, grp in enumerate(self.groups):
+            seen = set()
+            for rid, held in self._requests.items():
+                for page in held.tables[g]:
+                    if page < 0:
+                        continue
+                    if page in seen:
+                        raise AssertionError("page %d of group %d is held twice" % (page, g))
+                    if not grp.pool.is_held(page):
+                        raise AssertionError("page %d of group %d is held by %r but marked free" % (page, g, rid))
+                    seen.add(page)
+            if len(seen) + grp.pool.num_free != grp.pool.num_pages:
+                raise AssertionError(
+                    "group %d: %d held + %d free != %d pages"
+                    % (g, len(seen), grp.pool.num_free, grp.pool.num_pages))
+        slots = [h.slot for h in self._requests.values()]
+        if len(set(slots)) != len(slots) or set(slots) & set(self._slots):
+            raise AssertionError("a request slot is held twice")
+        if len(slots) + len(self._slots) != self.max_requests:
+            raise AssertionError("a request slot is lost")

@@ -1,0 +1,68 @@
+"""The device memory behind the cache manager's page numbers and slots."""
+
+from dataclasses import dataclass
+
+import torch
+
+
+@dataclass
+class LayerCacheView:
+    """What one mixer sees of the cache in one step."""
+
+    keys: torch.Tensor = None          # (pages, kv_heads, page_size, head_dim)
+    values: torch.Tensor = None
+    block_table: torch.Tensor = None   # int32 (B, W), this step's requests in batch order
+    writes: bool = True
+    state: torch.Tensor = None         # (slots, *state_shape); index with batch.state_slots
+
+
+class CacheStorage:
+    """Per paged group one tensor (planes, 2, pages, kv_heads, page_size, head_dim)
+    in the activation dtype: within a page, one head's rows are contiguous, so a
+    workgroup that serves one key head streams page_size * head_dim elements at a
+    time. Per state group one tensor (planes, slots, *shape), zeroed per slot
+    at admission."""
+
+    def __init__(self, manager, act_dtype, device):
+        self.manager = manager
+        self.device = torch.device(device)
+        self.paged = []
+        for grp in manager.groups:
+            self.paged.append(torch.zeros(
+                (len(grp.planes), 2, grp.pool.num_pages, grp.kv_heads, manager.page_size, grp.head_dim),
+                dtype=act_dtype, device=self.device))
+        self.states = []
+        for grp in manager.state_groups:
+            self.states.append(torch.zeros(
+                (len(grp.planes), manager.max_requests) + tuple(grp.shape),
+                dtype=grp.dtype, device=self.device))
+        self._block_tables = None
+
+    def bytes(self):
+        return sum(t.numel() * t.element_size() for t in self.paged + self.states)
+
+    def clear_fresh_slots(self):
+        fresh, self.manager.fresh_slots = self.manager.fresh_slots, []
+        if fresh and self.states:
+            index = torch.tensor(fresh, dtype=torch.long, device=self.device)
+            for t in self.states:
+                t[:, index] = 0
+
+    def bind(self, block_tables):
+        """`block_tables`: per paged group the step's int32 (B, W) device tensor."""
+        self._block_tables = block_tables
+
+    def view(self, plane, writes=True):
+        m = self.manager
+        view = LayerCacheView(writes=writes)
+        g = m.group_of_plane[plane]
+        if g >= 0:
+            local = m.groups[g].planes.index(plane)
+            view.keys = self.paged[g][local, 0]
+            view.values = self.paged[g][local, 1]
+            view.block_table = self._block_tables[g]
+        s = m.state_group_of_plane[plane]
+        if s >= 0:
+            local = m.state_groups[s].planes.index(plane)
+            view.state = self.states[s][local]
+        return view

@@ -1,0 +1,104 @@
+"""One step's batch: the tokens it brings and where they sit."""
+
+from dataclasses import dataclass, field
+
+import numpy as np
+import torch
+
+
+@dataclass
+class StepEntry:
+    """A request's next tokens in this step and the places among them (0-based
+    indices into `tokens`) whose logits are wanted."""
+
+    request_id: object
+    tokens: list
+    want: list = field(default_factory=list)
+
+
+@dataclass
+class StepBatch:
+    """Device tensors (int32) and host numbers that describe the packed batch.
+
+    Rows of all entries are packed on one token axis without padding, in the
+    order of the entries (src/qwen3_from_scratch/inference/model_worker.py:177-210
+    builds the same quantities as separate uploads and a global context).
+    """
+
+    num_tokens: int
+    num_seqs: int
+    token_ids: torch.Tensor        # (T,)
+    positions: torch.Tensor        # (T,) absolute position of each token in its request
+    seq_index: torch.Tensor        # (T,) which entry a token belongs to
+    cu_seqlens_q: torch.Tensor     # (B+1,) prefix sums of tokens per entry
+    kv_lens: torch.Tensor          # (B,) keys visible after this step's write
+    state_slots: torch.Tensor      # (B,) per-request slot of fixed-size state
+    logits_rows: torch.Tensor      # (R,) packed rows whose logits are wanted
+    max_q_len: int
+    max_kv_len: int
+    q_lens: list                   # host copies
+    kv_lens_host: list
+
+
+def pack_step(entries, lengths, slots, tables_per_group, device, min_table_width=1):
+    """Build the batch on the host and move it to the device in one copy.
+
+    `lengths[i]`: tokens entry i's request already has in the cache.
+    `tables_per_group[g][i]`: the request's page list in group g (-1 = given back).
+    Returns (StepBatch, [block table per group]).
+    """
+    B = len(entries)
+    q_lens = [len(e.tokens) for e in entries]
+    T = sum(q_lens)
+    kv = [lengths[i] + q_lens[i] for i in range(B)]
+    rows = []
+    offset = 0
+    for i, e in enumerate(entries):
+        for w in e.want:
+            if not (0 <= w < q_lens[i]):
+                raise ValueError("request %r wants place %d of %d tokens" % (e.request_id, w, q_lens[i]))
+            rows.append(offset + w)
+        offset += q_lens[i]
+    R = len(rows)
+    widths = []
+    for tables in tables_per_group:
+        widths.append(max([min_table_width] + [len(t) for t in tables]))
+    total = 3 * T + (B + 1) + 2 * B + R + sum(B * w for w in widths)
+    host = np.empty(total, dtype=np.int32)
+    o = 0
+
+    def put(values, n):
+        nonlocal o
+        host[o:o + n] = values
+        sl = slice(o, o + n)
+        o += n
+        return sl
+
+    tok = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries]) if T else np.zeros(0, np.int64)
+    pos = np.concatenate([np.arange(lengths[i], kv[i]) for i in range(B)]) if T else np.zeros(0, np.int64)
+    seq = np.repeat(np.arange(B), q_lens) if T else np.zeros(0, np.int64)
+    s_tok = put(tok, T)
+    s_pos = put(pos, T)
+    s_seq = put(seq, T)
+    s_cu = put(np.concatenate([[0], np.cumsum(q_lens)]), B + 1)
+    s_kv = put(kv, B)
+    s_slot = put(slots, B)
+    s_rows = put(rows, R)
+    s_tables = []
+    for tables, w in zip(tables_per_group, widths):
+        flat = np.full((B, w), -1, dtype=np.int32)
+        for i, t in enumerate(tables):
+            flat[i, :len(t)] = t
+        s_tables.append((put(flat.reshape(-1), B * w), w))
+    dev = torch.from_numpy(host)
+    if torch.device(device).type == "cuda":
+        dev = dev.pin_memory().to(device, non_blocking=True)
+    batch = StepBatch(
+        num_tokens=T, num_seqs=B,
+        token_ids=dev[s_tok], positions=dev[s_pos], seq_index=dev[s_seq],
+        cu_seqlens_q=dev[s_cu], kv_lens=dev[s_kv], state_slots=dev[s_slot], logits_rows=dev[s_rows],
+        max_q_len=max(q_lens) if q_lens else 0, max_kv_len=max(kv) if kv else 0,
+        q_lens=q_lens, kv_lens_host=kv,
+    )
+    block_tables = [dev[sl].view(B, w) for sl, w in s_tables]
+    return batch, block_tables

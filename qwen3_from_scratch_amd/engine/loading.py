@@ -1,0 +1,34 @@
+"""From a model folder (or a configuration and a seed) to a runner."""
+
+import torch
+
+from ..config.registry import load_model_config
+from ..models.decoder import build_model
+from ..parts.base import Precision
+from ..weights import Checkpoint, RandomWeights
+
+
+def load_model(model_dir, dtype="bfloat16", device="cuda"):
+    """Read config.json, pick the model by its architecture, load model.safetensors."""
+    config = load_model_config(model_dir)
+    model = build_model(config, Precision.named(dtype), device)
+    model.load(Checkpoint(model_dir))
+    model.config = config
+    return model
+
+
+def random_model(config, dtype="bfloat16", device="cuda", seed=0, std=0.02, norm_jitter=0.1):
+    """A model of `config` with seeded random weights drawn on the device."""
+    model = build_model(config, Precision.named(dtype), device)
+    on = device if torch.device(device).type == "cuda" else None
+    model.load(RandomWeights(model.tensors(), seed=seed, std=std, norm_jitter=norm_jitter, generate_on=on))
+    model.config = config
+    return model
+
+
+def load_runner(model_dir, dtype="bfloat16", device="cuda", page_size=16, max_tokens=8192, max_requests=32):
+    from .runner import ModelRunner
+
+    model = load_model(model_dir, dtype, device)
+    num_pages = -(-max_tokens // page_size)
+    return ModelRunner(model, page_size, num_pages, max_requests)

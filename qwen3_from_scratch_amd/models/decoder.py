@@ -1,0 +1,116 @@
+"""A decoder put together from a ModelSpec: embedding, position encoding, the
+layers in their run order, final norm, head. It knows parts only through their
+interfaces, never by architecture."""
+
+import torch
+
+from ..parts.base import build_part
+from ..weights.checkpoint import check_tensors
+
+
+class _Layer:
+    def __init__(self, spec, precision, device, position):
+        p = spec.prefix
+        self.block = build_part(spec.block, p, precision, device)
+        self.mixer = build_part(spec.mixer, p + "." + spec.mixer_prefix, precision, device)
+        self.feed_forward = build_part(spec.feed_forward, p + "." + spec.feed_forward_prefix, precision, device)
+        self.mixer_norm = build_part(spec.mixer_norm, p + "." + spec.mixer_norm_prefix, precision, device)
+        self.feed_forward_norm = build_part(
+            spec.feed_forward_norm, p + "." + spec.feed_forward_norm_prefix, precision, device)
+        if hasattr(self.mixer, "attach_position"):
+            self.mixer.attach_position(position)
+        self.block.attach(self.mixer, self.feed_forward, self.mixer_norm, self.feed_forward_norm)
+
+    def parts(self):
+        return (self.block, self.mixer, self.feed_forward, self.mixer_norm, self.feed_forward_norm)
+
+
+class DecoderModel:
+    def __init__(self, spec, precision, device):
+        self.spec = spec
+        self.precision = precision
+        self.device = torch.device(device)
+        self.embedding = build_part(spec.embedding, spec.embedding_prefix, precision, device)
+        self.position = build_part(spec.position, "", precision, device)
+        self.layers = [_Layer(ls, precision, device, self.position) for ls in spec.layers]
+        self.final_norm = build_part(spec.final_norm, spec.final_norm_prefix, precision, device)
+        self.head = build_part(spec.head, spec.head_prefix, precision, device)
+        # each run-order entry that owns a cache gets a plane; readers point at the owner's
+        self.plane_of_step = []
+        self.plane_needs = []
+        for i, step in enumerate(spec.order):
+            if step.reads_cache_of is None:
+                mixer = self.layers[step.layer].mixer
+                need = mixer.cache_need() if hasattr(mixer, "cache_need") else None
+                self.plane_of_step.append(len(self.plane_needs))
+                self.plane_needs.append(need)
+            else:
+                self.plane_of_step.append(self.plane_of_step[step.reads_cache_of])
+
+    def parts(self):
+        yield self.embedding
+        yield self.position
+        for layer in self.layers:
+            yield from layer.parts()
+        yield self.final_norm
+        yield self.head
+
+    def tensors(self):
+        names = {}
+        for part in self.parts():
+            for name, shape in part.tensors().items():
+                if name in names and tuple(names[name]) != tuple(shape):
+                    raise ValueError("tensor %s is wanted with shapes %s and %s" % (name, names[name], shape))
+                names[name] = tuple(shape)
+        return names
+
+    def load(self, source):
+        """Check the source's names and shapes against the model, then load."""
+        check_tensors(source, self.tensors(), ignorable=self.spec.ignorable_tensors)
+        kept = {}
+
+        def fetch(name, dtype=None, keep=True):
+            key = (name, dtype)
+            if key in kept:
+                return kept[key]
+            tensor = source.get(name, self.device)
+            if dtype is not None and tensor.dtype != dtype:
+                if not tensor.dtype.is_floating_point:
+                    raise ValueError("%s is an integer table and cannot become %s" % (name, dtype))
+                tensor = tensor.to(dtype)
+            if keep:
+                kept[key] = tensor
+            return tensor
+
+        with torch.no_grad():
+            for part in self.parts():
+                part.load(fetch)
+        return self
+
+    @torch.no_grad()
+    def forward(self, batch, cache):
+        """Logits (R, V) float32 at batch.logits_rows, from batch.token_ids and
+        what `cache` holds. `cache.view(plane, writes)` gives a mixer its view."""
+        x = self.embedding.forward(batch.token_ids)
+        x = self.position.on_embeddings(x, batch)
+        pending = None
+        for i, step in enumerate(self.spec.order):
+            view = cache.view(self.plane_of_step[i], writes=step.reads_cache_of is None)
+            x, pending = self.layers[step.layer].block.forward(x, pending, batch, view)
+        h = self.final_norm.forward(x, delta=pending, rows=batch.logits_rows)
+        return self.head.forward(h)
+
+
+def expected_tensors(spec):
+    """{name: shape} of every tensor a model of this spec loads."""
+    from ..parts.base import Precision
+
+    return DecoderModel(spec, Precision(torch.bfloat16), "cpu").tensors()
+
+
+def build_model(config, precision, device):
+    """The model of `config`'s architecture, unloaded."""
+    from ..config.registry import lookup_architecture
+
+    _, build_spec = lookup_architecture(config.architecture)
+    return DecoderModel(build_spec(config), precision, device)

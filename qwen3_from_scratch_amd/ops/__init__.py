@@ -1,0 +1,277 @@
+"""The operations the model is made of, each a hand-written HIP kernel.
+
+Every function checks its operands on the host (device, dtype, contiguity and
+the shapes the kernel's grid assumes) and then launches on the current HIP
+stream. Tensors must live on the GPU: there is no host implementation, and a
+missing or unbuildable extension raises `ExtensionError`.
+
+Activations and matrices are bfloat16 or float32 (the same for all operands of
+one call unless stated); the residual stream, rotation tables, softmax
+statistics and logits are float32 in both modes.
+"""
+
+import ctypes
+
+import torch
+
+from .build import ExtensionError, build_all, library, loaded_libraries
+
+__all__ = [
+    "ExtensionError",
+    "build_all",
+    "loaded_libraries",
+    "embed_rows",
+    "rmsnorm",
+    "rope_table",
+    "qk_norm_rope_store",
+    "paged_attention",
+    "swiglu",
+    "linear",
+    "sample",
+]
+
+_DT = {torch.float32: 0, torch.bfloat16: 1}
+
+
+class OperandError(ValueError):
+    """An operand has a shape, dtype or placement the kernel does not take."""
+
+
+def _ptr(t):
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _need(cond, message):
+    if not cond:
+        raise OperandError(message)
+
+
+def _dev(*tensors):
+    for t in tensors:
+        if t is None:
+            continue
+        _need(t.is_cuda, "operands must be on the GPU; there is no host implementation")
+        _need(t.is_contiguous(), "operands must be contiguous")
+
+
+def _check(status, what):
+    if status != 0:
+        raise RuntimeError("%s failed: HIP error %d" % (what, status))
+
+
+def embed_rows(ids, table, out=None):
+    """out[t, :] = float32(table[ids[t], :]). ids int32 (T,), table (V, H)."""
+    _dev(ids, table, out)
+    _need(ids.dtype == torch.int32 and ids.dim() == 1, "ids must be int32 (T,)")
+    _need(table.dim() == 2 and table.dtype in _DT, "table must be (V, H) bfloat16 or float32")
+    T, (V, H) = ids.shape[0], table.shape
+    if out is None:
+        out = torch.empty((T, H), dtype=torch.float32, device=table.device)
+    _need(out.shape == (T, H) and out.dtype == torch.float32, "out must be float32 (T, H)")
+    if T:
+        _check(library("elementwise").q3_embed_rows(
+            _ptr(ids), _ptr(table), _ptr(out), T, H, V, _DT[table.dtype], _stream()), "embed_rows")
+    return out
+
+
+def swiglu(gate_up, out=None):
+    """out = silu(gate) * up for gate_up = [gate | up] of shape (T, 2I)."""
+    _dev(gate_up, out)
+    _need(gate_up.dim() == 2 and gate_up.shape[1] % 2 == 0 and gate_up.dtype in _DT,
+          "gate_up must be (T, 2I) bfloat16 or float32")
+    T, I = gate_up.shape[0], gate_up.shape[1] // 2
+    if out is None:
+        out = torch.empty((T, I), dtype=gate_up.dtype, device=gate_up.device)
+    _need(out.shape == (T, I) and out.dtype == gate_up.dtype, "out must be (T, I) of the input's dtype")
+    if T:
+        _check(library("elementwise").q3_swiglu(
+            _ptr(gate_up), _ptr(out), T, I, _DT[gate_up.dtype], _stream()), "swiglu")
+    return out
+
+
+def rmsnorm(x, weight, eps, out_dtype, delta=None, rows=None, write_back=True, out=None):
+    """Root-mean-square norm of the float32 residual stream.
+
+    For each output row r (source row s = rows[r], or r when rows is None):
+    v = x[s] + delta[s] (delta optional), written back to x[s] if `write_back`
+    and delta is given; out[r] = v * rsqrt(mean(v^2) + eps) * weight, rounded
+    once to `out_dtype`. All arithmetic is float32.
+    """
+    _dev(x, weight, delta, rows, out)
+    _need(x.dim() == 2 and x.dtype == torch.float32, "x must be float32 (T, H)")
+    T, H = x.shape
+    _need(weight.shape == (H,) and weight.dtype in _DT, "weight must be (H,) bfloat16 or float32")
+    _need(out_dtype in _DT, "out_dtype must be bfloat16 or float32")
+    if delta is not None:
+        _need(delta.shape == (T, H) and delta.dtype == out_dtype,
+              "delta must be (T, H) of the activation dtype")
+    n_out = T
+    if rows is not None:
+        _need(rows.dtype == torch.int32 and rows.dim() == 1, "rows must be int32 (R,)")
+        n_out = rows.shape[0]
+    if out is None:
+        out = torch.empty((n_out, H), dtype=out_dtype, device=x.device)
+    _need(out.shape == (n_out, H) and out.dtype == out_dtype, "out must be (rows, H) of out_dtype")
+    if n_out:
+        _check(library("norm").q3_rmsnorm(
+            _ptr(x), _ptr(delta), _ptr(weight), _ptr(rows), _ptr(out), n_out, T, H,
+            ctypes.c_float(eps), _DT[out_dtype], _DT[weight.dtype],
+            1 if (write_back and delta is not None) else 0, _stream()), "rmsnorm")
+    return out
+
+
+def rope_table(inv_freq, max_positions):
+    """table[p] = [cos(p * inv_freq) | sin(p * inv_freq)], float32 (P, 2 * len(inv_freq))."""
+    _dev(inv_freq)
+    _need(inv_freq.dtype == torch.float32 and inv_freq.dim() == 1, "inv_freq must be float32 (D/2,)")
+    half = inv_freq.shape[0]
+    table = torch.empty((max_positions, 2 * half), dtype=torch.float32, device=inv_freq.device)
+    _check(library("rotary").q3_rope_table(
+        _ptr(inv_freq), _ptr(table), max_positions, half, _stream()), "rope_table")
+    return table
+
+
+def qk_norm_rope_store(qkv, num_q_heads, num_kv_heads, head_dim, positions, seq_index,
+                       q_weight=None, k_weight=None, eps=0.0, table=None,
+                       block_table=None, k_cache=None, v_cache=None):
+    """Per-head RMSNorm of q and k, rotation by position, and the cache write, in one pass.
+
+    qkv (T, (Hq + 2 Hkv) D) holds [q heads | k heads | v heads]. q heads are
+    normalised with `q_weight`, rotated, and written back in place. k heads
+    are normalised with `k_weight`, rotated, and stored; v heads are stored as
+    they are. The store goes to page block_table[seq_index[t], pos // page] at
+    offset pos % page of caches shaped (pages, Hkv, page, D); entries below
+    zero are skipped, and nothing is stored when no cache is given. Norm and
+    rotation are each skipped when their operand is None. The rotation pairs
+    element i with i + R/2 over the first R = table.shape[1] elements.
+    """
+    _dev(qkv, positions, seq_index, q_weight, k_weight, table, block_table, k_cache, v_cache)
+    Hq, Hkv, D = num_q_heads, num_kv_heads, head_dim
+    _need(qkv.dim() == 2 and qkv.shape[1] == (Hq + 2 * Hkv) * D and qkv.dtype in _DT,
+          "qkv must be (T, (Hq + 2 Hkv) D) bfloat16 or float32")
+    T = qkv.shape[0]
+    _need(1 <= D <= 512, "head_dim must be in 1..512")
+    for t in (positions, seq_index):
+        _need(t.dtype == torch.int32 and t.shape == (T,), "positions and seq_index must be int32 (T,)")
+    w_dtype = 0
+    if (q_weight is None) != (k_weight is None):
+        raise OperandError("q_weight and k_weight are given together or not at all")
+    if q_weight is not None:
+        _need(q_weight.shape == (D,) and k_weight.shape == (D,) and q_weight.dtype in _DT
+              and k_weight.dtype == q_weight.dtype, "norm weights must be (D,), same dtype")
+        w_dtype = _DT[q_weight.dtype]
+    rotary_dim, max_pos = 0, 0
+    if table is not None:
+        _need(table.dim() == 2 and table.dtype == torch.float32, "table must be float32 (P, R)")
+        max_pos, rotary_dim = table.shape
+        _need(rotary_dim % 2 == 0 and rotary_dim <= D, "rotary dim must be even and at most D")
+    page, stride = 0, 0
+    if k_cache is not None:
+        _need(v_cache is not None and block_table is not None, "a cache needs k, v and a block table")
+        _need(k_cache.dim() == 4 and k_cache.shape == v_cache.shape and k_cache.shape[1] == Hkv
+              and k_cache.shape[3] == D and k_cache.dtype == qkv.dtype and v_cache.dtype == qkv.dtype,
+              "caches must be (pages, Hkv, page, D) of the activation dtype")
+        _need(block_table.dim() == 2 and block_table.dtype == torch.int32, "block_table must be int32 (B, W)")
+        page, stride = k_cache.shape[2], block_table.shape[1]
+    if T:
+        _check(library("rotary").q3_qk_norm_rope_store(
+            _ptr(qkv), _ptr(q_weight), _ptr(k_weight), w_dtype, ctypes.c_float(eps),
+            _ptr(table), rotary_dim, max_pos, _ptr(positions), _ptr(seq_index),
+            _ptr(block_table), stride, 0 if block_table is None else block_table.shape[0],
+            _ptr(k_cache), _ptr(v_cache), page, 0 if k_cache is None else k_cache.shape[0],
+            T, Hq, Hkv, D, _DT[qkv.dtype], _stream()), "qk_norm_rope_store")
+    return qkv
+
+
+def paged_attention(q, num_q_heads, k_cache, v_cache, block_table, cu_seqlens_q, kv_lens,
+                    max_q_len, max_kv_len, scale, window=0, out=None):
+    """Causal softmax attention of packed query rows over paged keys and values.
+
+    q is (T, Hq, D) seen through a row stride (a view of the qkv buffer is
+    fine). Sequence b owns rows cu_seqlens_q[b]..cu_seqlens_q[b+1]; its keys
+    0..kv_lens[b]-1 lie in pages block_table[b, j // page]; its query row i sits
+    at position kv_lens[b] - q_len + i and sees keys at positions <= its own
+    and, if window > 0, fewer than `window` behind it. Query head h reads
+    key head h // (Hq / Hkv). Softmax statistics and accumulation are float32.
+    """
+    _dev(k_cache, v_cache, block_table, cu_seqlens_q, kv_lens, out)
+    _need(q.is_cuda and q.dim() == 3 and q.stride(2) == 1 and q.stride(1) == q.shape[2],
+          "q must be (T, Hq, D) with contiguous heads")
+    T, Hq, D = q.shape
+    _need(Hq == num_q_heads, "q's head count differs from num_q_heads")
+    _need(q.dtype in _DT and k_cache.dtype == q.dtype and v_cache.dtype == q.dtype,
+          "q and the caches must share bfloat16 or float32")
+    _need(k_cache.dim() == 4 and k_cache.shape == v_cache.shape and k_cache.shape[3] == D,
+          "caches must be (pages, Hkv, page, D)")
+    Hkv, page = k_cache.shape[1], k_cache.shape[2]
+    _need(Hq % Hkv == 0, "query heads must be a multiple of key heads")
+    _need(D % 16 == 0 and 16 <= D <= 256, "head_dim must be a multiple of 16 in 16..256, found %d" % D)
+    B = kv_lens.shape[0]
+    _need(cu_seqlens_q.dtype == torch.int32 and cu_seqlens_q.shape == (B + 1,), "cu_seqlens_q must be int32 (B+1,)")
+    _need(kv_lens.dtype == torch.int32, "kv_lens must be int32 (B,)")
+    _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.shape[0] >= B,
+          "block_table must be int32 (B, W)")
+    _need(block_table.shape[1] * page >= max_kv_len, "block_table is narrower than the longest sequence")
+    if out is None:
+        out = torch.empty((T, Hq * D), dtype=q.dtype, device=q.device)
+    _need(out.shape == (T, Hq * D) and out.dtype == q.dtype, "out must be (T, Hq D)")
+    if T and B:
+        _check(library("attention").q3_paged_attention(
+            _ptr(q), q.stride(0), _ptr(out), _ptr(k_cache), _ptr(v_cache), k_cache.shape[0],
+            _ptr(block_table), block_table.shape[1], _ptr(cu_seqlens_q), _ptr(kv_lens),
+            B, T, Hq, Hkv, D, page, ctypes.c_float(scale), int(window), int(max_q_len),
+            int(max_kv_len), _DT[q.dtype], _stream()), "paged_attention")
+    return out
+
+
+def linear(x, weight, out_dtype=None, out=None):
+    """out = x @ weight^T with float32 accumulation. x (M, K), weight (N, K).
+
+    float32 operands take a float32 kernel with no reduced-precision mode.
+    """
+    _dev(x, weight, out)
+    _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1], "x (M, K) and weight (N, K)")
+    _need(x.dtype in _DT and weight.dtype == x.dtype, "x and weight must share bfloat16 or float32")
+    M, K = x.shape
+    N = weight.shape[0]
+    out_dtype = out_dtype or x.dtype
+    _need(out_dtype in _DT, "out dtype must be bfloat16 or float32")
+    _need(not (x.dtype == torch.float32 and out_dtype != torch.float32), "float32 inputs give float32 output")
+    if out is None:
+        out = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    _need(out.shape == (M, N) and out.dtype == out_dtype, "out must be (M, N) of out_dtype")
+    if M:
+        _check(library("gemm").q3_linear(
+            _ptr(x), _ptr(weight), _ptr(out), M, N, K, _DT[x.dtype], _DT[out_dtype], _stream()), "linear")
+    return out
+
+
+def sample(logits, temperature, top_k, seed, counter, out=None):
+    """One token per row of float32 logits (R, V).
+
+    Row r: temperature[r] <= 0 takes the arg-max (lowest index among equals).
+    Otherwise it draws from softmax(logits / temperature) restricted, when
+    top_k[r] > 0, to logits not below the k-th largest; the draw is the
+    arg-max of logits / temperature + Gumbel noise from a counter-based
+    generator keyed by (seed[r], counter[r], column), so a request's tokens do
+    not depend on what else is in the batch.
+    """
+    _dev(logits, temperature, top_k, seed, counter, out)
+    _need(logits.dim() == 2 and logits.dtype == torch.float32, "logits must be float32 (R, V)")
+    R, V = logits.shape
+    _need(temperature.shape == (R,) and temperature.dtype == torch.float32, "temperature float32 (R,)")
+    _need(top_k.shape == (R,) and top_k.dtype == torch.int32, "top_k int32 (R,)")
+    _need(seed.shape == (R,) and seed.dtype == torch.int64, "seed int64 (R,)")
+    _need(counter.shape == (R,) and counter.dtype == torch.int32, "counter int32 (R,)")
+    if out is None:
+        out = torch.empty((R,), dtype=torch.int32, device=logits.device)
+    _need(out.shape == (R,) and out.dtype == torch.int32, "out int32 (R,)")
+    if R:
+        _check(library("sampling").q3_sample(
+            _ptr(logits), _ptr(temperature), _ptr(top_k), _ptr(seed), _ptr(counter), _ptr(out),
+            R, V, _stream()), "sample")
+    return out

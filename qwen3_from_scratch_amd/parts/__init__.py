@@ -1,0 +1,6 @@
+"""The parts a model is put together from. Importing registers them."""
+
+from .base import CacheNeed, Part, PartSpec, Precision, build_part
+from . import attention, block, embedding, feed_forward, head, norm, position  # noqa: F401
+
+__all__ = ["CacheNeed", "Part", "PartSpec", "Precision", "build_part"]

@@ -1,0 +1,89 @@
+"""Softmax attention over the paged cache, with grouped heads."""
+
+import torch
+
+from .. import ops
+from ..config.registry import register_part
+from .base import CacheNeed, Part
+
+
+@register_part("mixer", "attention")
+class PagedAttention(Part):
+    """q, k, v projections (no bias), optional per-head RMSNorm of q and k before
+    rotation, rotation by the position part's table, cache write, causal
+    attention over everything the cache holds for the request, output
+    projection (src/qwen3_from_scratch/models/self_attn.py:310-342). The
+    three projections are one matrix [q | k | v]. This step's keys and values
+    are written first and attention then reads old and new alike from the
+    cache (self_attn.py:382-384), which is what makes portions of prompts and
+    single decoded tokens uniform.
+
+    Parameters: hidden_size, num_heads, num_kv_heads, head_dim, qk_norm (bool),
+    qk_norm_eps, window (0 = all keys), scale (None = head_dim ** -0.5).
+    """
+
+    def __init__(self, prefix, precision, device, hidden_size, num_heads, num_kv_heads, head_dim,
+                 qk_norm=True, qk_norm_eps=1e-6, window=0, scale=None):
+        super().__init__(prefix, precision, device)
+        if num_heads % num_kv_heads:
+            raise ValueError("num_heads (%d) must be a multiple of num_kv_heads (%d)"
+                             % (num_heads, num_kv_heads))
+        self.hidden_size = hidden_size
+        self.num_heads = num_heads
+        self.num_kv_heads = num_kv_heads
+        self.head_dim = head_dim
+        self.qk_norm = bool(qk_norm)
+        self.qk_norm_eps = float(qk_norm_eps)
+        self.window = int(window)
+        self.scale = float(scale) if scale is not None else head_dim ** -0.5
+        self.position = None
+        self.qkv = self.out = self.q_weight = self.k_weight = None
+
+    def attach_position(self, position):
+        self.position = position
+
+    def cache_need(self):
+        return CacheNeed(kv_heads=self.num_kv_heads, head_dim=self.head_dim, window=self.window)
+
+    def tensors(self):
+        H, Hq, Hkv, D = self.hidden_size, self.num_heads, self.num_kv_heads, self.head_dim
+        names = {
+            self._name("q_proj.weight"): (Hq * D, H),
+            self._name("k_proj.weight"): (Hkv * D, H),
+            self._name("v_proj.weight"): (Hkv * D, H),
+            self._name("o_proj.weight"): (H, Hq * D),
+        }
+        if self.qk_norm:
+            names[self._name("q_norm.weight")] = (D,)
+            names[self._name("k_norm.weight")] = (D,)
+        return names
+
+    def load(self, fetch):
+        act = self.precision.act
+        Hq, Hkv, D = self.num_heads, self.num_kv_heads, self.head_dim
+        self.qkv = torch.empty(((Hq + 2 * Hkv) * D, self.hidden_size), dtype=act, device=self.device)
+        self.qkv[: Hq * D].copy_(fetch(self._name("q_proj.weight"), act, keep=False))
+        self.qkv[Hq * D: (Hq + Hkv) * D].copy_(fetch(self._name("k_proj.weight"), act, keep=False))
+        self.qkv[(Hq + Hkv) * D:].copy_(fetch(self._name("v_proj.weight"), act, keep=False))
+        self.out = fetch(self._name("o_proj.weight"), act)
+        if self.qk_norm:
+            self.q_weight = fetch(self._name("q_norm.weight"))
+            self.k_weight = fetch(self._name("k_norm.weight"))
+
+    def forward(self, x, batch, cache):
+        Hq, Hkv, D = self.num_heads, self.num_kv_heads, self.head_dim
+        qkv = ops.linear(x, self.qkv)
+        table = self.position.rotation_table() if self.position is not None else None
+        ops.qk_norm_rope_store(
+            qkv, Hq, Hkv, D, batch.positions, batch.seq_index,
+            q_weight=self.q_weight, k_weight=self.k_weight, eps=self.qk_norm_eps, table=table,
+            block_table=cache.block_table if cache.writes else None,
+            k_cache=cache.keys if cache.writes else None,
+            v_cache=cache.values if cache.writes else None,
+        )
+        q = qkv[:, : Hq * D].unflatten(1, (Hq, D))
+        o = ops.paged_attention(
+            q, Hq, cache.keys, cache.values, cache.block_table, batch.cu_seqlens_q, batch.kv_lens,
+            batch.max_q_len, batch.max_kv_len, self.scale, window=self.window,
+        )
+        return ops.linear(o, self.out)

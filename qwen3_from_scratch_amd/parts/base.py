@@ -1,0 +1,105 @@
+"""What every part is: a named, parameterised piece with tensors of its own.
+
+A part is described by a `PartSpec` (kind, registered name, parameters) and
+built by `build_part`. It declares the checkpoint tensors it needs
+(`tensors()`), receives them (`load()`), and computes (`forward` with the
+signature of its kind, see each module). Parameters carry every size and
+constant; a part never looks at a model configuration and does not know which
+model it is in.
+"""
+
+from dataclasses import dataclass, field
+
+import torch
+
+from ..config.registry import lookup_part
+
+
+@dataclass(frozen=True)
+class Precision:
+    """Compute dtypes of one engine instance. Activations, matrices and the
+    cache share `act`; the residual stream and logits are float32."""
+
+    act: torch.dtype
+
+    @classmethod
+    def named(cls, name):
+        name = str(name).replace("torch.", "")
+        if name in ("bfloat16", "bf16"):
+            return cls(torch.bfloat16)
+        if name in ("float32", "fp32"):
+            return cls(torch.float32)
+        raise ValueError("dtype must be bfloat16 or float32, found %r" % (name,))
+
+    @property
+    def name(self):
+        return "bfloat16" if self.act == torch.bfloat16 else "float32"
+
+
+@dataclass(frozen=True)
+class PartSpec:
+    kind: str
+    name: str
+    params: tuple = ()
+
+    @classmethod
+    def of(cls, kind, name, **params):
+        return cls(kind, name, tuple(sorted(params.items())))
+
+    def get(self, key, default=None):
+        return dict(self.params).get(key, default)
+
+    def with_params(self, **more):
+        merged = dict(self.params)
+        merged.update(more)
+        return PartSpec(self.kind, self.name, tuple(sorted(merged.items())))
+
+
+class Part:
+    """Base class. `prefix` is the checkpoint name prefix of the part's tensors."""
+
+    def __init__(self, prefix, precision, device):
+        self.prefix = prefix
+        self.precision = precision
+        self.device = torch.device(device)
+
+    def tensors(self):
+        """{checkpoint tensor name: shape} of everything this part loads."""
+        return {}
+
+    def load(self, fetch):
+        """`fetch(name, dtype=None)` returns the tensor on the device, in its
+        stored dtype or converted to `dtype`; equal requests share one tensor."""
+
+    def _name(self, leaf):
+        return self.prefix + "." + leaf if self.prefix else leaf
+
+
+def build_part(spec, prefix, precision, device):
+    cls = lookup_part(spec.kind, spec.name)
+    return cls(prefix=prefix, precision=precision, device=device, **dict(spec.params))
+
+
+@dataclass
+class CacheNeed:
+    """What a mixer keeps per request between steps.
+
+    paged: keys and values that grow by one row per token, (kv_heads, head_dim)
+    each, all of them kept (window == 0) or the last `window`. state: a tensor
+    of fixed `state_shape` and `state_dtype` per request. A mixer may need
+    neither, either or both.
+    """
+
+    kv_heads: int = 0
+    head_dim: int = 0
+    window: int = 0
+    state_shape: tuple = ()
+    state_dtype: torch.dtype = torch.float32
+
+    @property
+    def paged(self):
+        return self.kv_heads > 0
+
+    @property
+    def has_state(self):
+        return len(self.state_shape) > 0

@@ -1,0 +1,34 @@
+"""Norms over the last dimension."""
+
+import torch
+
+from .. import ops
+from ..config.registry import register_part
+from .base import Part
+
+
+@register_part("norm", "rms")
+class RMSNorm(Part):
+    """y = x * rsqrt(mean(x^2) + eps) * weight, eps inside the root, plain weight
+    (src/qwen3_from_scratch/models/norm.py:18-22,51-53). It reads the float32
+    residual stream and can fold the pending addition `x += delta` into the
+    same pass; the sum, the mean and the products are float32 and the result
+    is rounded once."""
+
+    def __init__(self, prefix, precision, device, size, eps):
+        super().__init__(prefix, precision, device)
+        self.size = size
+        self.eps = float(eps)
+        self.weight = None
+
+    def tensors(self):
+        return {self._name("weight"): (self.size,)}
+
+    def load(self, fetch):
+        self.weight = fetch(self._name("weight"))
+
+    def forward(self, x, delta=None, rows=None):
+        """Normalised rows in the activation dtype. With `delta`, x += delta
+        first (in place, unless `rows` selects a subset: then x is left alone)."""
+        return ops.rmsnorm(x, self.weight, self.eps, self.precision.act, delta=delta,
+                           rows=rows, write_back=rows is None)

@@ -1,0 +1,152 @@
+"""Tiny configurations, model folders and trace builders shared by the tests."""
+
+import os
+
+import torch
+
+from qwen3_from_scratch_amd.config import ModelConfig
+from qwen3_from_scratch_amd.weights import write_random_model
+
+# Two configurations that differ in every size and option; neither has a size
+# that is a power of two throughout. A third exercises odd head counts.
+TINY = {
+    "A": dict(
+        config=dict(architectures=["Qwen3ForCausalLM"], vocab_size=256, hidden_size=64, hidden_act="silu",
+                    num_hidden_layers=2, max_position_embeddings=256, num_attention_heads=4,
+                    num_key_value_heads=2, head_dim=16, intermediate_size=128, rms_norm_eps=1e-6,
+                    rope_theta=10000.0, tie_word_embeddings=True),
+        seed=11, std=0.02, norm_jitter=0.1, page_size=16),
+    "B": dict(
+        config=dict(architectures=["Qwen3ForCausalLM"], vocab_size=384, hidden_size=96, hidden_act="silu",
+                    num_hidden_layers=3, max_position_embeddings=512, num_attention_heads=8,
+                    num_key_value_heads=2, head_dim=32, intermediate_size=224, rms_norm_eps=1e-5,
+                    rope_theta=1000000.0, tie_word_embeddings=False),
+        seed=23, std=0.03, norm_jitter=0.2, page_size=8),
+    "C": dict(
+        config=dict(architectures=["Qwen3ForCausalLM"], vocab_size=331, hidden_size=72, hidden_act="silu",
+                    num_hidden_layers=2, max_position_embeddings=640, num_attention_heads=6,
+                    num_key_value_heads=3, head_dim=48, intermediate_size=200, rms_norm_eps=3e-6,
+                    rope_theta=50000.0, tie_word_embeddings=False),
+        seed=37, std=0.05, norm_jitter=0.3, page_size=16),
+}
+
+
+def tiny_config(name):
+    return ModelConfig.from_dict(TINY[name]["config"])
+
+
+def make_folder(folder, name):
+    t = TINY[name]
+    write_random_model(folder, tiny_config(name), seed=t["seed"], std=t["std"], norm_jitter=t["norm_jitter"])
+    return folder
+
+
+def random_tokens(n, vocab, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
+
+
+# ---- traces: lists of steps; a step is (entries, ends); an entry is (id, tokens, want) ----
+
+def trace_whole(requests):
+    """Each request alone and whole, all places wanted."""
+    steps = []
+    for rid, toks in requests.items():
+        steps.append(([(rid, toks, list(range(len(toks))))], [rid]))
+    return steps
+
+
+def trace_tail_decoded(requests, tail=32):
+    """Most of each request in one step, its last `tail` tokens one by one."""
+    steps = []
+    for rid, toks in requests.items():
+        head = max(len(toks) - tail, 1)
+        steps.append(([(rid, toks[:head], list(range(head)))], []))
+        for i in range(head, len(toks)):
+            steps.append(([(rid, [toks[i]], [0])], [rid] if i == len(toks) - 1 else []))
+        if head == len(toks):
+            steps[-1] = (steps[-1][0], [rid])
+    return steps
+
+
+def trace_portions(requests, sizes=(24, 7, 2, 16, 3, 2, 33, 5, 2, 9)):
+    """Each request alone, cut into portions of changing size, down to two tokens."""
+    steps = []
+    for rid, toks in requests.items():
+        at, k = 0, 0
+        while at < len(toks):
+            n = min(sizes[k % len(sizes)], len(toks) - at)
+            k += 1
+            last = at + n == len(toks)
+            steps.append(([(rid, toks[at:at + n], list(range(n)))], [rid] if last else []))
+            at += n
+    return steps
+
+
+def trace_mixed(requests, max_live=4, seed=0, decode_tail=12):
+    """Up to `max_live` requests at a time; each goes through its prompt in
+    portions of random size and through its last `decode_tail` tokens one at a
+    time, so that portions of some sit beside single tokens of others; a
+    request may sit a step out. New requests start as earlier ones end."""
+    g = torch.Generator().manual_seed(seed)
+
+    def rnd(n):
+        return int(torch.randint(0, n, (1,), generator=g))
+
+    waiting = list(requests.items())
+    live = {}
+    steps = []
+    while waiting or live:
+        while waiting and len(live) < max_live:
+            rid, toks = waiting.pop(0)
+            live[rid] = [toks, 0]
+        entries, ends = [], []
+        for rid in list(live):
+            toks, at = live[rid]
+            if len(live) > 1 and rnd(5) == 0:
+                continue                                   # sits this step out
+            left = len(toks) - at
+            if left <= decode_tail:
+                n = 1
+            else:
+                n = min(left - decode_tail, 2 + rnd(30))
+            entries.append((rid, toks[at:at + n], list(range(n))))
+            live[rid][1] = at + n
+            if at + n == len(toks):
+                ends.append(rid)
+                del live[rid]
+        if entries:
+            steps.append((entries, ends))
+    return steps
+
+
+def run_trace(runner, steps):
+    """Drive a ModelRunner through a trace; returns {(id, position): logits row}."""
+    from qwen3_from_scratch_amd.engine import StepEntry
+
+    got = {}
+    for entries, ends in steps:
+        where = []
+        for rid, toks, want in entries:
+            base = runner.length(rid)
+            where += [(rid, base + w) for w in want]
+        logits = runner.step([StepEntry(rid, toks, want) for rid, toks, want in entries])
+        logits = logits.float().cpu()
+        for key, row in zip(where, logits):
+            got[key] = row
+        for rid in ends:
+            runner.finish(rid)
+        runner.manager.audit()
+    return got
+
+
+def max_live_tokens(steps, page=64):
+    """The most tokens live requests hold at any time, each rounded up to `page`."""
+    held, worst = {}, 0
+    for entries, ends in steps:
+        for rid, toks, _ in entries:
+            held[rid] = held.get(rid, 0) + len(toks)
+        worst = max(worst, sum(-(-n // page) * page for n in held.values()))
+        for rid in ends:
+            held.pop(rid, None)
+    return worst

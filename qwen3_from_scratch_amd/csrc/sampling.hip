@@ -1,0 +1,150 @@
+// One token per row of float32 logits: arg-max, or a draw from the softmax at a
+// temperature, optionally among the k best, as the arg-max of
+// logit / temperature + Gumbel noise.
+#include "common.h"
+
+#include <math.h>
+
+// Philox-4x32 with 10 rounds (Salmon et al., "Parallel random numbers: as easy
+// as 1, 2, 3"): a counter-based generator, so the noise of (seed, counter,
+// column) does not depend on which rows share the launch.
+__device__ inline void philox4x32_10(uint32_t c[4], uint32_t k0, uint32_t k1) {
+#pragma unroll
+  for (int round = 0; round < 10; ++round) {
+    const uint32_t hi0 = __umulhi(0xD2511F53u, c[0]), lo0 = 0xD2511F53u * c[0];
+    const uint32_t hi1 = __umulhi(0xCD9E8D57u, c[2]), lo1 = 0xCD9E8D57u * c[2];
+    const uint32_t n0 = hi1 ^ c[1] ^ k0, n2 = hi0 ^ c[3] ^ k1;
+    c[0] = n0; c[1] = lo1; c[2] = n2; c[3] = lo0;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+}
+
+// Larger float <=> larger key.
+__device__ inline uint32_t order_key(float f) {
+  const uint32_t u = __float_as_uint(f);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+struct Best {
+  float value;
+  int index;
+};
+
+__device__ inline Best better(Best a, Best b) {
+  if (b.value > a.value || (b.value == a.value && b.index < a.index)) return b;
+  return a;
+}
+
+__device__ inline Best block_best(Best mine, Best* scratch) {
+#pragma unroll
+  for (int off = Q3_WAVE / 2; off > 0; off >>= 1) {
+    Best other;
+    other.value = __shfl_xor(mine.value, off, Q3_WAVE);
+    other.index = __shfl_xor(mine.index, off, Q3_WAVE);
+    mine = better(mine, other);
+  }
+  const int lane = threadIdx.x & (Q3_WAVE - 1), wave = threadIdx.x / Q3_WAVE;
+  __syncthreads();
+  if (lane == 0) scratch[wave] = mine;
+  __syncthreads();
+  Best total = scratch[0];
+  for (int i = 1; i < (int)(blockDim.x / Q3_WAVE); ++i) total = better(total, scratch[i]);
+  return total;
+}
+
+__global__ __launch_bounds__(1024) void sample_kernel(const float* __restrict__ logits,
+                                                      const float* __restrict__ temperature,
+                                                      const int* __restrict__ top_k,
+                                                      const long long* __restrict__ seed,
+                                                      const int* __restrict__ counter,
+                                                      int* __restrict__ out, int V) {
+  __shared__ Best best_scratch[16];
+  __shared__ unsigned int hist[256];
+  __shared__ uint32_t sh_prefix, sh_remaining;
+  const int r = blockIdx.x;
+  const float* row = logits + (size_t)r * V;
+  const float temp = temperature[r];
+  Best mine;
+  mine.value = -INFINITY;
+  mine.index = 0x7fffffff;
+
+  if (!(temp > 0.f)) {
+    for (int j = threadIdx.x; j < V; j += blockDim.x) {
+      Best c;
+      c.value = row[j];
+      c.index = j;
+      mine = better(mine, c);
+    }
+    const Best total = block_best(mine, best_scratch);
+    if (threadIdx.x == 0) out[r] = total.index < V ? total.index : 0;
+    return;
+  }
+
+  // the key of the k-th largest logit, by a radix select over the four bytes
+  uint32_t threshold = 0;  // every key passes
+  const int k = top_k[r];
+  if (k > 0 && k < V) {
+    uint32_t prefix = 0, mask = 0;
+    uint32_t remaining = (uint32_t)k;
+    for (int shift = 24; shift >= 0; shift -= 8) {
+      for (int i = threadIdx.x; i < 256; i += blockDim.x) hist[i] = 0;
+      __syncthreads();
+      for (int j = threadIdx.x; j < V; j += blockDim.x) {
+        const uint32_t key = order_key(row[j]);
+        if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
+      }
+      __syncthreads();
+      if (threadIdx.x == 0) {
+        uint32_t left = remaining;
+        int bin = 255;
+        for (; bin > 0; --bin) {
+          if (hist[bin] >= left) break;
+          left -= hist[bin];
+        }
+        sh_prefix = prefix | ((uint32_t)bin << shift);
+        sh_remaining = left;
+      }
+      __syncthreads();
+      prefix = sh_prefix;
+      remaining = sh_remaining;
+      mask |= 255u << shift;
+      __syncthreads();
+    }
+    threshold = prefix;
+  }
+
+  const unsigned long long sd = (unsigned long long)seed[r];
+  const uint32_t k0 = (uint32_t)sd, k1 = (uint32_t)(sd >> 32);
+  const uint32_t step = (uint32_t)counter[r];
+  const float inv_t = 1.f / temp;
+  for (int j4 = threadIdx.x * 4; j4 < V; j4 += blockDim.x * 4) {
+    uint32_t c[4] = {(uint32_t)(j4 >> 2), step, 0u, 0u};
+    philox4x32_10(c, k0, k1);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int j = j4 + i;
+      if (j >= V) break;
+      const float x = row[j];
+      if (order_key(x) < threshold) continue;
+      const float u = ((float)(c[i] >> 9) + 0.5f) * (1.f / 8388608.f);  // in (0, 1), exact
+      Best cand;
+      cand.value = x * inv_t - logf(-logf(u));
+      cand.index = j;
+      mine = better(mine, cand);
+    }
+  }
+  const Best total = block_best(mine, best_scratch);
+  if (threadIdx.x == 0) out[r] = total.index < V ? total.index : 0;
+}
+
+extern "C" int q3_sample(const float* logits, const float* temperature, const int* top_k,
+                         const long long* seed, const int* counter, int* out, int R, int V,
+                         hipStream_t stream) {
+  if (R <= 0 || V <= 0) return Q3_ERR_BAD_ARGUMENT;
+  int threads = 64;
+  while (threads < 1024 && threads * 4 < V) threads *= 2;
+  hipLaunchKernelGGL(sample_kernel, dim3(R), dim3(threads), 0, stream, logits, temperature, top_k, seed,
+                     counter, out, V);
+  return q3_launch_status();
+}

@@ -22,6 +22,7 @@ class ModelRunner:
         self.manager = CacheManager(model.plane_needs, page_size, num_pages, max_requests)
         self.storage = CacheStorage(self.manager, model.precision.act, self.device)
         self.vocab_size = model.spec.vocab_size
+        self.max_positions = getattr(model.position, "max_positions", None)
 
     def step(self, entries):
         """entries: list of StepEntry. Returns logits (R, V) float32 on the
@@ -38,6 +39,11 @@ class ModelRunner:
             if min(e.tokens) < 0 or max(e.tokens) >= self.vocab_size:
                 raise ValueError("request %r has a token outside 0..%d" % (e.request_id, self.vocab_size - 1))
         m = self.manager
+        if self.max_positions is not None:
+            for e in entries:
+                if self.length(e.request_id) + len(e.tokens) > self.max_positions:
+                    raise ValueError("request %r would pass position %d, the model's last"
+                                     % (e.request_id, self.max_positions - 1))
         admitted, reserved = [], []
         try:
             for e in entries:

@@ -244,7 +244,14 @@ def linear(x, weight, out_dtype=None, out=None):
     if out is None:
         out = torch.empty((M, N), dtype=out_dtype, device=x.device)
     _need(out.shape == (M, N) and out.dtype == out_dtype, "out must be (M, N) of out_dtype")
-    if M:
+    if M and x.dtype == torch.bfloat16:
+        # bfloat16 products go to the vendor library (hipBLASLt through torch), as the
+        # reference's engine uses its vendor library for them; accumulation is float32
+        if out_dtype == torch.bfloat16:
+            torch.mm(x, weight.t(), out=out)
+        else:
+            torch.mm(x, weight.t(), out_dtype=torch.float32, out=out)
+    elif M:
         _check(library("gemm").q3_linear(
             _ptr(x), _ptr(weight), _ptr(out), M, N, K, _DT[x.dtype], _DT[out_dtype], _stream()), "linear")
     return out

@@ -1,0 +1,97 @@
+"""The engine on the GPU against the plain implementation, in float32 and in
+bfloat16: every request alone and whole; most of it in one step and the last 32
+tokens one by one; portions of changing size; mixed batches with so few pages
+that they are used again; long decoding; the first tokens of a sequence."""
+
+import pytest
+import torch
+
+import plain_qwen3
+from helpers import (TINY, max_live_tokens, random_tokens, run_trace, trace_mixed, trace_portions,
+                     trace_tail_decoded, trace_whole)
+from qwen3_from_scratch_amd.engine import load_runner
+
+pytestmark = pytest.mark.gpu
+
+# float32: the engine and the plain implementation differ by rounding order only.
+# bfloat16: activations are rounded to 8 bits of mantissa between kernels; the
+# bound is a fraction of the logits' spread, which the weights' scale sets.
+TOL = {"float32": 2e-4, "bfloat16": 6e-2}
+
+_plain_cache = {}
+
+
+def _requests(name, lengths, seed=5):
+    vocab = TINY[name]["config"]["vocab_size"]
+    return {"r%d" % i: random_tokens(n, vocab, seed + i) for i, n in enumerate(lengths)}
+
+
+def _plain(folder, name, requests):
+    out = {}
+    cfg, w = None, None
+    for rid, toks in requests.items():
+        key = (name, tuple(toks))
+        if key not in _plain_cache:
+            if cfg is None:
+                cfg, w = plain_qwen3.read_model_folder(folder)
+            _plain_cache[key] = plain_qwen3.logits_of_sequence(cfg, w, toks)
+        out[rid] = _plain_cache[key]
+    return out
+
+
+def _compare(got, want, dtype):
+    worst, scale = 0.0, 0.0
+    for rid, logits in want.items():
+        scale = max(scale, float(logits.abs().max()))
+        for p in range(logits.shape[0]):
+            assert (rid, p) in got, "no logits for %s at %d" % (rid, p)
+            diff = float((got[(rid, p)] - logits[p]).abs().max())
+            if diff > worst:
+                worst, where = diff, (rid, p)
+    bound = TOL[dtype] * max(1.0, scale)
+    assert worst <= bound, "largest difference %g at %s (bound %g)" % (worst, where, bound)
+
+
+CASES = [("A", [5, 17, 33, 80]), ("B", [1, 9, 64, 130]), ("C", [40, 70, 3, 201])]
+FAMILIES = {"whole": trace_whole, "tail": trace_tail_decoded, "portions": trace_portions, "mixed": trace_mixed}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,lengths", CASES)
+@pytest.mark.parametrize("family", list(FAMILIES))
+def test_every_cutting_matches_plain(model_folders, dtype, name, lengths, family):
+    requests = _requests(name, lengths)
+    want = _plain(model_folders[name], name, requests)
+    steps = FAMILIES[family](requests)
+    page = TINY[name]["page_size"]
+    runner = load_runner(model_folders[name], dtype=dtype, device="cuda", page_size=page,
+                         max_tokens=max_live_tokens(steps, page=page), max_requests=4)
+    got = run_trace(runner, steps)
+    _compare(got, want, dtype)
+    assert runner.manager.num_free() == runner.manager.num_pages()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(model_folders, dtype):
+    """A short prompt and then hundreds of tokens one by one, across many pages."""
+    name = "B"
+    toks = random_tokens(400, TINY[name]["config"]["vocab_size"], 77)
+    requests = {"long": toks}
+    want = _plain(model_folders[name], name, requests)
+    steps = trace_tail_decoded(requests, tail=390)
+    runner = load_runner(model_folders[name], dtype=dtype, device="cuda", page_size=8, max_tokens=448,
+                         max_requests=2)
+    _compare(run_trace(runner, steps), want, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_first_tokens(model_folders, dtype):
+    """Positions 0, 1, 2 of a sequence, each fed alone: one key, two keys, three."""
+    for name in ("A", "B"):
+        toks = random_tokens(3, TINY[name]["config"]["vocab_size"], 3)
+        requests = {"f": toks}
+        want = _plain(model_folders[name], name, requests)
+        steps = [([("f", [t], [0])], ["f"] if i == 2 else []) for i, t in enumerate(toks)]
+        runner = load_runner(model_folders[name], dtype=dtype, device="cuda",
+                             page_size=TINY[name]["page_size"], max_tokens=64, max_requests=2)
+        _compare(run_trace(runner, steps), want, dtype)

@@ -1,0 +1,308 @@
+"""Each HIP kernel alone against its plain PyTorch twin, at sizes other than the
+tiny models', in float32 (tight) and bfloat16 (against the float32 twin fed the
+same bfloat16-representable inputs)."""
+
+import math
+
+import pytest
+import torch
+
+import torch_ops
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def _ops():
+    from qwen3_from_scratch_amd import ops
+    return ops
+
+
+def _rand(shape, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype).cuda()
+
+
+def _tol(dtype):
+    return dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=1.6e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,H,V", [(1, 40, 7), (37, 1000, 331), (5, 4096, 100)])
+def test_embed_rows(dtype, T, H, V):
+    table = _rand((V, H), dtype, 1)
+    ids = torch.randint(0, V, (T,), dtype=torch.int32).cuda()
+    got = _ops().embed_rows(ids, table)
+    assert got.dtype == torch.float32
+    assert torch.equal(got, torch_ops.embed_rows(ids, table))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,I", [(1, 24), (9, 1000), (130, 333)])
+def test_swiglu(dtype, T, I):
+    x = _rand((T, 2 * I), dtype, 2, scale=3.0)
+    got = _ops().swiglu(x)
+    want = torch_ops.swiglu(x.float())
+    torch.testing.assert_close(got.float(), want, **_tol(dtype))
+    zero = torch.zeros((3, 2 * I), dtype=dtype, device="cuda")
+    assert torch.count_nonzero(_ops().swiglu(zero)) == 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("wdtype", DTYPES)
+@pytest.mark.parametrize("T,H", [(1, 16), (7, 1000), (33, 5120), (2, 13000)])
+def test_rmsnorm_plain_add_and_rows(dtype, wdtype, T, H):
+    ops = _ops()
+    x = _rand((T, H), torch.float32, 3, scale=2.0)
+    w = (1 + 0.3 * _rand((H,), torch.float32, 4)).to(wdtype)
+    d = _rand((T, H), dtype, 5)
+    eps = 1e-3
+    tol = _tol(dtype)
+    torch.testing.assert_close(ops.rmsnorm(x.clone(), w, eps, dtype).float(),
+                               torch_ops.rmsnorm(x.clone(), w, eps, torch.float32), **tol)
+    x1, x2 = x.clone(), x.clone()
+    got = ops.rmsnorm(x1, w, eps, dtype, delta=d)
+    want = torch_ops.rmsnorm(x2, w, eps, torch.float32, delta=d)
+    torch.testing.assert_close(got.float(), want, **tol)
+    torch.testing.assert_close(x1, x2, rtol=0, atol=0)          # the stream was updated in place
+    rows = torch.tensor([T - 1, 0, T // 2], dtype=torch.int32).cuda()
+    x3 = x.clone()
+    got = ops.rmsnorm(x3, w, eps, dtype, delta=d, rows=rows, write_back=False)
+    want = torch_ops.rmsnorm(x.clone(), w, eps, torch.float32, delta=d, rows=rows, write_back=False)
+    torch.testing.assert_close(got.float(), want, **tol)
+    assert torch.equal(x3, x)                                    # and left alone here
+
+
+def test_rope_table_matches_closed_form():
+    # src/qwen3_from_scratch: test/models/test_rotary.py:19-54 (head 128, base 1e5, 1024 positions)
+    D, base, P = 128, 100000.0, 1024
+    inv = 1.0 / (base ** (torch.arange(0, D, 2, dtype=torch.float) / D))
+    table = _ops().rope_table(inv.cuda(), P).cpu()
+    freqs = torch.outer(torch.arange(P, dtype=torch.float), inv)
+    assert table.shape == (P, D)
+    torch.testing.assert_close(table[:, :D // 2], freqs.cos(), rtol=0, atol=1e-5)
+    torch.testing.assert_close(table[:, D // 2:], freqs.sin(), rtol=0, atol=1e-5)
+    # far positions: angles of tens of thousands of radians need full range reduction
+    P = 40960
+    table = _ops().rope_table(inv.cuda(), P).cpu()
+    freqs = torch.outer(torch.arange(P, dtype=torch.float), inv)
+    torch.testing.assert_close(table[-64:, :D // 2], freqs[-64:].cos(), rtol=0, atol=2e-6)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("Hq,Hkv,D,R,page", [(4, 2, 16, 16, 16), (6, 3, 48, 48, 8), (5, 1, 80, 32, 4),
+                                             (32, 8, 128, 128, 16), (2, 2, 256, 256, 16)])
+def test_qk_norm_rope_store(dtype, Hq, Hkv, D, R, page):
+    ops = _ops()
+    T, B, P = 23, 3, 300
+    inv = 1.0 / (10000.0 ** (torch.arange(0, R, 2, dtype=torch.float) / R))
+    table = torch_ops.rope_table(inv, P).cuda()
+    qkv = _rand((T, (Hq + 2 * Hkv) * D), dtype, 6)
+    qw = (1 + 0.2 * _rand((D,), torch.float32, 7)).to(dtype)
+    kw = (1 + 0.2 * _rand((D,), torch.float32, 8)).to(dtype)
+    seq = torch.tensor([0] * 9 + [1] * 1 + [2] * 13, dtype=torch.int32).cuda()
+    pos = torch.tensor(list(range(40, 49)) + [77] + list(range(0, 13)), dtype=torch.int32).cuda()
+    W = 100 // page + 1
+    pages = torch.randperm(3 * W)[: 3 * W].view(3, W).to(torch.int32)
+    pages[2, 1] = -1                                   # a page given back: nothing is stored there
+    bt = pages.cuda()
+    npages = 3 * W
+    kc = torch.full((npages, Hkv, page, D), -7.0, dtype=dtype, device="cuda")
+    vc = torch.full((npages, Hkv, page, D), -7.0, dtype=dtype, device="cuda")
+    kc2, vc2 = kc.float(), vc.float()
+    got = qkv.clone()
+    ops.qk_norm_rope_store(got, Hq, Hkv, D, pos, seq, q_weight=qw, k_weight=kw, eps=1e-5, table=table,
+                           block_table=bt, k_cache=kc, v_cache=vc)
+    want = qkv.float()
+    torch_ops.qk_norm_rope_store(want, Hq, Hkv, D, pos, seq, q_weight=qw, k_weight=kw, eps=1e-5,
+                                 table=table, block_table=bt, k_cache=kc2, v_cache=vc2)
+    tol = _tol(dtype)
+    torch.testing.assert_close(got.float()[:, :Hq * D], want[:, :Hq * D], **tol)
+    assert torch.equal(got[:, Hq * D:], qkv[:, Hq * D:])            # k and v columns of qkv untouched
+    torch.testing.assert_close(kc.float(), kc2, **tol)
+    assert torch.equal(vc.float(), vc2)                             # values are copied bit for bit
+    assert (kc2 == -7.0).any()                                      # untouched slots keep the sentinel
+    # without norm, without rotation, without cache: q comes back as it went in
+    same = qkv.clone()
+    ops.qk_norm_rope_store(same, Hq, Hkv, D, pos, seq)
+    assert torch.equal(same, qkv)
+
+
+def _paged_case(dtype, B, Hq, Hkv, D, page, q_lens, kv_lens, seed, spread=True):
+    g = torch.Generator().manual_seed(seed)
+    T = sum(q_lens)
+    W = max(-(-L // page) for L in kv_lens) + 1
+    npages = B * W + 3
+    perm = torch.randperm(npages, generator=g)[: B * W].view(B, W).to(torch.int32)
+    for b in range(B):                                    # -1 padding beyond the last page is never read
+        perm[b, -(-kv_lens[b] // page):] = -1
+    kc = (torch.randn((npages, Hkv, page, D), generator=g)).to(dtype).cuda()
+    vc = (torch.randn((npages, Hkv, page, D), generator=g)).to(dtype).cuda()
+    q = (torch.randn((T, Hq, D), generator=g) * (2.0 if spread else 1.0)).to(dtype).cuda()
+    cu = torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32).cuda()
+    kvl = torch.tensor(kv_lens, dtype=torch.int32).cuda()
+    return q, kc, vc, perm.cuda(), cu, kvl
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("Hq,Hkv,D,page", [(4, 2, 16, 16), (8, 2, 32, 8), (6, 3, 48, 16), (5, 5, 80, 4),
+                                           (32, 8, 128, 16), (3, 1, 256, 32), (16, 2, 64, 16)])
+@pytest.mark.parametrize("window", [0, 19])
+def test_paged_attention_mixed_batch(dtype, Hq, Hkv, D, page, window):
+    ops = _ops()
+    q_lens = [1, 37, 4, 1, 70]
+    kv_lens = [16, 37, 20, 131, 200]
+    q, kc, vc, bt, cu, kvl = _paged_case(dtype, 5, Hq, Hkv, D, page, q_lens, kv_lens, 9)
+    scale = D ** -0.5
+    got = ops.paged_attention(q, Hq, kc, vc, bt, cu, kvl, max(q_lens), max(kv_lens), scale, window=window)
+    want = torch_ops.paged_attention(q.float(), Hq, kc.float(), vc.float(), bt, cu, kvl, max(q_lens),
+                                     max(kv_lens), scale, window=window)
+    tol = dict(rtol=1e-4, atol=2e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(got.float(), want, **tol)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_paged_attention_far_key_stands_out(dtype):
+    """One key far back is made to dominate: a kernel that drops, repeats or
+    misplaces a page shows at once."""
+    ops = _ops()
+    Hq, Hkv, D, page = 8, 2, 128, 16
+    for L, far in [(1000, 3), (777, 400), (2049, 2048 - 17)]:
+        q, kc, vc, bt, cu, kvl = _paged_case(dtype, 1, Hq, Hkv, D, page, [1], [L], 10 + L, spread=False)
+        pg = int(bt[0, far // page])
+        kc[pg, :, far % page] = (q[0].view(Hkv, Hq // Hkv, D)[:, 0] * 4).to(dtype)
+        scale = D ** -0.5
+        got = ops.paged_attention(q, Hq, kc, vc, bt, cu, kvl, 1, L, scale)
+        want = torch_ops.paged_attention(q.float(), Hq, kc.float(), vc.float(), bt, cu, kvl, 1, L, scale)
+        tol = dict(rtol=1e-4, atol=2e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+        torch.testing.assert_close(got.float(), want, **tol)
+        # the dominating key's value is (nearly) the answer for the first head of each group
+        v_far = vc[pg, :, far % page].float()
+        first = got.float().view(Hq, D)[:: Hq // Hkv]
+        assert (first - v_far).abs().max() < 0.2
+
+
+def test_paged_attention_first_token_returns_first_value():
+    ops = _ops()
+    q, kc, vc, bt, cu, kvl = _paged_case(torch.float32, 2, 4, 2, 32, 8, [1, 1], [1, 1], 11)
+    got = ops.paged_attention(q, 4, kc, vc, bt, cu, kvl, 1, 1, 32 ** -0.5).view(2, 4, 32)
+    for b in range(2):
+        v0 = vc[int(bt[b, 0]), :, 0]
+        torch.testing.assert_close(got[b], v0.repeat_interleave(2, dim=0), rtol=1e-6, atol=1e-6)
+
+
+def test_paged_attention_ignores_garbage_beyond_the_sequence():
+    ops = _ops()
+    q, kc, vc, bt, cu, kvl = _paged_case(torch.float32, 2, 4, 2, 32, 8, [3, 1], [11, 21], 12)
+    a = ops.paged_attention(q, 4, kc, vc, bt, cu, kvl, 3, 21, 0.2)
+    # poison every slot past each sequence's end, and every page it does not own
+    owned = set()
+    for b, L in enumerate([11, 21]):
+        for j in range(L):
+            owned.add((int(bt[b, j // 8]), j % 8))
+    for pg in range(kc.shape[0]):
+        for s in range(8):
+            if (pg, s) not in owned:
+                kc[pg, :, s] = float("nan")
+                vc[pg, :, s] = float("nan")
+    b_ = ops.paged_attention(q, 4, kc, vc, bt, cu, kvl, 3, 21, 0.2)
+    assert torch.equal(a, b_)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,N,K", [(1, 64, 64), (2, 100, 72), (8, 331, 200), (33, 1000, 96), (64, 257, 1030),
+                                   (130, 384, 224), (300, 129, 515)])
+def test_linear(dtype, M, N, K):
+    ops = _ops()
+    x = _rand((M, K), dtype, 13)
+    w = _rand((N, K), dtype, 14, scale=0.1)
+    want = x.double() @ w.double().T
+    got = ops.linear(x, w)
+    assert got.dtype == dtype
+    tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=1.6e-2, atol=1e-2)
+    torch.testing.assert_close(got.double(), want, **tol)
+    got32 = ops.linear(x, w, out_dtype=torch.float32)
+    assert got32.dtype == torch.float32
+    torch.testing.assert_close(got32.double(), want, rtol=1e-4, atol=1e-4)
+
+
+def test_linear_float32_is_true_float32():
+    """Inputs whose products need all 24 bits: a matrix mode of reduced precision
+    (bf16 or tf32-like splitting) would be off by far more than float32 rounding."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(15)
+    x = (1.0 + torch.rand((16, 512), generator=g) * 2 ** -10).cuda()
+    w = (1.0 + torch.rand((24, 512), generator=g) * 2 ** -10).cuda()
+    want = (x.double() @ w.double().T)
+    got = ops.linear(x, w).double()
+    assert ((got - want).abs() / want).max() < 2e-6
+
+
+def test_sample_greedy_and_ties():
+    ops = _ops()
+    R, V = 5, 1000
+    logits = _rand((R, V), torch.float32, 16)
+    logits[2, 17] = logits[2, 900] = 50.0               # equal maxima: the lowest index wins
+    z = torch.zeros(R, device="cuda")
+    got = ops.sample(logits, z, torch.zeros(R, dtype=torch.int32, device="cuda"),
+                     torch.zeros(R, dtype=torch.int64, device="cuda"),
+                     torch.zeros(R, dtype=torch.int32, device="cuda"))
+    assert got.tolist() == torch.argmax(logits, dim=-1).tolist()
+    assert got[2] == 17
+
+
+def test_sample_temperature_follows_softmax_and_seed():
+    ops = _ops()
+    V, R = 11, 40000
+    base = torch.tensor([0.5, -1.0, 2.0, 0.0, 1.0, -3.0, 0.3, 1.7, -0.4, 0.9, 0.1])
+    logits = base.repeat(R, 1).cuda().contiguous()
+    T = 0.8
+    temp = torch.full((R,), T, device="cuda")
+    k0 = torch.zeros(R, dtype=torch.int32, device="cuda")
+    seed = torch.full((R,), 1234, dtype=torch.int64, device="cuda")
+    counter = torch.arange(R, dtype=torch.int32, device="cuda")
+    got = ops.sample(logits, temp, k0, seed, counter)
+    freq = torch.bincount(got.cpu().long(), minlength=V).double() / R
+    p = torch.softmax(base.double() / T, dim=-1)
+    chi2 = float((R * (freq - p) ** 2 / p).sum())
+    assert chi2 < 40.0, chi2                              # 10 degrees of freedom; 40 is far in the tail
+    # the same (seed, counter) gives the same token whatever else is in the batch
+    again = ops.sample(logits[:100].contiguous(), temp[:100], k0[:100], seed[:100], counter[:100])
+    assert torch.equal(again, got[:100])
+    other = ops.sample(logits, temp, k0, seed + 1, counter)
+    assert not torch.equal(other, got)
+    # top-k: only the k best are ever drawn, with their renormalised frequencies
+    k = 3
+    got = ops.sample(logits, temp, torch.full((R,), k, dtype=torch.int32, device="cuda"), seed, counter)
+    top = torch.topk(base, k).indices
+    freq = torch.bincount(got.cpu().long(), minlength=V).double() / R
+    assert set(torch.nonzero(freq).flatten().tolist()) == set(top.tolist())
+    pk = torch.zeros(V, dtype=torch.double)
+    pk[top] = torch.softmax(base[top].double() / T, dim=-1)
+    chi2 = float((R * (freq[top] - pk[top]) ** 2 / pk[top]).sum())
+    assert chi2 < 30.0, chi2
+    # as the temperature goes to zero the draw becomes the arg-max
+    cold = ops.sample(logits[:50].contiguous(), torch.full((50,), 1e-3, device="cuda"), k0[:50], seed[:50],
+                      counter[:50])
+    assert (cold == 2).all()
+
+
+def test_sample_large_vocabulary_top_k():
+    ops = _ops()
+    R, V, k = 3, 151936, 40
+    logits = _rand((R, V), torch.float32, 17, scale=3.0)
+    temp = torch.ones(R, device="cuda")
+    seed = torch.arange(R, dtype=torch.int64, device="cuda")
+    allowed = [set(torch.topk(logits[r], k).indices.tolist()) for r in range(R)]
+    for c in range(20):
+        got = ops.sample(logits, temp, torch.full((R,), k, dtype=torch.int32, device="cuda"), seed,
+                         torch.full((R,), c, dtype=torch.int32, device="cuda"))
+        for r in range(R):
+            assert int(got[r]) in allowed[r]
+
+
+def test_operands_on_the_host_are_refused():
+    ops = _ops()
+    with pytest.raises(ValueError):
+        ops.swiglu(torch.zeros(2, 8))

@@ -1,0 +1,257 @@
+"""The in-process engine: continuous batching over the step function.
+
+Interface and metric fields are those of the reference's SyncEngine
+(src/qwen3_from_scratch/inference/sync_engine.py:28-182): `warmup`,
+`generate_stream`, `generate`, `batch_generate`; `StreamChunk` and `PerfMetrics`
+(inference/llm_engine.py:48-68), `BatchPerfMetrics` (sync_engine.py:17-25).
+Besides the YAML file of the reference, an `EngineConfig` can be passed, and
+prompts may be lists of token ids, which is all a model of random weights
+understands.
+"""
+
+import itertools
+import json
+import os
+import time
+from dataclasses import dataclass
+
+import torch
+
+from ..config.engine_config import EngineConfig
+from ..sampling import Sampler, SamplingParams
+from .batch import StepEntry
+from .loading import load_model
+from .runner import ModelRunner
+from .scheduler import Request, RequestStatus, Scheduler
+
+
+@dataclass
+class PerfMetrics:
+    ttft: float
+    token_count: int
+    tps: float
+    total_elapsed: float
+
+
+@dataclass
+class StreamChunk:
+    delta: str
+    metrics: PerfMetrics
+    req_id: str = ""
+    prompt_tokens: int = 0
+    token_id: int = -1
+
+
+@dataclass
+class BatchPerfMetrics:
+    per_request: list
+    num_requests: int
+    total_tokens: int
+    total_elapsed: float
+    aggregate_tps: float
+
+
+def _load_tokenizer(path):
+    if not any(os.path.isfile(os.path.join(path, f)) for f in ("tokenizer.json", "tokenizer_config.json")):
+        return None
+    from transformers import AutoTokenizer
+
+    return AutoTokenizer.from_pretrained(path)
+
+
+class SyncEngine:
+    def __init__(self, config_path=None, model_name=None, log_interval=0, *, config=None, model=None,
+                 **overrides):
+        """`SyncEngine(config_path, model_name)` reads the reference's YAML;
+        `SyncEngine(config=EngineConfig(path=...))` or keyword options
+        (`path=..., dtype=..., max_num_seqs=...`) do without a file. `model`
+        hands in an already loaded model."""
+        if config is None:
+            if config_path is not None:
+                config = EngineConfig.from_yaml(str(config_path), model_name, **overrides)
+            else:
+                config = EngineConfig(**overrides)
+        self.config = config
+        self.model_name = model_name or config.name
+        self.log_interval = log_interval
+        self.model = model if model is not None else load_model(config.path, config.dtype, config.device)
+        self.tokenizer = _load_tokenizer(config.path) if config.path else None
+        mc = self.model.config
+        self.max_len = min(config.max_len, mc.max_position_embeddings)
+        num_blocks = config.num_blocks or self._blocks_from_memory()
+        self.runner = ModelRunner(self.model, config.block_size, num_blocks, max_requests=config.max_num_seqs)
+        self.sampler = Sampler(self.model.device)
+        self.scheduler = Scheduler(
+            self.runner.manager, config.max_num_seqs, config.max_num_tokens, config.chunked_prefill_size,
+            max_len=self.max_len, release=self.runner.finish)
+        self.eos_ids = self._eos_ids()
+        self._ids = itertools.count()
+        self.steps = 0
+
+    # ---- set-up ----
+    def _blocks_from_memory(self):
+        """Pages that fit in `gpu_utilization` of the free memory, halved for
+        keys and values, as the reference sizes its cache
+        (src/qwen3_from_scratch/inference/kv_cache/paged_cache.py:36-49)."""
+        per_token = 0
+        itemsize = 2 if self.model.precision.act == torch.bfloat16 else 4
+        for need in self.model.plane_needs:
+            if need is not None and need.paged:
+                per_token += 2 * need.kv_heads * need.head_dim * itemsize
+        per_page = max(1, per_token * self.config.block_size)
+        if self.model.device.type == "cuda":
+            free = torch.cuda.mem_get_info(self.model.device)[0]
+        else:
+            free = 1 << 30
+        wanted = int(free * self.config.gpu_utilization) // per_page
+        enough = self.config.max_num_seqs * (-(-self.max_len // self.config.block_size))
+        return max(1, min(wanted, enough))
+
+    def _eos_ids(self):
+        ids = set(self.model.config.eos_token_ids)
+        gen = os.path.join(self.config.path, "generation_config.json") if self.config.path else ""
+        if gen and os.path.isfile(gen):
+            with open(gen) as fh:
+                eos = json.load(fh).get("eos_token_id")
+            if isinstance(eos, int):
+                ids.add(eos)
+            elif isinstance(eos, list):
+                ids.update(eos)
+        if self.tokenizer is not None and self.tokenizer.eos_token_id is not None:
+            ids.add(int(self.tokenizer.eos_token_id))
+        return tuple(sorted(ids))
+
+    # ---- requests ----
+    def _encode(self, prompt):
+        if isinstance(prompt, (list, tuple)) and (not prompt or isinstance(prompt[0], int)):
+            return list(prompt)
+        if self.tokenizer is None:
+            raise ValueError("the model folder has no tokenizer: pass prompts as lists of token ids")
+        if not isinstance(prompt, str):
+            prompt = self.tokenizer.apply_chat_template(prompt, tokenize=False, add_generation_prompt=True)
+        return list(self.tokenizer(prompt).input_ids)
+
+    def _decode(self, ids):
+        if self.tokenizer is None:
+            return ""
+        return self.tokenizer.decode(ids, skip_special_tokens=True)
+
+    def default_params(self, max_new_tokens=None, **kw):
+        gen = self.config.generation
+        return SamplingParams(
+            temperature=kw.get("temperature", gen.temperature),
+            top_k=kw.get("top_k", gen.top_k),
+            seed=kw.get("seed", self.config.seed),
+            max_new_tokens=max_new_tokens if max_new_tokens else gen.max_new_tokens,
+            ignore_eos=kw.get("ignore_eos", False),
+        )
+
+    def add_request(self, prompt, params=None, request_id=None):
+        """Queue a prompt (text, chat messages or token ids); returns the Request."""
+        request = Request(
+            request_id=request_id if request_id is not None else "req-%d" % next(self._ids),
+            prompt=self._encode(prompt), params=params or self.default_params(), eos_ids=self.eos_ids)
+        self.scheduler.add(request)
+        return request
+
+    # ---- the loop body ----
+    def step(self):
+        """Schedule, run the step function, sample, book-keep. Returns the plan
+        (a list of Scheduled); requests that got a token have it in
+        `last_token_id`, finished ones have status FINISHED."""
+        plan = self.scheduler.schedule()
+        if not plan:
+            return plan
+        entries = []
+        for s in plan:
+            req = s.request
+            tokens = req.tokens[req.computed: req.computed + s.num_tokens]
+            entries.append(StepEntry(req.request_id, tokens, [s.num_tokens - 1] if s.samples else []))
+        logits = self.runner.step(entries)
+        sampling = [s.request for s in plan if s.samples]
+        sampled = self.sampler.sample(logits, [r.params for r in sampling],
+                                      [len(r.generated) for r in sampling])
+        self.scheduler.after_step(plan, sampled)
+        self.steps += 1
+        return plan
+
+    # ---- the reference's interface ----
+    def warmup(self, prompt=None, num_tokens=3):
+        """A short request, so that what is built or tuned at first use does
+        not count against the first real request."""
+        if prompt is None:
+            prompt = [1, 2, 3] if self.tokenizer is None else "你好"
+        for _ in self.generate_stream(prompt, num_tokens):
+            pass
+
+    def generate_stream(self, prompt, max_new_tokens=None, **sampling):
+        request = self.add_request(prompt, self.default_params(max_new_tokens, **sampling))
+        start = time.perf_counter()
+        first = None
+        count = 0
+        while True:
+            plan = self.step()
+            now = time.perf_counter()
+            for s in plan:
+                if s.request is not request or not s.samples:
+                    continue
+                count += 1
+                if first is None:
+                    first = now
+                    metrics = PerfMetrics(now - start, 1, 0.0, now - start)
+                else:
+                    span = now - first
+                    metrics = PerfMetrics(first - start, count, (count - 1) / span if span > 0 else 0.0,
+                                          now - start)
+                yield StreamChunk(self._decode([request.last_token_id]), metrics, str(request.request_id),
+                                  len(request.prompt), request.last_token_id)
+                if request.status == RequestStatus.FINISHED:
+                    return
+
+    def generate(self, prompt, max_new_tokens=None, **sampling):
+        """The whole answer as text (token ids joined by spaces without a tokenizer)."""
+        chunks = list(self.generate_stream(prompt, max_new_tokens, **sampling))
+        if self.tokenizer is None:
+            return " ".join(str(c.token_id) for c in chunks)
+        return "".join(c.delta for c in chunks)
+
+    def generate_ids(self, prompts, max_new_tokens=None, **sampling):
+        """Token-level batch generation: list of generated id lists, in order."""
+        requests = [self.add_request(p, self.default_params(max_new_tokens, **sampling)) for p in prompts]
+        while any(r.status != RequestStatus.FINISHED for r in requests):
+            self.step()
+        return [list(r.generated) for r in requests]
+
+    def batch_generate(self, prompts, max_new_tokens=None, **sampling):
+        """All prompts queued at once and batched continuously until all have
+        ended; returns (texts in order, BatchPerfMetrics)."""
+        start = time.perf_counter()
+        requests = [self.add_request(p, self.default_params(max_new_tokens, **sampling)) for p in prompts]
+        first, last, counts = {}, {}, {}
+        while any(r.status != RequestStatus.FINISHED for r in requests):
+            plan = self.step()
+            now = time.perf_counter()
+            for s in plan:
+                if s.samples:
+                    rid = s.request.request_id
+                    first.setdefault(rid, now)
+                    last[rid] = now
+                    counts[rid] = counts.get(rid, 0) + 1
+            if self.log_interval > 0 and self.steps % self.log_interval == 0:
+                done = sum(r.status == RequestStatus.FINISHED for r in requests)
+                total = sum(len(r.generated) for r in requests)
+                print("[batch] step=%d pending=%d completed=%d total_tokens=%d aggregate_tps=%.2f"
+                      % (self.steps, len(requests) - done, done, total, total / max(now - start, 1e-9)))
+        elapsed = time.perf_counter() - start
+        per_request = []
+        for r in requests:
+            rid = r.request_id
+            n = counts.get(rid, 0)
+            span = last.get(rid, start) - first.get(rid, start)
+            per_request.append(PerfMetrics(first.get(rid, start) - start, n,
+                                           (n - 1) / span if span > 0 else 0.0, last.get(rid, start) - start))
+        total = sum(len(r.generated) for r in requests)
+        texts = [self._decode(r.generated) if self.tokenizer is not None
+                 else " ".join(map(str, r.generated)) for r in requests]
+        return texts, BatchPerfMetrics(per_request, len(requests), total, elapsed,
+                                       total / elapsed if elapsed > 0 else 0.0)

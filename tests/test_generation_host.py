@@ -1,0 +1,82 @@
+"""Generation through the entry point on the CPU (plain twins in place of the
+kernels): greedy tokens equal the plain implementation's, whatever the batching,
+the portions, and the preemptions."""
+
+import pytest
+import torch
+
+import plain_qwen3
+from helpers import TINY, random_tokens
+from qwen3_from_scratch_amd.engine import SyncEngine
+
+
+def _plain_greedy(folder, prompts, n):
+    cfg, w = plain_qwen3.read_model_folder(folder)
+    return [plain_qwen3.greedy_generate(cfg, w, p, n) for p in prompts]
+
+
+def test_greedy_generation_matches_plain_a(cpu_ops, model_folders):
+    # the workload of the first tiny configuration: prompts of 5, 17 and 33 tokens, 16 greedy tokens each
+    vocab = TINY["A"]["config"]["vocab_size"]
+    prompts = [random_tokens(n, vocab, 40 + n) for n in (5, 17, 33)]
+    want = _plain_greedy(model_folders["A"], prompts, 16)
+    engine = SyncEngine(path=model_folders["A"], dtype="float32", device="cpu", block_size=16, num_blocks=12,
+                        max_num_seqs=4)
+    got = engine.generate_ids(prompts, max_new_tokens=16, temperature=0.0, ignore_eos=True)
+    assert got == want
+    assert engine.runner.manager.num_free() == 12
+
+
+def test_chunked_mixed_generation_matches_plain_b(cpu_ops, model_folders):
+    # the second: prompts of 1, 9, 64 and 130 tokens in portions of 24 beside decoding requests
+    vocab = TINY["B"]["config"]["vocab_size"]
+    prompts = [random_tokens(n, vocab, 50 + n) for n in (1, 9, 64, 130)]
+    want = _plain_greedy(model_folders["B"], prompts, 6)
+    engine = SyncEngine(path=model_folders["B"], dtype="float32", device="cpu", block_size=8, num_blocks=40,
+                        max_num_seqs=4, max_num_tokens=30, chunked_prefill_size=24)
+    got = engine.generate_ids(prompts, max_new_tokens=6, temperature=0.0, ignore_eos=True)
+    assert got == want
+
+
+def test_preemption_changes_no_token(cpu_ops, model_folders):
+    vocab = TINY["B"]["config"]["vocab_size"]
+    prompts = [random_tokens(n, vocab, 60 + n) for n in (30, 28, 17)]
+    want = _plain_greedy(model_folders["B"], prompts, 12)
+    # 11 pages of 8: the three requests need 6 + 5 + 4 pages at their ends
+    engine = SyncEngine(path=model_folders["B"], dtype="float32", device="cpu", block_size=8, num_blocks=11,
+                        max_num_seqs=3, chunked_prefill_size=16)
+    requests = [engine.add_request(p, engine.default_params(12, temperature=0.0, ignore_eos=True))
+                for p in prompts]
+    while engine.scheduler.has_work():
+        engine.step()
+        engine.runner.manager.audit()
+    assert [r.generated for r in requests] == want
+    assert sum(r.preemptions for r in requests) > 0
+    assert engine.runner.manager.num_free() == 11
+
+
+def test_stream_and_metrics(cpu_ops, model_folders):
+    engine = SyncEngine(path=model_folders["A"], dtype="float32", device="cpu", num_blocks=8, max_num_seqs=2)
+    engine.warmup()
+    chunks = list(engine.generate_stream([3, 1, 4, 1, 5], max_new_tokens=4, temperature=0.0, ignore_eos=True))
+    assert len(chunks) == 4 and chunks[-1].metrics.token_count == 4
+    assert chunks[0].metrics.tps == 0.0 and chunks[-1].metrics.total_elapsed >= chunks[0].metrics.ttft
+    assert chunks[0].prompt_tokens == 5
+    texts, batch = engine.batch_generate([[1, 2, 3], [4, 5]], max_new_tokens=3, ignore_eos=True, temperature=0.0)
+    assert batch.num_requests == 2 and batch.total_tokens == 6 and len(batch.per_request) == 2
+    assert len(texts[0].split()) == 3
+    with pytest.raises(ValueError):
+        engine.generate("text needs a tokenizer", 2)
+
+
+def test_sampling_is_reproducible_per_request(cpu_ops, model_folders):
+    vocab = TINY["B"]["config"]["vocab_size"]
+    prompts = [random_tokens(n, vocab, 70 + n) for n in (9, 20)]
+    kw = dict(path=model_folders["B"], dtype="float32", device="cpu", block_size=8, num_blocks=40)
+    alone = SyncEngine(max_num_seqs=1, **kw).generate_ids([prompts[0]], 8, temperature=0.8, seed=5,
+                                                          ignore_eos=True)[0]
+    both = SyncEngine(max_num_seqs=2, **kw).generate_ids(prompts, 8, temperature=0.8, seed=5, ignore_eos=True)
+    assert both[0] == alone
+    other = SyncEngine(max_num_seqs=1, **kw).generate_ids([prompts[0]], 8, temperature=0.8, seed=6,
+                                                          ignore_eos=True)[0]
+    assert other != alone

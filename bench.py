@@ -1,0 +1,161 @@
+"""Decode and prefill throughput of the Qwen3-8B-shaped model on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L]
+
+Random bfloat16 weights, uniform-random prompts of 2,048 tokens, greedy decoding
+through the engine's own step loop (scheduler, step function, sampling). A
+"step" is one decode step of the whole batch. One JSON line is printed:
+`value` is decoded tokens per second at the default batch; `prefill` is one
+2,048-token prompt in one step; `roofline` prices the decode step against HBM
+bandwidth; `points` holds decoding at batch 1 and 64.
+"""
+
+import argparse
+import json
+import sys
+import time
+
+PEAK_HBM = 8.0e12            # bytes/s, MI355X HBM3E
+PEAK_FLOPS = {"bfloat16": 2.5e15, "float32": 157.3e12}   # dense MFMA peaks
+
+QWEN3_8B = dict(architectures=["Qwen3ForCausalLM"], vocab_size=151936, hidden_size=4096, hidden_act="silu",
+                num_hidden_layers=36, max_position_embeddings=40960, num_attention_heads=32,
+                num_key_value_heads=8, head_dim=128, intermediate_size=12288, rms_norm_eps=1e-6,
+                rope_theta=1000000.0, tie_word_embeddings=False)
+CONTEXT = 8192
+PROMPT = 2048
+BLOCK = 16
+
+
+def layer_params(c):
+    qkv = (c.num_attention_heads + 2 * c.num_key_value_heads) * c.head_dim * c.hidden_size
+    o = c.hidden_size * c.num_attention_heads * c.head_dim
+    mlp = 3 * c.hidden_size * c.intermediate_size
+    return qkv + o + mlp
+
+
+def decode_bytes(c, contexts, itemsize):
+    """Bytes one decode step has to read: every weight it uses once, and the
+    keys and values of the live requests."""
+    weights = (c.num_hidden_layers * layer_params(c) + c.vocab_size * c.hidden_size) * itemsize
+    kv_per_token = 2 * c.num_hidden_layers * c.num_key_value_heads * c.head_dim * itemsize
+    return weights + kv_per_token * sum(contexts)
+
+
+def prefill_flops(c, tokens):
+    gemm = 2.0 * tokens * c.num_hidden_layers * layer_params(c) + 2.0 * c.vocab_size * c.hidden_size
+    attn = 4.0 * (tokens * (tokens + 1) / 2) * c.head_dim * c.num_attention_heads * c.num_hidden_layers
+    return gemm + attn
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration (0 = all)")
+    ap.add_argument("--dtype", default="bfloat16")
+    ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 points")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this engine runs on one GPU; --gpus %d is not supported" % args.gpus)
+        return 2
+
+    import torch
+
+    from qwen3_from_scratch_amd.config import ModelConfig
+    from qwen3_from_scratch_amd.engine import SyncEngine, random_model
+
+    raw = dict(QWEN3_8B)
+    full_layers = raw["num_hidden_layers"]
+    if args.layers:
+        raw["num_hidden_layers"] = args.layers
+    config = ModelConfig.from_dict(raw)
+    itemsize = 2 if args.dtype == "bfloat16" else 4
+    torch.cuda.set_device(0)
+    model = random_model(config, dtype=args.dtype, device="cuda:0", seed=0, std=0.02)
+    gen = torch.Generator().manual_seed(1)
+
+    def prompts(n):
+        return [torch.randint(0, config.vocab_size, (PROMPT,), generator=gen).tolist() for _ in range(n)]
+
+    def engine_for(batch):
+        pages = batch * (CONTEXT // BLOCK)
+        return SyncEngine(model=model, path="", dtype=args.dtype, device="cuda:0", max_len=CONTEXT,
+                          block_size=BLOCK, num_blocks=pages, max_num_seqs=batch,
+                          max_num_tokens=max(PROMPT, batch), chunked_prefill_size=PROMPT)
+
+    def sync():
+        torch.cuda.synchronize()
+
+    # ---- prefill: one prompt of 2,048 tokens in one step ----
+    engine = engine_for(1)
+    for _ in range(2):                               # warm-up, then the timed one
+        req = engine.add_request(prompts(1)[0], engine.default_params(1, temperature=0.0, ignore_eos=True))
+        sync()
+        t0 = time.perf_counter()
+        plan = engine.step()
+        sync()
+        prefill_s = time.perf_counter() - t0
+        assert len(plan) == 1 and plan[0].num_tokens == PROMPT
+        while engine.scheduler.has_work():
+            engine.step()
+    prefill = {"value": round(PROMPT / prefill_s, 1), "tokens": PROMPT, "ms": round(prefill_s * 1e3, 3),
+               "frac": round(prefill_flops(config, PROMPT) / prefill_s / PEAK_FLOPS[args.dtype], 4)}
+    del engine
+
+    # ---- decode ----
+    def decode(batch, steps, warmup):
+        engine = engine_for(batch)
+        params = engine.default_params(CONTEXT - PROMPT - 1, temperature=0.0, ignore_eos=True)
+        requests = [engine.add_request(p, params) for p in prompts(batch)]
+        while any(r.is_prefill for r in requests) or len(engine.scheduler.waiting):
+            engine.step()
+        for _ in range(warmup):
+            engine.step()
+        contexts = [r.num_tokens for r in requests]
+        sync()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            plan = engine.step()
+        sync()
+        dt = time.perf_counter() - t0
+        assert len(plan) == batch and all(s.num_tokens == 1 for s in plan)
+        mean_contexts = [n + steps / 2 for n in contexts]
+        return batch * steps / dt, dt / steps, mean_contexts
+
+    tps, step_s, contexts = decode(args.batch, args.steps, args.warmup)
+    need = decode_bytes(config, contexts, itemsize)
+    roofline = {"bound": "hbm", "achieved": round(need / step_s / 1e9, 1), "peak": PEAK_HBM / 1e9,
+                "unit": "GB/s", "frac": round(need / step_s / PEAK_HBM, 4)}
+    points = {}
+    if not args.no_points:
+        for b in (1, 64):
+            if b == args.batch:
+                points["decode_b%d" % b] = round(tps, 1)
+                continue
+            p_tps, _, _ = decode(b, max(16, args.steps // 4), max(4, args.warmup // 2))
+            points["decode_b%d" % b] = round(p_tps, 1)
+
+    line = {
+        "metric": "decode tok/s at batch 1/8/64 + prefill tok/s at 2048 tokens, Qwen3-8B bf16",
+        "value": round(tps, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
+        "config": {
+            "model": "Qwen3-8B-shaped, random weights N(0, 0.02)", "global_batch": args.batch,
+            "seq_len": PROMPT, "parallelism": "single-gpu", "context_len": CONTEXT,
+            "layers": config.num_hidden_layers, "layers_full": full_layers, "hidden_size": config.hidden_size,
+            "num_attention_heads": config.num_attention_heads, "num_key_value_heads": config.num_key_value_heads,
+            "head_dim": config.head_dim, "intermediate_size": config.intermediate_size,
+            "vocab_size": config.vocab_size, "kv_block_size": BLOCK, "sampling": "greedy",
+        },
+        "prefill": prefill, "roofline": roofline, "points": points,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -10,27 +10,32 @@ class LayerCacheView:
     """What one mixer sees of the cache in one step."""
 
     keys: torch.Tensor = None          # (pages, kv_heads, page_size, head_dim)
-    values: torch.Tensor = None
+    values: torch.Tensor = None        # (pages, kv_heads, head_dim, page_size)
     block_table: torch.Tensor = None   # int32 (B, W), this step's requests in batch order
     writes: bool = True
     state: torch.Tensor = None         # (slots, *state_shape); index with batch.state_slots
 
 
 class CacheStorage:
-    """Per paged group one tensor (planes, 2, pages, kv_heads, page_size, head_dim)
-    in the activation dtype: within a page, one head's rows are contiguous, so a
-    workgroup that serves one key head streams page_size * head_dim elements at a
-    time. Per state group one tensor (planes, slots, *shape), zeroed per slot
-    at admission."""
+    """Per paged group two tensors in the activation dtype: keys
+    (planes, pages, kv_heads, page_size, head_dim) and values
+    (planes, pages, kv_heads, head_dim, page_size). Within a page one head's
+    keys are contiguous, so a workgroup that serves one key head streams
+    page_size * head_dim elements at a time; values are kept transposed within
+    the page, so that the keys a matrix-core lane multiplies together lie side
+    by side in memory and need no transposition on the way to the registers.
+    Per state group one tensor (planes, slots, *shape), zeroed per slot at
+    admission."""
 
     def __init__(self, manager, act_dtype, device):
         self.manager = manager
         self.device = torch.device(device)
-        self.paged = []
+        self.keys, self.values = [], []
         for grp in manager.groups:
-            self.paged.append(torch.zeros(
-                (len(grp.planes), 2, grp.pool.num_pages, grp.kv_heads, manager.page_size, grp.head_dim),
-                dtype=act_dtype, device=self.device))
+            shape = (len(grp.planes), grp.pool.num_pages, grp.kv_heads, manager.page_size, grp.head_dim)
+            self.keys.append(torch.zeros(shape, dtype=act_dtype, device=self.device))
+            self.values.append(torch.zeros(shape[:3] + (grp.head_dim, manager.page_size),
+                                           dtype=act_dtype, device=self.device))
         self.states = []
         for grp in manager.state_groups:
             self.states.append(torch.zeros(
@@ -39,7 +44,7 @@ class CacheStorage:
         self._block_tables = None
 
     def bytes(self):
-        return sum(t.numel() * t.element_size() for t in self.paged + self.states)
+        return sum(t.numel() * t.element_size() for t in self.keys + self.values + self.states)
 
     def clear_fresh_slots(self):
         fresh, self.manager.fresh_slots = self.manager.fresh_slots, []
@@ -58,8 +63,8 @@ class CacheStorage:
         g = m.group_of_plane[plane]
         if g >= 0:
             local = m.groups[g].planes.index(plane)
-            view.keys = self.paged[g][local, 0]
-            view.values = self.paged[g][local, 1]
+            view.keys = self.keys[g][local]
+            view.values = self.values[g][local]
             view.block_table = self._block_tables[g]
         s = m.state_group_of_plane[plane]
         if s >= 0:

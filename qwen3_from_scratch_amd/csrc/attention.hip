@@ -1,7 +1,8 @@
 // Causal softmax attention of packed query rows over paged keys and values.
 //
-// Layout: caches are (pages, Hkv, page, D); sequence b's key j lives in page
-// block_table[b, j / page] at row j % page. Query row i of a sequence with q_len
+// Layout: the key cache is (pages, Hkv, page, D), the value cache is transposed
+// within the page, (pages, Hkv, D, page); sequence b's key j lives in page
+// block_table[b, j / page] at slot j % page. Query row i of a sequence with q_len
 // rows and kv_len keys sits at position kv_len - q_len + i and sees keys at
 // positions <= its own, and, with a window w > 0, only those fewer than w behind.
 #include "common.h"
@@ -114,9 +115,9 @@ __global__ __launch_bounds__(256) void attn_general_kernel(
       const T* src = nullptr;
       if (kj < k_end) {
         const int pg = block_table[(size_t)b * bt_stride + kj / page];
-        if (pg >= 0 && pg < num_pages) src = v_cache + (((size_t)pg * Hkv + g) * page + kj % page) * D;
+        if (pg >= 0 && pg < num_pages) src = v_cache + ((size_t)pg * Hkv + g) * D * page + kj % page;
       }
-      for (int d = sub; d < D; d += 16) kv[jj * ldk + d] = src ? to_float(src[d]) : 0.f;
+      for (int d = sub; d < D; d += 16) kv[jj * ldk + d] = src ? to_float(src[(size_t)d * page]) : 0.f;
     }
     __syncthreads();
     for (int jj = 0; jj < GEN_BN; ++jj) {
@@ -148,16 +149,426 @@ static int launch_general(const void* q, int q_stride, void* out, const void* k_
   return q3_launch_status();
 }
 
+
+// ---------------------------------------------------------------------------
+// The matrix-core kernels: bfloat16, head size 64 or 128, page size a multiple
+// of 16. One wavefront works on query rows in blocks of 16 against tiles of 32
+// keys, with v_mfma_f32_16x16x32_bf16:
+//
+//   S^T (keys x rows)  = K (keys x d) . Q^T (d x rows)        A = K rows, B = Q rows
+//   O^T (d x rows)    += V^T (d x keys) . P^T (keys x rows)   A = V^T rows, B = P
+//
+// Both products put the query row in the lane's low four bits (lane % 16), so
+// the softmax statistics of a row, its probabilities and its output
+// accumulators all live in the same lanes and nothing is transposed. A lane of
+// group g = lane / 16 holds, after S^T, the scores of keys 4g..4g+3 of each of
+// the tile's two 16-key blocks; these eight are exactly the keys its P operand
+// multiplies, and the value cache is transposed within the page so that the
+// matching V^T operand is two 8-byte loads. K operands are 16-byte loads. No
+// shared memory is used on the way from the cache to the matrix cores.
+//
+// A "row" is a (token, query head of the group) pair: row r of a workgroup is
+// token r / G, head r % G of the key head's group, so that all heads of a group
+// share each key and value load.
+// ---------------------------------------------------------------------------
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+
+union Pack16 {
+  uint4 u;
+  uint2 h[2];
+  bf16x8_t v;
+  __bf16 e[8];
+};
+
+#define FAST_TILE 32
+
+// Scores, softmax update and value accumulation of one 32-key tile for QB
+// blocks of 16 rows. row_pos[qb]: position of this lane's row, below zero for a
+// row that does not exist. m, l: running maximum (log2 domain) and this lane's
+// share of the running sum.
+template <int D, int QB>
+__device__ __forceinline__ void attend_tile(const Pack16 (&qreg)[QB][D / 32], const bf16_t* __restrict__ k_cache,
+                                            const bf16_t* __restrict__ v_cache, int num_pages,
+                                            const int* __restrict__ bt_row, int Hkv, int g_kv, int page,
+                                            int key0, int kv_len, const int (&row_pos)[QB], int window,
+                                            float scale_log2, f32x4_t (&acc)[QB][D / 16], float (&m_run)[QB],
+                                            float (&l_run)[QB]) {
+  const int lane = threadIdx.x & 63;
+  const int col = lane & 15;
+  const int grp = lane >> 4;
+  // the two 16-key blocks of the tile: where they lie
+  const bf16_t* kp[2];
+  const bf16_t* vp[2];
+#pragma unroll
+  for (int kb = 0; kb < 2; ++kb) {
+    const int kbase = key0 + 16 * kb;
+    kp[kb] = nullptr;
+    vp[kb] = nullptr;
+    if (kbase < kv_len) {
+      const int pg = bt_row[kbase / page];
+      if (pg >= 0 && pg < num_pages) {
+        const int slot0 = kbase % page;
+        kp[kb] = k_cache + (((size_t)pg * Hkv + g_kv) * page + slot0 + col) * D + 8 * grp;
+        vp[kb] = v_cache + (((size_t)pg * Hkv + g_kv) * D + col) * page + slot0 + 4 * grp;
+      }
+    }
+  }
+  // S^T for both key blocks
+  f32x4_t s[QB][2];
+#pragma unroll
+  for (int kb = 0; kb < 2; ++kb) {
+    Pack16 a[D / 32];
+#pragma unroll
+    for (int i = 0; i < D / 32; ++i) {
+      if (kp[kb])
+        a[i].u = *reinterpret_cast<const uint4*>(kp[kb] + 32 * i);
+      else
+        a[i].u = make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+      f32x4_t c = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int i = 0; i < D / 32; ++i) c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i].v, qreg[qb][i].v, c, 0, 0, 0);
+      s[qb][kb] = c;
+    }
+  }
+  // values: issue the loads before the softmax arithmetic
+  Pack16 vt[D / 16];
+  const bool tail = key0 + FAST_TILE > kv_len;
+#pragma unroll
+  for (int nb = 0; nb < D / 16; ++nb) {
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+      if (vp[kb])
+        vt[nb].h[kb] = *reinterpret_cast<const uint2*>(vp[kb] + (size_t)16 * nb * page);
+      else
+        vt[nb].h[kb] = make_uint2(0, 0);
+    }
+    if (tail) {  // slots past the sequence's end hold anything: zero them, 0 * NaN is NaN
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (key0 + 16 * (j >> 2) + 4 * grp + (j & 3) >= kv_len) vt[nb].e[j] = (__bf16)0.f;
+    }
+  }
+  Pack16 p[QB];
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) {
+    float v[8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int key = key0 + 16 * (j >> 2) + 4 * grp + (j & 3);
+      bool seen = key <= row_pos[qb];
+      if (window > 0 && row_pos[qb] - key >= window) seen = false;
+      v[j] = seen ? s[qb][j >> 2][j & 3] * scale_log2 : -INFINITY;
+      mx = fmaxf(mx, v[j]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m_run[qb], mx);
+    float alpha = 1.f, sum = 0.f;
+    if (m_new > -INFINITY) {
+      alpha = exp2f(m_run[qb] - m_new);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float e = exp2f(v[j] - m_new);
+        sum += e;
+        p[qb].e[j] = (__bf16)e;
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) p[qb].e[j] = (__bf16)0.f;
+    }
+    l_run[qb] = l_run[qb] * alpha + sum;
+    m_run[qb] = m_new;
+#pragma unroll
+    for (int nb = 0; nb < D / 16; ++nb) acc[qb][nb] *= alpha;
+  }
+#pragma unroll
+  for (int nb = 0; nb < D / 16; ++nb)
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb)
+      acc[qb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt[nb].v, p[qb].v, acc[qb][nb], 0, 0, 0);
+}
+
+// ---- sequences with few rows (q_len * G <= 16): decoding ---------------------
+// grid (splits, Hkv, B), 256 threads. The four wavefronts of a block take the
+// tiles of the block's share of the keys in turn and are merged through shared
+// memory; with more than one split the block leaves an unnormalised partial
+// result (maximum, sum, accumulator) in the workspace for the reduction kernel.
+template <int D>
+__global__ __launch_bounds__(256) void attn_decode_kernel(
+    const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, const bf16_t* __restrict__ k_cache,
+    const bf16_t* __restrict__ v_cache, int num_pages, const int* __restrict__ block_table, int bt_stride,
+    const int* __restrict__ cu_q, const int* __restrict__ kv_lens, int Hq, int Hkv, int page, float scale_log2,
+    int window, int splits, float* __restrict__ ws_acc, float* __restrict__ ws_ml) {
+  const int b = blockIdx.z, g_kv = blockIdx.y, split = blockIdx.x;
+  const int G = Hq / Hkv;
+  const int q0 = cu_q[b];
+  const int q_len = cu_q[b + 1] - q0;
+  if (q_len <= 0 || q_len * G > 16) return;  // the other kernel's sequence
+  const int kv_len = kv_lens[b];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = lane & 15, grp = lane >> 4;
+  const int rows = q_len * G;
+  const int first_pos = kv_len - q_len;
+
+  int row_pos[1];
+  row_pos[0] = col < rows ? first_pos + col / G : -1;
+  Pack16 qreg[1][D / 32];
+#pragma unroll
+  for (int i = 0; i < D / 32; ++i) {
+    if (col < rows)
+      qreg[0][i].u = *reinterpret_cast<const uint4*>(q + (size_t)(q0 + col / G) * q_stride +
+                                                    (size_t)(g_kv * G + col % G) * D + 32 * i + 8 * grp);
+    else
+      qreg[0][i].u = make_uint4(0, 0, 0, 0);
+  }
+  f32x4_t acc[1][D / 16];
+#pragma unroll
+  for (int nb = 0; nb < D / 16; ++nb) acc[0][nb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  float m_run[1] = {-INFINITY}, l_run[1] = {0.f};
+
+  int tile_lo = 0;
+  if (window > 0) tile_lo = max(0, first_pos - window + 1) / FAST_TILE;
+  const int tile_hi = (kv_len + FAST_TILE - 1) / FAST_TILE;
+  const int per_split = (tile_hi - tile_lo + splits - 1) / splits;
+  const int t0 = tile_lo + split * per_split;
+  const int t1 = min(tile_hi, t0 + per_split);
+  const int* bt_row = block_table + (size_t)b * bt_stride;
+  for (int t = t0 + wave; t < t1; t += 4)
+    attend_tile<D, 1>(qreg, k_cache, v_cache, num_pages, bt_row, Hkv, g_kv, page, t * FAST_TILE, kv_len,
+                      row_pos, window, scale_log2, acc, m_run, l_run);
+
+  // this lane's sum covers its own keys only
+  float l = l_run[0];
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+
+  __shared__ float sh_m[4][16], sh_l[4][16];
+  __shared__ float sh_acc[4][16][D + 4];
+  if (grp == 0) {
+    sh_m[wave][col] = m_run[0];
+    sh_l[wave][col] = l;
+  }
+  __syncthreads();
+  float m_all = fmaxf(fmaxf(sh_m[0][col], sh_m[1][col]), fmaxf(sh_m[2][col], sh_m[3][col]));
+  const float w_mine = m_run[0] > -INFINITY ? exp2f(m_run[0] - m_all) : 0.f;
+#pragma unroll
+  for (int nb = 0; nb < D / 16; ++nb)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) sh_acc[wave][col][16 * nb + 4 * grp + j] = acc[0][nb][j] * w_mine;
+  __syncthreads();
+  // 256 threads: thread -> (row = t / 16, d = t % 16 + 16 k)
+  const int r = threadIdx.x >> 4, dd = threadIdx.x & 15;
+  if (r >= rows) return;
+  const float mr = fmaxf(fmaxf(sh_m[0][r], sh_m[1][r]), fmaxf(sh_m[2][r], sh_m[3][r]));
+  float lr = 0.f;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) lr += sh_m[w][r] > -INFINITY ? sh_l[w][r] * exp2f(sh_m[w][r] - mr) : 0.f;
+  const int token = q0 + r / G, head = g_kv * G + r % G;
+  if (splits == 1) {
+    const float inv = 1.f / lr;
+    for (int d = dd; d < D; d += 16) {
+      const float o = sh_acc[0][r][d] + sh_acc[1][r][d] + sh_acc[2][r][d] + sh_acc[3][r][d];
+      out[(size_t)token * Hq * D + (size_t)head * D + d] = float_to_bf16(o * inv);
+    }
+  } else {
+    const size_t slot = (((size_t)b * Hkv + g_kv) * splits + split) * 16 + r;
+    for (int d = dd; d < D; d += 16)
+      ws_acc[slot * D + d] = sh_acc[0][r][d] + sh_acc[1][r][d] + sh_acc[2][r][d] + sh_acc[3][r][d];
+    if (dd == 0) {
+      ws_ml[slot * 2] = mr;
+      ws_ml[slot * 2 + 1] = lr;
+    }
+  }
+}
+
+// Merge the splits' partial results: grid (Hkv, B), 256 threads.
+template <int D>
+__global__ __launch_bounds__(256) void attn_decode_reduce_kernel(
+    bf16_t* __restrict__ out, const int* __restrict__ cu_q, int Hq, int Hkv, int splits,
+    const float* __restrict__ ws_acc, const float* __restrict__ ws_ml) {
+  const int b = blockIdx.y, g_kv = blockIdx.x;
+  const int G = Hq / Hkv;
+  const int q0 = cu_q[b];
+  const int q_len = cu_q[b + 1] - q0;
+  if (q_len <= 0 || q_len * G > 16) return;
+  const int rows = q_len * G;
+  const int r = threadIdx.x >> 4, dd = threadIdx.x & 15;
+  if (r >= rows) return;
+  const size_t base = ((size_t)b * Hkv + g_kv) * splits;
+  float m_all = -INFINITY;
+  for (int s = 0; s < splits; ++s) m_all = fmaxf(m_all, ws_ml[((base + s) * 16 + r) * 2]);
+  float l_all = 0.f;
+  for (int s = 0; s < splits; ++s) {
+    const float ms = ws_ml[((base + s) * 16 + r) * 2];
+    if (ms > -INFINITY) l_all += ws_ml[((base + s) * 16 + r) * 2 + 1] * exp2f(ms - m_all);
+  }
+  const float inv = 1.f / l_all;
+  const int token = q0 + r / G, head = g_kv * G + r % G;
+  for (int d = dd; d < D; d += 16) {
+    float o = 0.f;
+    for (int s = 0; s < splits; ++s) {
+      const float ms = ws_ml[((base + s) * 16 + r) * 2];
+      if (ms > -INFINITY) o += ws_acc[((base + s) * 16 + r) * D + d] * exp2f(ms - m_all);
+    }
+    out[(size_t)token * Hq * D + (size_t)head * D + d] = float_to_bf16(o * inv);
+  }
+}
+
+// ---- sequences with many rows: portions of prompts ----------------------------
+// grid (row tiles, Hkv, B), 256 threads; a block owns 128 / G tokens x G heads,
+// each wavefront 32 rows of them (two blocks of 16) against all the keys they see.
+// Row tiles are taken from the end of the sequence first: they have the most keys.
+template <int D>
+__global__ __launch_bounds__(256) void attn_prefill_kernel(
+    const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, const bf16_t* __restrict__ k_cache,
+    const bf16_t* __restrict__ v_cache, int num_pages, const int* __restrict__ block_table, int bt_stride,
+    const int* __restrict__ cu_q, const int* __restrict__ kv_lens, int Hq, int Hkv, int page, float scale_log2,
+    int window, int tokens_per_block) {
+  const int b = blockIdx.z, g_kv = blockIdx.y;
+  const int G = Hq / Hkv;
+  const int q0 = cu_q[b];
+  const int q_len = cu_q[b + 1] - q0;
+  if (q_len * G <= 16) return;  // the other kernel's sequence
+  const int n_tiles = (q_len + tokens_per_block - 1) / tokens_per_block;
+  if ((int)blockIdx.x >= n_tiles) return;
+  const int tile = n_tiles - 1 - blockIdx.x;
+  const int kv_len = kv_lens[b];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = lane & 15, grp = lane >> 4;
+  const int first_pos = kv_len - q_len;
+  const int rows_in_block = tokens_per_block * G;  // <= 128
+
+  int row_pos[2], row_tok[2], row_head[2];
+  Pack16 qreg[2][D / 32];
+  int pos_max = -1, pos_min = 0x7fffffff;
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb) {
+    const int r = wave * 32 + qb * 16 + col;
+    const int tok = tile * tokens_per_block + r / G;
+    const bool ok = r < rows_in_block && tok < q_len;
+    row_tok[qb] = q0 + tok;
+    row_head[qb] = g_kv * G + r % G;
+    row_pos[qb] = ok ? first_pos + tok : -1;
+    if (ok) {
+      pos_max = max(pos_max, row_pos[qb]);
+      pos_min = min(pos_min, row_pos[qb]);
+    }
+#pragma unroll
+    for (int i = 0; i < D / 32; ++i) {
+      if (ok)
+        qreg[qb][i].u = *reinterpret_cast<const uint4*>(q + (size_t)row_tok[qb] * q_stride +
+                                                       (size_t)row_head[qb] * D + 32 * i + 8 * grp);
+      else
+        qreg[qb][i].u = make_uint4(0, 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    pos_max = max(pos_max, __shfl_xor(pos_max, off, 64));
+    pos_min = min(pos_min, __shfl_xor(pos_min, off, 64));
+  }
+  if (pos_max < 0) return;  // none of this wavefront's rows exists
+  f32x4_t acc[2][D / 16];
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+    for (int nb = 0; nb < D / 16; ++nb) acc[qb][nb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  float m_run[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.f, 0.f};
+
+  int tile_lo = 0;
+  if (window > 0) tile_lo = max(0, pos_min - window + 1) / FAST_TILE;
+  const int tile_hi = pos_max / FAST_TILE + 1;
+  const int* bt_row = block_table + (size_t)b * bt_stride;
+  for (int t = tile_lo; t < tile_hi; ++t)
+    attend_tile<D, 2>(qreg, k_cache, v_cache, num_pages, bt_row, Hkv, g_kv, page, t * FAST_TILE, kv_len, row_pos,
+                      window, scale_log2, acc, m_run, l_run);
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb) {
+    float l = l_run[qb];
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    if (row_pos[qb] < 0) continue;
+    const float inv = 1.f / l;
+    bf16_t* o = out + (size_t)row_tok[qb] * Hq * D + (size_t)row_head[qb] * D + 4 * grp;
+#pragma unroll
+    for (int nb = 0; nb < D / 16; ++nb) {
+      union {
+        uint2 u;
+        bf16_t e[4];
+      } pk;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) pk.e[j] = float_to_bf16(acc[qb][nb][j] * inv);
+      *reinterpret_cast<uint2*>(o + 16 * nb) = pk.u;
+    }
+  }
+}
+
+template <int D>
+static int launch_fast(const void* q, int q_stride, void* out, const void* k_cache, const void* v_cache,
+                       int num_pages, const int* block_table, int bt_stride, const int* cu_q, const int* kv_lens,
+                       int B, int Hq, int Hkv, int page, float scale, int window, int max_q_len, int min_q_len,
+                       int splits, float* ws_acc, float* ws_ml, hipStream_t stream) {
+  const int G = Hq / Hkv;
+  const float scale_log2 = scale * 1.4426950408889634f;
+  if (min_q_len * G <= 16) {
+    hipLaunchKernelGGL(attn_decode_kernel<D>, dim3(splits, Hkv, B), dim3(256), 0, stream, (const bf16_t*)q, q_stride,
+                       (bf16_t*)out, (const bf16_t*)k_cache, (const bf16_t*)v_cache, num_pages, block_table,
+                       bt_stride, cu_q, kv_lens, Hq, Hkv, page, scale_log2, window, splits, ws_acc, ws_ml);
+    if (splits > 1)
+      hipLaunchKernelGGL(attn_decode_reduce_kernel<D>, dim3(Hkv, B), dim3(256), 0, stream, (bf16_t*)out, cu_q, Hq,
+                         Hkv, splits, ws_acc, ws_ml);
+  }
+  if (max_q_len * G > 16) {
+    const int tokens_per_block = 128 / G;
+    const int tiles = (max_q_len + tokens_per_block - 1) / tokens_per_block;
+    hipLaunchKernelGGL(attn_prefill_kernel<D>, dim3(tiles, Hkv, B), dim3(256), 0, stream, (const bf16_t*)q, q_stride,
+                       (bf16_t*)out, (const bf16_t*)k_cache, (const bf16_t*)v_cache, num_pages, block_table,
+                       bt_stride, cu_q, kv_lens, Hq, Hkv, page, scale_log2, window, tokens_per_block);
+  }
+  return q3_launch_status();
+}
+
+// Whether the matrix-core kernels take this problem; otherwise the general kernel does.
+extern "C" int q3_paged_attention_fast_path(int Hq, int Hkv, int D, int page, int dtype) {
+  if (dtype != Q3_BF16) return 0;
+  if (D != 64 && D != 128) return 0;
+  if (page % 16) return 0;
+  if (Hq % Hkv || Hq / Hkv > 16) return 0;
+  return 1;
+}
+
+// Floats of workspace the split decoding needs: accumulators, then (max, sum) pairs.
+extern "C" long q3_paged_attention_workspace(int B, int Hkv, int D, int splits) {
+  return splits > 1 ? (long)B * Hkv * splits * 16 * (D + 2) : 0;
+}
+
 extern "C" int q3_paged_attention(const void* q, int q_stride, void* out, const void* k_cache,
                                   const void* v_cache, int num_pages, const int* block_table,
                                   int bt_stride, const int* cu_q, const int* kv_lens, int B, int T_, int Hq,
                                   int Hkv, int D, int page, float scale, int window, int max_q_len,
-                                  int max_kv_len, int dtype, hipStream_t stream) {
-  if (B <= 0 || T_ <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || page <= 0 || max_q_len <= 0)
+                                  int min_q_len, int max_kv_len, int dtype, int splits, float* workspace,
+                                  hipStream_t stream) {
+  if (B <= 0 || T_ <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || page <= 0 || max_q_len <= 0 || min_q_len <= 0 ||
+      min_q_len > max_q_len)
     return Q3_ERR_BAD_ARGUMENT;
   if (D % 16 || D < 16 || D > 256) return Q3_ERR_UNSUPPORTED;
   if (B > 65535 || Hq > 65535) return Q3_ERR_UNSUPPORTED;
   (void)max_kv_len;
+  if (q3_paged_attention_fast_path(Hq, Hkv, D, page, dtype) && (q_stride % 8) == 0) {
+    if (splits < 1 || splits > 65535 || (splits > 1 && workspace == nullptr)) return Q3_ERR_BAD_ARGUMENT;
+    float* ws_acc = workspace;
+    float* ws_ml = workspace ? workspace + (size_t)B * Hkv * splits * 16 * D : nullptr;
+    if (D == 64)
+      return launch_fast<64>(q, q_stride, out, k_cache, v_cache, num_pages, block_table, bt_stride, cu_q, kv_lens,
+                             B, Hq, Hkv, page, scale, window, max_q_len, min_q_len, splits, ws_acc, ws_ml, stream);
+    return launch_fast<128>(q, q_stride, out, k_cache, v_cache, num_pages, block_table, bt_stride, cu_q, kv_lens, B,
+                            Hq, Hkv, page, scale, window, max_q_len, min_q_len, splits, ws_acc, ws_ml, stream);
+  }
   Q3_DISPATCH_DTYPE(dtype, TT, return launch_general<TT>(q, q_stride, out, k_cache, v_cache, num_pages,
                                                         block_table, bt_stride, cu_q, kv_lens, B, Hq, Hkv,
                                                         D, page, scale, window, max_q_len, stream));

@@ -24,8 +24,10 @@ __global__ void rope_table_kernel(const float* __restrict__ inv_freq, float* __r
 // rotate pairs element i with i + R/2 for i < R/2 (R = rotary_dim) and leaves
 // elements >= R alone: y_i = x_i c - x_{i+R/2} s, y_{i+R/2} = x_{i+R/2} c + x_i s.
 // The cache row of token t is page block_table[seq_index[t], pos / page], slot
-// pos % page, in a cache laid out (pages, Hkv, page, D). Everything is float32
-// until the single rounding at the store.
+// pos % page. Keys are laid out (pages, Hkv, page, D); values are transposed
+// within the page, (pages, Hkv, D, page), so element j of a value row goes to
+// [page, head, j, slot]. Everything is float32 until the single rounding at the
+// store.
 template <typename T, typename W, int PER_LANE>
 __global__ void qk_norm_rope_store_kernel(T* __restrict__ qkv, const W* __restrict__ q_weight,
                                           const W* __restrict__ k_weight, float eps,
@@ -45,22 +47,26 @@ __global__ void qk_norm_rope_store_kernel(T* __restrict__ qkv, const W* __restri
 
   // where a key or value row goes, or nullptr if it is not stored
   T* dst = nullptr;
+  int dst_stride = 1;  // distance between consecutive elements of the row at dst
   if (head >= Hq && k_cache != nullptr) {
     const int b = seq_index[t];
     const int blk = pos / page_size;
     if (b >= 0 && b < bt_rows && blk < bt_stride && pos >= 0) {
       const int page = block_table[(size_t)b * bt_stride + blk];
       if (page >= 0 && page < num_pages) {
-        const int g = head < Hq + Hkv ? head - Hq : head - Hq - Hkv;
-        T* base = head < Hq + Hkv ? k_cache : v_cache;
-        dst = base + (((size_t)page * Hkv + g) * page_size + (pos % page_size)) * D;
+        if (head < Hq + Hkv) {
+          dst = k_cache + (((size_t)page * Hkv + (head - Hq)) * page_size + (pos % page_size)) * D;
+        } else {
+          dst = v_cache + ((size_t)page * Hkv + (head - Hq - Hkv)) * D * page_size + (pos % page_size);
+          dst_stride = page_size;
+        }
       }
     }
   }
 
   if (head >= Hq + Hkv) {  // a value head: copy
     if (dst)
-      for (int j = lane; j < D; j += Q3_WAVE) dst[j] = src[j];
+      for (int j = lane; j < D; j += Q3_WAVE) dst[(size_t)j * dst_stride] = src[j];
     return;
   }
 

@@ -35,6 +35,7 @@ class StepBatch:
     state_slots: torch.Tensor      # (B,) per-request slot of fixed-size state
     logits_rows: torch.Tensor      # (R,) packed rows whose logits are wanted
     max_q_len: int
+    min_q_len: int
     max_kv_len: int
     q_lens: list                   # host copies
     kv_lens_host: list
@@ -97,7 +98,8 @@ def pack_step(entries, lengths, slots, tables_per_group, device, min_table_width
         num_tokens=T, num_seqs=B,
         token_ids=dev[s_tok], positions=dev[s_pos], seq_index=dev[s_seq],
         cu_seqlens_q=dev[s_cu], kv_lens=dev[s_kv], state_slots=dev[s_slot], logits_rows=dev[s_rows],
-        max_q_len=max(q_lens) if q_lens else 0, max_kv_len=max(kv) if kv else 0,
+        max_q_len=max(q_lens) if q_lens else 0, min_q_len=min(q_lens) if q_lens else 0,
+        max_kv_len=max(kv) if kv else 0,
         q_lens=q_lens, kv_lens_host=kv,
     )
     block_tables = [dev[sl].view(B, w) for sl, w in s_tables]

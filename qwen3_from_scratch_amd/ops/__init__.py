@@ -144,8 +144,9 @@ def qk_norm_rope_store(qkv, num_q_heads, num_kv_heads, head_dim, positions, seq_
     normalised with `q_weight`, rotated, and written back in place. k heads
     are normalised with `k_weight`, rotated, and stored; v heads are stored as
     they are. The store goes to page block_table[seq_index[t], pos // page] at
-    offset pos % page of caches shaped (pages, Hkv, page, D); entries below
-    zero are skipped, and nothing is stored when no cache is given. Norm and
+    slot pos % page of a key cache shaped (pages, Hkv, page, D) and a value
+    cache shaped (pages, Hkv, D, page); entries below zero are skipped, and
+    nothing is stored when no cache is given. Norm and
     rotation are each skipped when their operand is None. The rotation pairs
     element i with i + R/2 over the first R = table.shape[1] elements.
     """
@@ -172,9 +173,10 @@ def qk_norm_rope_store(qkv, num_q_heads, num_kv_heads, head_dim, positions, seq_
     page, stride = 0, 0
     if k_cache is not None:
         _need(v_cache is not None and block_table is not None, "a cache needs k, v and a block table")
-        _need(k_cache.dim() == 4 and k_cache.shape == v_cache.shape and k_cache.shape[1] == Hkv
-              and k_cache.shape[3] == D and k_cache.dtype == qkv.dtype and v_cache.dtype == qkv.dtype,
-              "caches must be (pages, Hkv, page, D) of the activation dtype")
+        _need(k_cache.dim() == 4 and k_cache.shape[1] == Hkv and k_cache.shape[3] == D
+              and v_cache.shape == (k_cache.shape[0], Hkv, D, k_cache.shape[2])
+              and k_cache.dtype == qkv.dtype and v_cache.dtype == qkv.dtype,
+              "caches must be keys (pages, Hkv, page, D) and values (pages, Hkv, D, page) of the activation dtype")
         _need(block_table.dim() == 2 and block_table.dtype == torch.int32, "block_table must be int32 (B, W)")
         page, stride = k_cache.shape[2], block_table.shape[1]
     if T:
@@ -188,15 +190,22 @@ def qk_norm_rope_store(qkv, num_q_heads, num_kv_heads, head_dim, positions, seq_
 
 
 def paged_attention(q, num_q_heads, k_cache, v_cache, block_table, cu_seqlens_q, kv_lens,
-                    max_q_len, max_kv_len, scale, window=0, out=None):
+                    max_q_len, max_kv_len, scale, window=0, out=None, min_q_len=1):
     """Causal softmax attention of packed query rows over paged keys and values.
 
     q is (T, Hq, D) seen through a row stride (a view of the qkv buffer is
-    fine). Sequence b owns rows cu_seqlens_q[b]..cu_seqlens_q[b+1]; its keys
+    fine). Keys are cached as (pages, Hkv, page, D), values as
+    (pages, Hkv, D, page). Sequence b owns rows cu_seqlens_q[b]..cu_seqlens_q[b+1]; its keys
     0..kv_lens[b]-1 lie in pages block_table[b, j // page]; its query row i sits
     at position kv_lens[b] - q_len + i and sees keys at positions <= its own
     and, if window > 0, fewer than `window` behind it. Query head h reads
     key head h // (Hq / Hkv). Softmax statistics and accumulation are float32.
+    `max_q_len` and `min_q_len` bound the sequences' row counts (they choose
+    between the kernels for few and for many rows; loose bounds cost time only).
+
+    bfloat16 with head size 64 or 128 and a page size that is a multiple of 16
+    runs on the matrix cores; everything else (float32, other head sizes in
+    steps of 16 up to 256, other page sizes) takes the general kernel.
     """
     _dev(k_cache, v_cache, block_table, cu_seqlens_q, kv_lens, out)
     _need(q.is_cuda and q.dim() == 3 and q.stride(2) == 1 and q.stride(1) == q.shape[2],
@@ -205,9 +214,9 @@ def paged_attention(q, num_q_heads, k_cache, v_cache, block_table, cu_seqlens_q,
     _need(Hq == num_q_heads, "q's head count differs from num_q_heads")
     _need(q.dtype in _DT and k_cache.dtype == q.dtype and v_cache.dtype == q.dtype,
           "q and the caches must share bfloat16 or float32")
-    _need(k_cache.dim() == 4 and k_cache.shape == v_cache.shape and k_cache.shape[3] == D,
-          "caches must be (pages, Hkv, page, D)")
+    _need(k_cache.dim() == 4 and k_cache.shape[3] == D, "the key cache must be (pages, Hkv, page, D)")
     Hkv, page = k_cache.shape[1], k_cache.shape[2]
+    _need(v_cache.shape == (k_cache.shape[0], Hkv, D, page), "the value cache must be (pages, Hkv, D, page)")
     _need(Hq % Hkv == 0, "query heads must be a multiple of key heads")
     _need(D % 16 == 0 and 16 <= D <= 256, "head_dim must be a multiple of 16 in 16..256, found %d" % D)
     B = kv_lens.shape[0]
@@ -216,15 +225,25 @@ def paged_attention(q, num_q_heads, k_cache, v_cache, block_table, cu_seqlens_q,
     _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.shape[0] >= B,
           "block_table must be int32 (B, W)")
     _need(block_table.shape[1] * page >= max_kv_len, "block_table is narrower than the longest sequence")
+    _need(1 <= min_q_len <= max_q_len, "need 1 <= min_q_len <= max_q_len")
     if out is None:
         out = torch.empty((T, Hq * D), dtype=q.dtype, device=q.device)
     _need(out.shape == (T, Hq * D) and out.dtype == q.dtype, "out must be (T, Hq D)")
     if T and B:
-        _check(library("attention").q3_paged_attention(
+        lib = library("attention")
+        splits, workspace = 1, None
+        if lib.q3_paged_attention_fast_path(Hq, Hkv, D, page, _DT[q.dtype]) and min_q_len * (Hq // Hkv) <= 16:
+            # few rows per sequence: split the keys over blocks until the chip is full
+            splits = max(1, min(max_kv_len // 256, -(-512 // (B * Hkv))))
+            if splits > 1:
+                lib.q3_paged_attention_workspace.restype = ctypes.c_long
+                n = lib.q3_paged_attention_workspace(B, Hkv, D, splits)
+                workspace = torch.empty((n,), dtype=torch.float32, device=q.device)
+        _check(lib.q3_paged_attention(
             _ptr(q), q.stride(0), _ptr(out), _ptr(k_cache), _ptr(v_cache), k_cache.shape[0],
             _ptr(block_table), block_table.shape[1], _ptr(cu_seqlens_q), _ptr(kv_lens),
-            B, T, Hq, Hkv, D, page, ctypes.c_float(scale), int(window), int(max_q_len),
-            int(max_kv_len), _DT[q.dtype], _stream()), "paged_attention")
+            B, T, Hq, Hkv, D, page, ctypes.c_float(scale), int(window), int(max_q_len), int(min_q_len),
+            int(max_kv_len), _DT[q.dtype], splits, _ptr(workspace), _stream()), "paged_attention")
     return out
 
 

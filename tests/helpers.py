@@ -28,6 +28,19 @@ TINY = {
                     num_key_value_heads=3, head_dim=48, intermediate_size=200, rms_norm_eps=3e-6,
                     rope_theta=50000.0, tie_word_embeddings=False),
         seed=37, std=0.05, norm_jitter=0.3, page_size=16),
+    # head sizes and page sizes that the matrix-core attention kernels take
+    "D": dict(
+        config=dict(architectures=["Qwen3ForCausalLM"], vocab_size=300, hidden_size=80, hidden_act="silu",
+                    num_hidden_layers=2, max_position_embeddings=1024, num_attention_heads=4,
+                    num_key_value_heads=2, head_dim=64, intermediate_size=144, rms_norm_eps=1e-6,
+                    rope_theta=10000.0, tie_word_embeddings=True),
+        seed=41, std=0.04, norm_jitter=0.2, page_size=16),
+    "E": dict(
+        config=dict(architectures=["Qwen3ForCausalLM"], vocab_size=270, hidden_size=96, hidden_act="silu",
+                    num_hidden_layers=2, max_position_embeddings=2048, num_attention_heads=6,
+                    num_key_value_heads=1, head_dim=128, intermediate_size=160, rms_norm_eps=1e-5,
+                    rope_theta=500000.0, tie_word_embeddings=False),
+        seed=43, std=0.04, norm_jitter=0.2, page_size=32),
 }
 
 

@@ -52,7 +52,8 @@ def _compare(got, want, dtype):
     assert worst <= bound, "largest difference %g at %s (bound %g)" % (worst, where, bound)
 
 
-CASES = [("A", [5, 17, 33, 80]), ("B", [1, 9, 64, 130]), ("C", [40, 70, 3, 201])]
+CASES = [("A", [5, 17, 33, 80]), ("B", [1, 9, 64, 130]), ("C", [40, 70, 3, 201]),
+         ("D", [33, 1, 150, 64, 300]), ("E", [129, 31, 260])]
 FAMILIES = {"whole": trace_whole, "tail": trace_tail_decoded, "portions": trace_portions, "mixed": trace_mixed}
 
 

@@ -31,7 +31,7 @@ def _compare(got, want, tol):
     assert worst <= tol, "largest difference %g" % worst
 
 
-@pytest.mark.parametrize("name,lengths", [("A", [5, 17, 33]), ("B", [1, 9, 64, 130]), ("C", [40, 70])])
+@pytest.mark.parametrize("name,lengths", [("A", [5, 17, 33]), ("B", [1, 9, 64, 130]), ("C", [40, 70]), ("D", [33, 70])])
 @pytest.mark.parametrize("family", ["whole", "tail", "portions", "mixed"])
 def test_every_cutting_matches_plain(cpu_ops, model_folders, name, lengths, family):
     requests = _requests(name, lengths)

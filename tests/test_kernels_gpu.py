@@ -109,7 +109,7 @@ def test_qk_norm_rope_store(dtype, Hq, Hkv, D, R, page):
     bt = pages.cuda()
     npages = 3 * W
     kc = torch.full((npages, Hkv, page, D), -7.0, dtype=dtype, device="cuda")
-    vc = torch.full((npages, Hkv, page, D), -7.0, dtype=dtype, device="cuda")
+    vc = torch.full((npages, Hkv, D, page), -7.0, dtype=dtype, device="cuda")
     kc2, vc2 = kc.float(), vc.float()
     got = qkv.clone()
     ops.qk_norm_rope_store(got, Hq, Hkv, D, pos, seq, q_weight=qw, k_weight=kw, eps=1e-5, table=table,
@@ -138,7 +138,7 @@ def _paged_case(dtype, B, Hq, Hkv, D, page, q_lens, kv_lens, seed, spread=True):
     for b in range(B):                                    # -1 padding beyond the last page is never read
         perm[b, -(-kv_lens[b] // page):] = -1
     kc = (torch.randn((npages, Hkv, page, D), generator=g)).to(dtype).cuda()
-    vc = (torch.randn((npages, Hkv, page, D), generator=g)).to(dtype).cuda()
+    vc = (torch.randn((npages, Hkv, D, page), generator=g)).to(dtype).cuda()   # values: transposed in the page
     q = (torch.randn((T, Hq, D), generator=g) * (2.0 if spread else 1.0)).to(dtype).cuda()
     cu = torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32).cuda()
     kvl = torch.tensor(kv_lens, dtype=torch.int32).cuda()
@@ -162,6 +162,35 @@ def test_paged_attention_mixed_batch(dtype, Hq, Hkv, D, page, window):
     torch.testing.assert_close(got.float(), want, **tol)
 
 
+@pytest.mark.parametrize("Hq,Hkv,D,page", [(32, 8, 128, 16), (8, 1, 64, 32), (3, 3, 128, 64), (16, 1, 128, 16)])
+@pytest.mark.parametrize("window", [0, 300])
+def test_paged_attention_decoding_batches(Hq, Hkv, D, page, window):
+    """Single tokens over contexts from one key to thousands: one split and many."""
+    ops = _ops()
+    for kv_lens in ([1, 2, 31, 32, 33, 255, 256, 257, 1000, 3001], [700] * 3, [4097], [15] * 70):
+        B = len(kv_lens)
+        q, kc, vc, bt, cu, kvl = _paged_case(torch.bfloat16, B, Hq, Hkv, D, page, [1] * B, kv_lens, 20 + B)
+        scale = D ** -0.5
+        got = ops.paged_attention(q, Hq, kc, vc, bt, cu, kvl, 1, max(kv_lens), scale, window=window)
+        want = torch_ops.paged_attention(q.float(), Hq, kc.float(), vc.float(), bt, cu, kvl, 1, max(kv_lens),
+                                         scale, window=window)
+        torch.testing.assert_close(got.float(), want, rtol=2e-2, atol=2e-2)
+
+
+def test_paged_attention_portions_over_long_prefixes():
+    """Portions of prompts with hundreds of cached keys before them, beside single tokens."""
+    ops = _ops()
+    Hq, Hkv, D, page = 32, 8, 128, 16
+    q_lens = [512, 1, 100, 3, 33]
+    kv_lens = [512, 900, 1100, 64, 2000]
+    q, kc, vc, bt, cu, kvl = _paged_case(torch.bfloat16, 5, Hq, Hkv, D, page, q_lens, kv_lens, 31)
+    scale = D ** -0.5
+    got = ops.paged_attention(q, Hq, kc, vc, bt, cu, kvl, max(q_lens), max(kv_lens), scale, min_q_len=1)
+    want = torch_ops.paged_attention(q.float(), Hq, kc.float(), vc.float(), bt, cu, kvl, max(q_lens),
+                                     max(kv_lens), scale)
+    torch.testing.assert_close(got.float(), want, rtol=2e-2, atol=2e-2)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_paged_attention_far_key_stands_out(dtype):
     """One key far back is made to dominate: a kernel that drops, repeats or
@@ -178,7 +207,7 @@ def test_paged_attention_far_key_stands_out(dtype):
         tol = dict(rtol=1e-4, atol=2e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
         torch.testing.assert_close(got.float(), want, **tol)
         # the dominating key's value is (nearly) the answer for the first head of each group
-        v_far = vc[pg, :, far % page].float()
+        v_far = vc[pg, :, :, far % page].float()
         first = got.float().view(Hq, D)[:: Hq // Hkv]
         assert (first - v_far).abs().max() < 0.2
 
@@ -188,7 +217,7 @@ def test_paged_attention_first_token_returns_first_value():
     q, kc, vc, bt, cu, kvl = _paged_case(torch.float32, 2, 4, 2, 32, 8, [1, 1], [1, 1], 11)
     got = ops.paged_attention(q, 4, kc, vc, bt, cu, kvl, 1, 1, 32 ** -0.5).view(2, 4, 32)
     for b in range(2):
-        v0 = vc[int(bt[b, 0]), :, 0]
+        v0 = vc[int(bt[b, 0]), :, :, 0]
         torch.testing.assert_close(got[b], v0.repeat_interleave(2, dim=0), rtol=1e-6, atol=1e-6)
 
 
@@ -205,7 +234,7 @@ def test_paged_attention_ignores_garbage_beyond_the_sequence():
         for s in range(8):
             if (pg, s) not in owned:
                 kc[pg, :, s] = float("nan")
-                vc[pg, :, s] = float("nan")
+                vc[pg, :, :, s] = float("nan")
     b_ = ops.paged_attention(q, 4, kc, vc, bt, cu, kvl, 3, 21, 0.2)
     assert torch.equal(a, b_)
 

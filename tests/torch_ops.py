@@ -85,12 +85,12 @@ def qk_norm_rope_store(qkv, num_q_heads, num_kv_heads, head_dim, positions, seq_
         pages = block_table[seq_index.long(), pos // page].long()
         ok = pages >= 0
         k_cache[pages[ok], :, (pos % page)[ok]] = k[ok].to(k_cache.dtype)
-        v_cache[pages[ok], :, (pos % page)[ok]] = v[ok].to(v_cache.dtype)
+        v_cache[pages[ok], :, :, (pos % page)[ok]] = v[ok].to(v_cache.dtype)     # values: (pages, Hkv, D, page)
     return qkv
 
 
 def paged_attention(q, num_q_heads, k_cache, v_cache, block_table, cu_seqlens_q, kv_lens,
-                    max_q_len, max_kv_len, scale, window=0, out=None):
+                    max_q_len, max_kv_len, scale, window=0, out=None, min_q_len=1):
     T, Hq, D = q.shape
     Hkv, page = k_cache.shape[1], k_cache.shape[2]
     G = Hq // Hkv
@@ -105,7 +105,7 @@ def paged_attention(q, num_q_heads, k_cache, v_cache, block_table, cu_seqlens_q,
         nblk = -(-L // page)
         pages = block_table[b, :nblk].long().clamp(min=0)
         K = k_cache[pages].float().permute(1, 0, 2, 3).reshape(Hkv, nblk * page, D)[:, :L]
-        V = v_cache[pages].float().permute(1, 0, 2, 3).reshape(Hkv, nblk * page, D)[:, :L]
+        V = v_cache[pages].float().permute(1, 0, 3, 2).reshape(Hkv, nblk * page, D)[:, :L]
         qpos = torch.arange(L - n, L, device=q.device)[:, None]
         kpos = torch.arange(L, device=q.device)[None, :]
         hidden = kpos > qpos

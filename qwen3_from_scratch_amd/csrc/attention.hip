@@ -356,10 +356,12 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   __syncthreads();
   float m_all = fmaxf(fmaxf(sh_m[0][col], sh_m[1][col]), fmaxf(sh_m[2][col], sh_m[3][col]));
   const float w_mine = m_run[0] > -INFINITY ? exp2f(m_run[0] - m_all) : 0.f;
+  if (col < rows) {
 #pragma unroll
-  for (int nb = 0; nb < D / 16; ++nb)
+    for (int nb = 0; nb < D / 16; ++nb)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) sh_acc[wave][col][16 * nb + 4 * grp + j] = acc[0][nb][j] * w_mine;
+      for (int j = 0; j < 4; ++j) sh_acc[wave][col][16 * nb + 4 * grp + j] = acc[0][nb][j] * w_mine;
+  }
   __syncthreads();
   // 256 threads: thread -> (row = t / 16, d = t % 16 + 16 k)
   const int r = threadIdx.x >> 4, dd = threadIdx.x & 15;
@@ -386,36 +388,52 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   }
 }
 
-// Merge the splits' partial results: grid (Hkv, B), 256 threads.
+// Merge the splits' partial results: grid (Hkv, B), 256 threads; splits <= 64.
+// The weights of the splits are formed once per row in shared memory, then
+// every thread sums a few output elements over the splits with loads that are
+// contiguous across the block.
+#define MAX_SPLITS 64
 template <int D>
 __global__ __launch_bounds__(256) void attn_decode_reduce_kernel(
     bf16_t* __restrict__ out, const int* __restrict__ cu_q, int Hq, int Hkv, int splits,
     const float* __restrict__ ws_acc, const float* __restrict__ ws_ml) {
+  __shared__ float sh_w[16][MAX_SPLITS];
   const int b = blockIdx.y, g_kv = blockIdx.x;
   const int G = Hq / Hkv;
   const int q0 = cu_q[b];
   const int q_len = cu_q[b + 1] - q0;
   if (q_len <= 0 || q_len * G > 16) return;
   const int rows = q_len * G;
-  const int r = threadIdx.x >> 4, dd = threadIdx.x & 15;
-  if (r >= rows) return;
   const size_t base = ((size_t)b * Hkv + g_kv) * splits;
-  float m_all = -INFINITY;
-  for (int s = 0; s < splits; ++s) m_all = fmaxf(m_all, ws_ml[((base + s) * 16 + r) * 2]);
-  float l_all = 0.f;
-  for (int s = 0; s < splits; ++s) {
-    const float ms = ws_ml[((base + s) * 16 + r) * 2];
-    if (ms > -INFINITY) l_all += ws_ml[((base + s) * 16 + r) * 2 + 1] * exp2f(ms - m_all);
+  for (int idx = threadIdx.x; idx < rows * splits; idx += blockDim.x) {
+    const int r = idx / splits, s = idx - r * splits;
+    sh_w[r][s] = ws_ml[((base + s) * 16 + r) * 2];  // the split's maximum, for now
   }
-  const float inv = 1.f / l_all;
-  const int token = q0 + r / G, head = g_kv * G + r % G;
-  for (int d = dd; d < D; d += 16) {
+  __syncthreads();
+  if ((int)threadIdx.x < rows) {
+    const int r = threadIdx.x;
+    float m_all = -INFINITY;
+    for (int s = 0; s < splits; ++s) m_all = fmaxf(m_all, sh_w[r][s]);
+    float l_all = 0.f;
+    for (int s = 0; s < splits; ++s) {
+      const float ms = sh_w[r][s];
+      const float e = ms > -INFINITY ? exp2f(ms - m_all) : 0.f;
+      l_all += ws_ml[((base + s) * 16 + r) * 2 + 1] * e;
+      sh_w[r][s] = e;
+    }
+    const float inv = 1.f / l_all;
+    for (int s = 0; s < splits; ++s) sh_w[r][s] *= inv;
+  }
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < rows * D; idx += blockDim.x) {
+    const int r = idx / D, d = idx - r * D;
     float o = 0.f;
     for (int s = 0; s < splits; ++s) {
-      const float ms = ws_ml[((base + s) * 16 + r) * 2];
-      if (ms > -INFINITY) o += ws_acc[((base + s) * 16 + r) * D + d] * exp2f(ms - m_all);
+      const float wgt = sh_w[r][s];
+      if (wgt != 0.f) o += ws_acc[((base + s) * 16 + r) * D + d] * wgt;
     }
-    out[(size_t)token * Hq * D + (size_t)head * D + d] = float_to_bf16(o * inv);
+    const int token = q0 + r / G, head = g_kv * G + r % G;
+    out[(size_t)token * Hq * D + (size_t)head * D + d] = float_to_bf16(o * 1.f);
   }
 }
 
@@ -560,7 +578,7 @@ extern "C" int q3_paged_attention(const void* q, int q_stride, void* out, const 
   if (B > 65535 || Hq > 65535) return Q3_ERR_UNSUPPORTED;
   (void)max_kv_len;
   if (q3_paged_attention_fast_path(Hq, Hkv, D, page, dtype) && (q_stride % 8) == 0) {
-    if (splits < 1 || splits > 65535 || (splits > 1 && workspace == nullptr)) return Q3_ERR_BAD_ARGUMENT;
+    if (splits < 1 || splits > MAX_SPLITS || (splits > 1 && workspace == nullptr)) return Q3_ERR_BAD_ARGUMENT;
     float* ws_acc = workspace;
     float* ws_ml = workspace ? workspace + (size_t)B * Hkv * splits * 16 * D : nullptr;
     if (D == 64)

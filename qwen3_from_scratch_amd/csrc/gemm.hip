@@ -88,6 +88,138 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
   }
 }
 
+
+// ---------------------------------------------------------------------------
+// bfloat16 with few rows (M <= 16 as dispatched; the kernel takes up to 64): a
+// weight-streaming kernel. Every weight is
+// read once from HBM and that read is the cost; the matrix cores do the sums
+// (v_mfma_f32_16x16x32_bf16) with 16 weight rows as the A operand and up to 16
+// rows of x as the B operand, so out^T tiles come out with x's row in the
+// lane's low bits: lane (m = lane % 16, g = lane / 16) ends with
+// out[m][n0 + 4g .. 4g+3], four consecutive outputs of one row.
+//
+// A wavefront owns a slab of 16 weight rows and a share of K; the `kw`
+// wavefronts that share a slab are summed through shared memory in a fixed
+// order, so the result does not depend on timing. Loads are 16 bytes per lane;
+// a lane's eight k-values are the same in A and B, which is all the product needs.
+// K must be a multiple of 8; rows of the weight beyond N and k beyond K read as zero.
+// ---------------------------------------------------------------------------
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+
+union Pack16 {
+  uint4 u;
+  bf16x8_t v;
+};
+
+template <int CB, typename OUT>
+__global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restrict__ x,
+                                                           const bf16_t* __restrict__ w, OUT* __restrict__ out,
+                                                           int M, int N, int K, int kw, int k_per_wave) {
+  extern __shared__ float red[];  // [waves][CB][64][4]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = lane & 15, grp = lane >> 4;
+  const int sw = (blockDim.x >> 6) / kw;
+  const int slab = blockIdx.x * sw + wave / kw;
+  const int ksplit = wave % kw;
+  const int n0 = slab * 16;
+  const int k_begin = ksplit * k_per_wave;
+  const int k_end = min(K, k_begin + k_per_wave);
+  f32x4_t acc[CB];
+#pragma unroll
+  for (int cb = 0; cb < CB; ++cb) acc[cb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  const bool row_ok = n0 + col < N;
+  const bf16_t* wp = w + (size_t)(row_ok ? n0 + col : 0) * K + 8 * grp;
+  const bf16_t* xp[CB];
+  bool x_ok[CB];
+#pragma unroll
+  for (int cb = 0; cb < CB; ++cb) {
+    x_ok[cb] = 16 * cb + col < M;
+    xp[cb] = x + (size_t)(x_ok[cb] ? 16 * cb + col : 0) * K + 8 * grp;
+  }
+  constexpr int U = CB == 1 ? 8 : (CB == 2 ? 4 : 2);
+  for (int k = k_begin; k < k_end; k += 32 * U) {
+    Pack16 a[U], b[CB][U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int kk = k + 32 * u;
+      const bool k_ok = kk + 8 * grp + 8 <= k_end;
+      a[u].u = (row_ok && k_ok) ? *reinterpret_cast<const uint4*>(wp + kk) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb)
+        b[cb][u].u = (x_ok[cb] && k_ok) ? *reinterpret_cast<const uint4*>(xp[cb] + kk) : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb)
+        acc[cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u].v, b[cb][u].v, acc[cb], 0, 0, 0);
+  }
+  if (kw > 1) {
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) red[((wave * CB + cb) * 64 + lane) * 4 + j] = acc[cb][j];
+    __syncthreads();
+    if (ksplit != 0) return;
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb)
+      for (int s = 1; s < kw; ++s)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[cb][j] += red[(((wave + s) * CB + cb) * 64 + lane) * 4 + j];
+  }
+#pragma unroll
+  for (int cb = 0; cb < CB; ++cb) {
+    const int m = 16 * cb + col;
+    if (m >= M) continue;
+    const int n = n0 + 4 * grp;
+    OUT* o = out + (size_t)m * N + n;
+    if (n + 3 < N && (N % 4) == 0) {
+      if constexpr (sizeof(OUT) == 4) {
+        *reinterpret_cast<float4*>(o) = make_float4(acc[cb][0], acc[cb][1], acc[cb][2], acc[cb][3]);
+      } else {
+        union {
+          uint2 u;
+          bf16_t e[4];
+        } pk;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) pk.e[j] = float_to_bf16(acc[cb][j]);
+        *reinterpret_cast<uint2*>(o) = pk.u;
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (n + j < N) o[j] = from_float<OUT>(acc[cb][j]);
+    }
+  }
+}
+
+template <int CB, typename OUT>
+static int launch_skinny(const void* x, const void* w, void* out, int M, int N, int K, hipStream_t stream) {
+  const int slabs = (N + 15) / 16;
+  // enough wavefronts to keep every CU's memory pipeline full, each with at least 4 k-steps
+  int kw = 1;
+  while (kw < 16 && slabs * kw < 2048 && K / (kw * 2) >= 128 && kw * 2 * CB <= 32) kw *= 2;
+  int sw = 1;
+  while (sw * kw < 4 && sw * 2 <= slabs) sw *= 2;
+  // k_per_wave: a multiple of the unrolled step, covering K
+  constexpr int U = CB == 1 ? 8 : (CB == 2 ? 4 : 2);
+  const int step = 32 * U;
+  int k_per_wave = (K + kw - 1) / kw;
+  k_per_wave = (k_per_wave + step - 1) / step * step;
+  const int blocks = (slabs + sw - 1) / sw;
+  const size_t smem = kw > 1 ? (size_t)sw * kw * CB * 64 * 4 * sizeof(float) : 0;
+  hipLaunchKernelGGL((gemm_skinny_kernel<CB, OUT>), dim3(blocks), dim3(64 * sw * kw), smem, stream, (const bf16_t*)x,
+                     (const bf16_t*)w, (OUT*)out, M, N, K, kw, k_per_wave);
+  return q3_launch_status();
+}
+
+// Whether the weight-streaming kernel takes this product.
+extern "C" int q3_linear_is_skinny(int M, int N, int K, int in_dtype) {
+  return in_dtype == Q3_BF16 && M >= 1 && M <= 16 && K % 8 == 0 && K >= 8;
+}
+
 extern "C" int q3_linear(const void* x, const void* weight, void* out, int M, int N, int K, int in_dtype,
                          int out_dtype, hipStream_t stream) {
   if (M <= 0 || N <= 0 || K <= 0) return Q3_ERR_BAD_ARGUMENT;
@@ -99,5 +231,12 @@ extern "C" int q3_linear(const void* x, const void* weight, void* out, int M, in
                        (float*)out, M, N, K);
     return q3_launch_status();
   }
-  return Q3_ERR_UNSUPPORTED;
+  if (!q3_linear_is_skinny(M, N, K, in_dtype)) return Q3_ERR_UNSUPPORTED;
+#define Q3_SKINNY(CB)                                                                      \
+  (out_dtype == Q3_F32 ? launch_skinny<CB, float>(x, weight, out, M, N, K, stream)         \
+                       : launch_skinny<CB, bf16_t>(x, weight, out, M, N, K, stream))
+  if (M <= 16) return Q3_SKINNY(1);
+  if (M <= 32) return Q3_SKINNY(2);
+  return Q3_SKINNY(4);
+#undef Q3_SKINNY
 }

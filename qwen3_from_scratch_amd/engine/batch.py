@@ -41,11 +41,20 @@ class StepBatch:
     kv_lens_host: list
 
 
-def pack_step(entries, lengths, slots, tables_per_group, device, min_table_width=1):
+def packed_size(B, T, R, widths):
+    return 3 * T + (B + 1) + 2 * B + R + sum(B * w for w in widths)
+
+
+def pack_step(entries, lengths, slots, tables_per_group, device, min_table_width=1, fixed_widths=None,
+              buffers=None, all_rows=False):
     """Build the batch on the host and move it to the device in one copy.
 
     `lengths[i]`: tokens entry i's request already has in the cache.
     `tables_per_group[g][i]`: the request's page list in group g (-1 = given back).
+    `fixed_widths`: block-table widths to use instead of the longest list's.
+    `buffers`: (pinned host int32 tensor, device int32 tensor) to pack into, so
+    that the batch lives at the same addresses every step (for graph replay).
+    `all_rows`: ask for logits at every packed row, whatever `want` says.
     Returns (StepBatch, [block table per group]).
     """
     B = len(entries)
@@ -60,12 +69,24 @@ def pack_step(entries, lengths, slots, tables_per_group, device, min_table_width
                 raise ValueError("request %r wants place %d of %d tokens" % (e.request_id, w, q_lens[i]))
             rows.append(offset + w)
         offset += q_lens[i]
+    if all_rows:
+        rows = list(range(T))
     R = len(rows)
-    widths = []
-    for tables in tables_per_group:
-        widths.append(max([min_table_width] + [len(t) for t in tables]))
-    total = 3 * T + (B + 1) + 2 * B + R + sum(B * w for w in widths)
-    host = np.empty(total, dtype=np.int32)
+    if fixed_widths is not None:
+        widths = list(fixed_widths)
+        for tables, w in zip(tables_per_group, widths):
+            if any(len(t) > w for t in tables):
+                raise ValueError("a block table is wider than the fixed width %d" % w)
+    else:
+        widths = [max([min_table_width] + [len(t) for t in tables]) for tables in tables_per_group]
+    total = packed_size(B, T, R, widths)
+    if buffers is not None:
+        host_t, dev_t = buffers
+        if host_t.numel() < total:
+            raise ValueError("the packing buffer is too small")
+        host = host_t.numpy()
+    else:
+        host = np.empty(total, dtype=np.int32)
     o = 0
 
     def put(values, n):
@@ -91,9 +112,13 @@ def pack_step(entries, lengths, slots, tables_per_group, device, min_table_width
         for i, t in enumerate(tables):
             flat[i, :len(t)] = t
         s_tables.append((put(flat.reshape(-1), B * w), w))
-    dev = torch.from_numpy(host)
-    if torch.device(device).type == "cuda":
-        dev = dev.pin_memory().to(device, non_blocking=True)
+    if buffers is not None:
+        dev_t[:total].copy_(host_t[:total], non_blocking=True)
+        dev = dev_t
+    else:
+        dev = torch.from_numpy(host)
+        if torch.device(device).type == "cuda":
+            dev = dev.pin_memory().to(device, non_blocking=True)
     batch = StepBatch(
         num_tokens=T, num_seqs=B,
         token_ids=dev[s_tok], positions=dev[s_pos], seq_index=dev[s_seq],

@@ -26,9 +26,10 @@ def random_model(config, dtype="bfloat16", device="cuda", seed=0, std=0.02, norm
     return model
 
 
-def load_runner(model_dir, dtype="bfloat16", device="cuda", page_size=16, max_tokens=8192, max_requests=32):
+def load_runner(model_dir, dtype="bfloat16", device="cuda", page_size=16, max_tokens=8192, max_requests=32,
+                use_graphs=True):
     from .runner import ModelRunner
 
     model = load_model(model_dir, dtype, device)
     num_pages = -(-max_tokens // page_size)
-    return ModelRunner(model, page_size, num_pages, max_requests)
+    return ModelRunner(model, page_size, num_pages, max_requests, use_graphs=use_graphs)

@@ -3,7 +3,48 @@
 import torch
 
 from ..cache import CacheManager, CacheStorage
-from .batch import StepEntry, pack_step
+from .batch import StepEntry, pack_step, packed_size
+
+
+class _DecodeGraph:
+    """A captured HIP graph of the model's forward pass for `B` requests with
+    one token each. The batch description lives in fixed device memory that is
+    refilled before every replay; sizes that the kernels' launches depend on
+    (the longest sequence, hence how keys are split over workgroups) are fixed
+    at the cache's capacity."""
+
+    def __init__(self, runner, B):
+        m = runner.manager
+        self.B = B
+        self.widths = [-(-runner.max_request_tokens // m.page_size)] * len(m.groups)
+        n = packed_size(B, B, B, self.widths)
+        self.host = torch.empty(n, dtype=torch.int32).pin_memory()
+        self.dev = torch.zeros(n, dtype=torch.int32, device=runner.device)
+        self.graph = None
+        self.logits = None
+        self.copied = torch.cuda.Event()
+
+    def run(self, runner, entries, lengths, slots, tables):
+        self.copied.synchronize()          # the last step's copy has left the host buffer
+        batch, block_tables = pack_step(entries, lengths, slots, tables, runner.device,
+                                        fixed_widths=self.widths, buffers=(self.host, self.dev), all_rows=True)
+        self.copied.record()
+        batch.max_kv_len = runner.max_request_tokens
+        runner.storage.bind(block_tables)
+        if self.graph is None:
+            # once eagerly on a side stream (libraries build and tune at first use), then capture
+            side = torch.cuda.Stream(device=runner.device)
+            side.wait_stream(torch.cuda.current_stream(runner.device))
+            with torch.cuda.stream(side):
+                runner.model.forward(batch, runner.storage)
+            torch.cuda.current_stream(runner.device).wait_stream(side)
+            torch.cuda.synchronize(runner.device)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                self.logits = runner.model.forward(batch, runner.storage)
+            self.graph = graph
+        self.graph.replay()
+        return self.logits
 
 
 class ModelRunner:
@@ -14,19 +55,30 @@ class ModelRunner:
     wanted places. The reference's counterpart returns sampled ids for the
     last row of every sequence (src/qwen3_from_scratch/inference/model_worker.py:212-227);
     sampling is a separate call here.
+
+    Steps in which every request brings a single token replay a captured HIP
+    graph (one per batch size), which takes the launch overhead of some
+    hundreds of kernels off the critical path; the graph runs the same model
+    code, kernels and cache as any other step.
     """
 
-    def __init__(self, model, page_size, num_pages, max_requests):
+    def __init__(self, model, page_size, num_pages, max_requests, use_graphs=True):
         self.model = model
         self.device = model.device
         self.manager = CacheManager(model.plane_needs, page_size, num_pages, max_requests)
         self.storage = CacheStorage(self.manager, model.precision.act, self.device)
         self.vocab_size = model.spec.vocab_size
         self.max_positions = getattr(model.position, "max_positions", None)
+        self.max_request_tokens = self.manager.capacity_tokens()
+        if self.max_positions is not None:
+            self.max_request_tokens = min(self.max_request_tokens, self.max_positions)
+        self.use_graphs = bool(use_graphs) and self.device.type == "cuda" and model.graph_safe()
+        self._graphs = {}
 
     def step(self, entries):
         """entries: list of StepEntry. Returns logits (R, V) float32 on the
-        device, rows in the order of the entries and of their `want`."""
+        device, rows in the order of the entries and of their `want`. The
+        tensor may be overwritten by the next call of step()."""
         if not entries:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
         seen = set()
@@ -44,14 +96,13 @@ class ModelRunner:
                 if self.length(e.request_id) + len(e.tokens) > self.max_positions:
                     raise ValueError("request %r would pass position %d, the model's last"
                                      % (e.request_id, self.max_positions - 1))
-        admitted, reserved = [], []
+        admitted = []
         try:
             for e in entries:
                 if not m.has(e.request_id):
                     m.admit(e.request_id)
                     admitted.append(e.request_id)
                 m.reserve(e.request_id, len(e.tokens))
-                reserved.append(e.request_id)
         except Exception:
             for rid in admitted:
                 m.release(rid)
@@ -59,13 +110,28 @@ class ModelRunner:
         lengths = [m.length(e.request_id) for e in entries]
         slots = [m.slot(e.request_id) for e in entries]
         tables = [[m.block_table(e.request_id, g) for e in entries] for g in range(len(m.groups))]
-        batch, block_tables = pack_step(entries, lengths, slots, tables, self.device)
         self.storage.clear_fresh_slots()
-        self.storage.bind(block_tables)
-        logits = self.model.forward(batch, self.storage)
+        if self.use_graphs and all(len(e.tokens) == 1 for e in entries):
+            logits = self._step_graph(entries, lengths, slots, tables)
+        else:
+            batch, block_tables = pack_step(entries, lengths, slots, tables, self.device)
+            self.storage.bind(block_tables)
+            logits = self.model.forward(batch, self.storage)
         for e in entries:
             m.commit(e.request_id, len(e.tokens))
         return logits
+
+    def _step_graph(self, entries, lengths, slots, tables):
+        B = len(entries)
+        graph = self._graphs.get(B)
+        if graph is None:
+            graph = self._graphs[B] = _DecodeGraph(self, B)
+        logits = graph.run(self, entries, lengths, slots, tables)
+        wanted = [i for i, e in enumerate(entries) for _ in e.want]
+        if wanted == list(range(B)):
+            return logits
+        index = torch.tensor(wanted, dtype=torch.long, device=self.device)
+        return logits.index_select(0, index)
 
     def length(self, request_id):
         return self.manager.length(request_id) if self.manager.has(request_id) else 0

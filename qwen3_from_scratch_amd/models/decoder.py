@@ -55,6 +55,12 @@ class DecoderModel:
         yield self.final_norm
         yield self.head
 
+    def graph_safe(self):
+        """Whether every part's forward may be captured in a HIP graph (no
+        host synchronisation, no shapes that depend on values). Parts say so
+        with a class attribute `graph_safe`; one that does not is taken not to be."""
+        return all(getattr(part, "graph_safe", False) for part in self.parts())
+
     def tensors(self):
         names = {}
         for part in self.parts():

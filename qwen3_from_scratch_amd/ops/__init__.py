@@ -234,7 +234,7 @@ def paged_attention(q, num_q_heads, k_cache, v_cache, block_table, cu_seqlens_q,
         splits, workspace = 1, None
         if lib.q3_paged_attention_fast_path(Hq, Hkv, D, page, _DT[q.dtype]) and min_q_len * (Hq // Hkv) <= 16:
             # few rows per sequence: split the keys over blocks until the chip is full
-            splits = max(1, min(max_kv_len // 256, -(-512 // (B * Hkv))))
+            splits = max(1, min(max_kv_len // 256, -(-512 // (B * Hkv)), 64))
             if splits > 1:
                 lib.q3_paged_attention_workspace.restype = ctypes.c_long
                 n = lib.q3_paged_attention_workspace(B, Hkv, D, splits)
@@ -250,7 +250,9 @@ def paged_attention(q, num_q_heads, k_cache, v_cache, block_table, cu_seqlens_q,
 def linear(x, weight, out_dtype=None, out=None):
     """out = x @ weight^T with float32 accumulation. x (M, K), weight (N, K).
 
-    float32 operands take a float32 kernel with no reduced-precision mode.
+    float32 operands take a float32 kernel with no reduced-precision mode;
+    bfloat16 operands with at most 16 rows take a weight-streaming matrix-core
+    kernel; bfloat16 with more rows is the vendor library's product.
     """
     _dev(x, weight, out)
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1], "x (M, K) and weight (N, K)")
@@ -263,9 +265,10 @@ def linear(x, weight, out_dtype=None, out=None):
     if out is None:
         out = torch.empty((M, N), dtype=out_dtype, device=x.device)
     _need(out.shape == (M, N) and out.dtype == out_dtype, "out must be (M, N) of out_dtype")
-    if M and x.dtype == torch.bfloat16:
-        # bfloat16 products go to the vendor library (hipBLASLt through torch), as the
-        # reference's engine uses its vendor library for them; accumulation is float32
+    if M and x.dtype == torch.bfloat16 and not library("gemm").q3_linear_is_skinny(M, N, K, 1):
+        # bfloat16 products with many rows go to the vendor library (hipBLASLt through
+        # torch), as the reference's engine uses its vendor library for them; accumulation
+        # is float32. Few rows take the weight-streaming kernel below.
         if out_dtype == torch.bfloat16:
             torch.mm(x, weight.t(), out=out)
         else:

@@ -22,6 +22,8 @@ class PagedAttention(Part):
     qk_norm_eps, window (0 = all keys), scale (None = head_dim ** -0.5).
     """
 
+    graph_safe = True
+
     def __init__(self, prefix, precision, device, hidden_size, num_heads, num_kv_heads, head_dim,
                  qk_norm=True, qk_norm_eps=1e-6, window=0, scale=None):
         super().__init__(prefix, precision, device)

@@ -58,6 +58,11 @@ class PartSpec:
 class Part:
     """Base class. `prefix` is the checkpoint name prefix of the part's tensors."""
 
+    # whether forward() may be captured in a HIP graph: it launches kernels only,
+    # never synchronises with the host, and sizes nothing by a tensor's values.
+    # A model with a part that does not declare this is run without graphs.
+    graph_safe = False
+
     def __init__(self, prefix, precision, device):
         self.prefix = prefix
         self.precision = precision

@@ -15,6 +15,8 @@ class PreNormBlock(Part):
     pair.
     """
 
+    graph_safe = True
+
     def __init__(self, prefix, precision, device):
         super().__init__(prefix, precision, device)
         self.mixer = self.feed_forward = self.mixer_norm = self.feed_forward_norm = None

@@ -10,6 +10,8 @@ class TokenEmbedding(Part):
     """x[t] = E[ids[t]], no scaling, no padding row
     (src/qwen3_from_scratch/models/qwen3.py:17-19,45)."""
 
+    graph_safe = True
+
     def __init__(self, prefix, precision, device, vocab_size, hidden_size):
         super().__init__(prefix, precision, device)
         self.vocab_size = vocab_size

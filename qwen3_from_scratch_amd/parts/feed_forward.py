@@ -13,6 +13,8 @@ class SwiGLU(Part):
     (src/qwen3_from_scratch/models/feedback.py:28-34). gate and up are kept as
     one matrix [gate | up] so that one product feeds the activation kernel."""
 
+    graph_safe = True
+
     def __init__(self, prefix, precision, device, hidden_size, intermediate_size):
         super().__init__(prefix, precision, device)
         self.hidden_size = hidden_size

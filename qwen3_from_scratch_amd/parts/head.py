@@ -13,6 +13,8 @@ class LinearHead(Part):
     `weight_name` is the full checkpoint name of W: the embedding's name ties
     the head to it (qwen3.py:69-70) and both then share one tensor."""
 
+    graph_safe = True
+
     def __init__(self, prefix, precision, device, hidden_size, vocab_size, weight_name):
         super().__init__(prefix, precision, device)
         self.hidden_size = hidden_size

@@ -15,6 +15,8 @@ class RMSNorm(Part):
     same pass; the sum, the mean and the products are float32 and the result
     is rounded once."""
 
+    graph_safe = True
+
     def __init__(self, prefix, precision, device, size, eps):
         super().__init__(prefix, precision, device)
         self.size = size

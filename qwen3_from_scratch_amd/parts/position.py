@@ -15,6 +15,8 @@ from .base import Part
 
 @register_part("position", "none")
 class NoPosition(Part):
+    graph_safe = True
+
     def __init__(self, prefix, precision, device):
         super().__init__(prefix, precision, device)
 

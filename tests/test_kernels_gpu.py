@@ -51,7 +51,7 @@ def test_swiglu(dtype, T, I):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("wdtype", DTYPES)
-@pytest.mark.parametrize("T,H", [(1, 16), (7, 1000), (33, 5120), (2, 13000)])
+@pytest.mark.parametrize("T,H", [(1, 16), (7, 1000), (33, 5120), (2, 13000), (3, 1001), (2, 20000), (5, 4096)])
 def test_rmsnorm_plain_add_and_rows(dtype, wdtype, T, H):
     ops = _ops()
     x = _rand((T, H), torch.float32, 3, scale=2.0)
@@ -254,6 +254,24 @@ def test_linear(dtype, M, N, K):
     got32 = ops.linear(x, w, out_dtype=torch.float32)
     assert got32.dtype == torch.float32
     torch.testing.assert_close(got32.double(), want, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 6144, 4096), (8, 4096, 4096), (5, 24576, 512), (16, 4096, 12288),
+                                   (17, 1000, 2056), (32, 50000, 256), (48, 777, 4104), (64, 4096, 4096)])
+def test_linear_few_rows_streams_weights(M, N, K):
+    """The shapes of decoding: every way the kernel splits K and stacks row blocks."""
+    ops = _ops()
+    x = _rand((M, K), torch.bfloat16, 18)
+    w = _rand((N, K), torch.bfloat16, 19, scale=0.05)
+    want = x.float() @ w.float().T
+    got = ops.linear(x, w, out_dtype=torch.float32)
+    torch.testing.assert_close(got, want, rtol=2e-3, atol=2e-3)
+    got16 = ops.linear(x, w)
+    torch.testing.assert_close(got16.float(), want, rtol=1.6e-2, atol=1e-2)
+    if M <= 16:
+        # up to 16 rows share one way of splitting K: a row's result does not depend on its neighbours
+        alone = ops.linear(x[:1].contiguous(), w, out_dtype=torch.float32)
+        assert torch.equal(alone[0], got[0])
 
 
 def test_linear_float32_is_true_float32():

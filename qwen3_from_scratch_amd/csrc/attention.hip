@@ -183,114 +183,187 @@ union Pack16 {
 
 #define FAST_TILE 32
 
-// Scores, softmax update and value accumulation of one 32-key tile for QB
-// blocks of 16 rows. row_pos[qb]: position of this lane's row, below zero for a
-// row that does not exist. m, l: running maximum (log2 domain) and this lane's
-// share of the running sum.
-template <int D, int QB>
-__device__ __forceinline__ void attend_tile(const Pack16 (&qreg)[QB][D / 32], const bf16_t* __restrict__ k_cache,
-                                            const bf16_t* __restrict__ v_cache, int num_pages,
-                                            const int* __restrict__ bt_row, int Hkv, int g_kv, int page,
-                                            int key0, int kv_len, const int (&row_pos)[QB], int window,
-                                            float scale_log2, f32x4_t (&acc)[QB][D / 16], float (&m_run)[QB],
-                                            float (&l_run)[QB]) {
+// v_exp_f32: 2^x without the library routine's handling of results below the
+// normal range, which are zero for our purposes (arguments are <= 0).
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// The softmax update of one block of 16 rows for one 32-key tile. s: this lane's
+// eight raw scores (two key blocks of four). Scores enter scaled by scale_log2
+// only inside the exponent: p = 2^(s * scale - m), with m the running maximum of
+// s * scale. `full` says that every key of the tile is visible to every row of
+// the wavefront, so no masking is needed. Returns the probabilities as the P
+// operand and rescales the accumulators only if some row's maximum moved.
+template <int NB>
+__device__ __forceinline__ Pack16 softmax_step(const f32x4_t (&s)[2], bool full, int key0, int grp, int row_pos,
+                                               int window, float scale_log2, float& m_run, float& l_run,
+                                               f32x4_t (&acc)[NB]) {
+  float v[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) v[j] = s[j >> 2][j & 3];
+  if (!full) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int key = key0 + 16 * (j >> 2) + 4 * grp + (j & 3);
+      bool seen = key <= row_pos;
+      if (window > 0 && row_pos - key >= window) seen = false;
+      if (!seen) v[j] = -INFINITY;
+    }
+  }
+  float mx = fmaxf(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])), fmaxf(fmaxf(v[4], v[5]), fmaxf(v[6], v[7])));
+  mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+  mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+  const float m_new = fmaxf(m_run, mx * scale_log2);
+  Pack16 p;
+  float sum = 0.f;
+  if (m_new > -INFINITY) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float e = fast_exp2(fmaf(v[j], scale_log2, -m_new));
+      sum += e;
+      p.e[j] = (__bf16)e;
+    }
+  } else {
+    p.u = make_uint4(0, 0, 0, 0);
+  }
+  const bool moved = m_new != m_run;
+  if (__builtin_amdgcn_ballot_w64(moved) != 0) {
+    const float alpha = m_new > -INFINITY ? fast_exp2(m_run - m_new) : 1.f;
+    l_run *= alpha;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) acc[nb] *= alpha;
+    m_run = m_new;
+  }
+  l_run += sum;
+  return p;
+}
+
+// Where the two 16-key blocks of the tile that starts at key0 lie in the caches
+// (nullptr for a block past the sequence's end or in a page given back), from
+// this lane's point of view: its K row and its V^T row.
+struct TileAddr {
+  const bf16_t* k[2];
+  const bf16_t* v[2];
+};
+
+__device__ __forceinline__ TileAddr tile_addr(const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+                                              int num_pages, const int* __restrict__ bt_row, int Hkv, int g_kv,
+                                              int page, int D, int key0, int kv_len) {
   const int lane = threadIdx.x & 63;
-  const int col = lane & 15;
-  const int grp = lane >> 4;
-  // the two 16-key blocks of the tile: where they lie
-  const bf16_t* kp[2];
-  const bf16_t* vp[2];
+  const int col = lane & 15, grp = lane >> 4;
+  TileAddr t;
 #pragma unroll
   for (int kb = 0; kb < 2; ++kb) {
     const int kbase = key0 + 16 * kb;
-    kp[kb] = nullptr;
-    vp[kb] = nullptr;
+    t.k[kb] = nullptr;
+    t.v[kb] = nullptr;
     if (kbase < kv_len) {
       const int pg = bt_row[kbase / page];
       if (pg >= 0 && pg < num_pages) {
         const int slot0 = kbase % page;
-        kp[kb] = k_cache + (((size_t)pg * Hkv + g_kv) * page + slot0 + col) * D + 8 * grp;
-        vp[kb] = v_cache + (((size_t)pg * Hkv + g_kv) * D + col) * page + slot0 + 4 * grp;
+        t.k[kb] = k_cache + (((size_t)pg * Hkv + g_kv) * page + slot0 + col) * D + 8 * grp;
+        t.v[kb] = v_cache + (((size_t)pg * Hkv + g_kv) * D + col) * page + slot0 + 4 * grp;
       }
     }
   }
-  // S^T for both key blocks
-  f32x4_t s[QB][2];
+  return t;
+}
+
+// The K operands of a tile: [key block][d step].
+template <int D>
+__device__ __forceinline__ void load_keys(Pack16 (&a)[2][D / 32], const TileAddr& t) {
 #pragma unroll
-  for (int kb = 0; kb < 2; ++kb) {
-    Pack16 a[D / 32];
+  for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
     for (int i = 0; i < D / 32; ++i) {
-      if (kp[kb])
-        a[i].u = *reinterpret_cast<const uint4*>(kp[kb] + 32 * i);
+      if (t.k[kb])
+        a[kb][i].u = *reinterpret_cast<const uint4*>(t.k[kb] + 32 * i);
       else
-        a[i].u = make_uint4(0, 0, 0, 0);
+        a[kb][i].u = make_uint4(0, 0, 0, 0);
     }
+}
+
+// Scores, softmax update and value accumulation of one 32-key tile for QB
+// blocks of 16 rows, with the tile's K operands already in registers. row_pos[qb]:
+// position of this lane's row, below zero for a row that does not exist. m, l:
+// running maximum (log2 domain) and this lane's share of the running sum. The
+// value loads are issued first and meet the probabilities after the softmax.
+template <int D, int QB>
+__device__ __forceinline__ void attend_tile(const Pack16 (&qreg)[QB][D / 32], const Pack16 (&a)[2][D / 32],
+                                            const TileAddr& t, int page, int key0, int kv_len,
+                                            const int (&row_pos)[QB], int window, float scale_log2,
+                                            f32x4_t (&acc)[QB][D / 16], float (&m_run)[QB], float (&l_run)[QB]) {
+  const int lane = threadIdx.x & 63;
+  const int grp = lane >> 4;
+  Pack16 vt[D / 16];
+#pragma unroll
+  for (int nb = 0; nb < D / 16; ++nb)
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+      if (t.v[kb])
+        vt[nb].h[kb] = *reinterpret_cast<const uint2*>(t.v[kb] + (size_t)16 * nb * page);
+      else
+        vt[nb].h[kb] = make_uint2(0, 0);
+    }
+  f32x4_t s[QB][2];
+#pragma unroll
+  for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
       f32x4_t c = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int i = 0; i < D / 32; ++i) c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i].v, qreg[qb][i].v, c, 0, 0, 0);
+      for (int i = 0; i < D / 32; ++i)
+        c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[kb][i].v, qreg[qb][i].v, c, 0, 0, 0);
       s[qb][kb] = c;
     }
-  }
-  // values: issue the loads before the softmax arithmetic
-  Pack16 vt[D / 16];
-  const bool tail = key0 + FAST_TILE > kv_len;
+  Pack16 p[QB];
 #pragma unroll
-  for (int nb = 0; nb < D / 16; ++nb) {
+  for (int qb = 0; qb < QB; ++qb)
+    p[qb] = softmax_step<D / 16>(s[qb], false, key0, grp, row_pos[qb], window, scale_log2, m_run[qb], l_run[qb],
+                                 acc[qb]);
+  if (key0 + FAST_TILE > kv_len) {  // slots past the sequence's end hold anything: zero them, 0 * NaN is NaN
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-      if (vp[kb])
-        vt[nb].h[kb] = *reinterpret_cast<const uint2*>(vp[kb] + (size_t)16 * nb * page);
-      else
-        vt[nb].h[kb] = make_uint2(0, 0);
-    }
-    if (tail) {  // slots past the sequence's end hold anything: zero them, 0 * NaN is NaN
+    for (int nb = 0; nb < D / 16; ++nb)
 #pragma unroll
       for (int j = 0; j < 8; ++j)
         if (key0 + 16 * (j >> 2) + 4 * grp + (j & 3) >= kv_len) vt[nb].e[j] = (__bf16)0.f;
-    }
-  }
-  Pack16 p[QB];
-#pragma unroll
-  for (int qb = 0; qb < QB; ++qb) {
-    float v[8];
-    float mx = -INFINITY;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int key = key0 + 16 * (j >> 2) + 4 * grp + (j & 3);
-      bool seen = key <= row_pos[qb];
-      if (window > 0 && row_pos[qb] - key >= window) seen = false;
-      v[j] = seen ? s[qb][j >> 2][j & 3] * scale_log2 : -INFINITY;
-      mx = fmaxf(mx, v[j]);
-    }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float m_new = fmaxf(m_run[qb], mx);
-    float alpha = 1.f, sum = 0.f;
-    if (m_new > -INFINITY) {
-      alpha = exp2f(m_run[qb] - m_new);
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const float e = exp2f(v[j] - m_new);
-        sum += e;
-        p[qb].e[j] = (__bf16)e;
-      }
-    } else {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) p[qb].e[j] = (__bf16)0.f;
-    }
-    l_run[qb] = l_run[qb] * alpha + sum;
-    m_run[qb] = m_new;
-#pragma unroll
-    for (int nb = 0; nb < D / 16; ++nb) acc[qb][nb] *= alpha;
   }
 #pragma unroll
   for (int nb = 0; nb < D / 16; ++nb)
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb)
       acc[qb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt[nb].v, p[qb].v, acc[qb][nb], 0, 0, 0);
+}
+
+// All tiles first, first + step, ... below last for one wavefront: the K operands
+// of the next tile are fetched while the current one is worked on.
+template <int D, int QB>
+__device__ __forceinline__ void attend_tiles(const Pack16 (&qreg)[QB][D / 32], const bf16_t* __restrict__ k_cache,
+                                             const bf16_t* __restrict__ v_cache, int num_pages,
+                                             const int* __restrict__ bt_row, int Hkv, int g_kv, int page, int first,
+                                             int last, int step, int kv_len, const int (&row_pos)[QB], int window,
+                                             float scale_log2, f32x4_t (&acc)[QB][D / 16], float (&m_run)[QB],
+                                             float (&l_run)[QB]) {
+  if (first >= last) return;
+  Pack16 a_cur[2][D / 32], a_nxt[2][D / 32];
+  TileAddr t_cur = tile_addr(k_cache, v_cache, num_pages, bt_row, Hkv, g_kv, page, D, first * FAST_TILE, kv_len);
+  load_keys<D>(a_cur, t_cur);
+  for (int t = first; t < last; t += step) {
+    TileAddr t_nxt;
+    const bool more = t + step < last;
+    if (more) {
+      t_nxt = tile_addr(k_cache, v_cache, num_pages, bt_row, Hkv, g_kv, page, D, (t + step) * FAST_TILE, kv_len);
+      load_keys<D>(a_nxt, t_nxt);
+    }
+    attend_tile<D, QB>(qreg, a_cur, t_cur, page, t * FAST_TILE, kv_len, row_pos, window, scale_log2, acc, m_run,
+                       l_run);
+    if (more) {
+      t_cur = t_nxt;
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int i = 0; i < D / 32; ++i) a_cur[kb][i] = a_nxt[kb][i];
+    }
+  }
 }
 
 // ---- sequences with few rows (q_len * G <= 16): decoding ---------------------
@@ -338,9 +411,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   const int t0 = tile_lo + split * per_split;
   const int t1 = min(tile_hi, t0 + per_split);
   const int* bt_row = block_table + (size_t)b * bt_stride;
-  for (int t = t0 + wave; t < t1; t += 4)
-    attend_tile<D, 1>(qreg, k_cache, v_cache, num_pages, bt_row, Hkv, g_kv, page, t * FAST_TILE, kv_len,
-                      row_pos, window, scale_log2, acc, m_run, l_run);
+  attend_tiles<D, 1>(qreg, k_cache, v_cache, num_pages, bt_row, Hkv, g_kv, page, t0 + wave, t1, 4, kv_len, row_pos,
+                     window, scale_log2, acc, m_run, l_run);
 
   // this lane's sum covers its own keys only
   float l = l_run[0];
@@ -439,14 +511,36 @@ __global__ __launch_bounds__(256) void attn_decode_reduce_kernel(
 
 // ---- sequences with many rows: portions of prompts ----------------------------
 // grid (row tiles, Hkv, B), 256 threads; a block owns 128 / G tokens x G heads,
-// each wavefront 32 rows of them (two blocks of 16) against all the keys they see.
+// each wavefront 32 rows of them (two blocks of 16). The block's threads bring
+// each 32-key tile from the cache into shared memory once, 16 bytes per load,
+// two tiles in flight (the next tile's loads are issued before the current
+// tile's arithmetic and stored after it); the wavefronts read their matrix-core
+// operands from there. K rows are padded by 16 bytes so that the sixteen rows a
+// read touches fall in different banks; V^T rows hold the tile's keys in the
+// order the P operand has them (for lane group g: keys 4g..4g+3 of the first
+// 16-key block, then of the second), so a V^T operand is one 16-byte read.
 // Row tiles are taken from the end of the sequence first: they have the most keys.
+// Block-table entries are copied to shared memory PREFILL_PAGES at a time, so
+// that no cache load waits for a table load.
+#define PREFILL_PAGES 2048
 template <int D>
-__global__ __launch_bounds__(256) void attn_prefill_kernel(
+struct PrefillSmem {
+  static constexpr int K_ROW = D * 2 + 16;   // bytes
+  static constexpr int V_ROW = 64 + 16;      // 32 keys * 2 bytes + pad
+  static constexpr int K_BYTES = FAST_TILE * K_ROW;
+  static constexpr int V_BYTES = D * V_ROW;
+  static constexpr int STAGE = K_BYTES + V_BYTES;
+};
+
+template <int D>
+__global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, int num_pages, const int* __restrict__ block_table, int bt_stride,
     const int* __restrict__ cu_q, const int* __restrict__ kv_lens, int Hq, int Hkv, int page, float scale_log2,
     int window, int tokens_per_block) {
+  typedef PrefillSmem<D> SM;
+  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * SM::STAGE];
+  __shared__ int sh_pages[PREFILL_PAGES];  // the block-table entries of the tiles in hand
   const int b = blockIdx.z, g_kv = blockIdx.y;
   const int G = Hq / Hkv;
   const int q0 = cu_q[b];
@@ -454,9 +548,13 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
   if (q_len * G <= 16) return;  // the other kernel's sequence
   const int n_tiles = (q_len + tokens_per_block - 1) / tokens_per_block;
   if ((int)blockIdx.x >= n_tiles) return;
-  const int tile = n_tiles - 1 - blockIdx.x;
+  // the first half of the key heads takes its row tiles from the sequence's end (most keys
+  // first), the second half from its start, so that blocks which come to share a CU add up
+  // to about the same work
+  const int tile = (2 * (int)blockIdx.y < Hkv || Hkv == 1) ? n_tiles - 1 - blockIdx.x : blockIdx.x;
   const int kv_len = kv_lens[b];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
   const int col = lane & 15, grp = lane >> 4;
   const int first_pos = kv_len - q_len;
   const int rows_in_block = tokens_per_block * G;  // <= 128
@@ -490,7 +588,6 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     pos_max = max(pos_max, __shfl_xor(pos_max, off, 64));
     pos_min = min(pos_min, __shfl_xor(pos_min, off, 64));
   }
-  if (pos_max < 0) return;  // none of this wavefront's rows exists
   f32x4_t acc[2][D / 16];
 #pragma unroll
   for (int qb = 0; qb < 2; ++qb)
@@ -498,13 +595,153 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     for (int nb = 0; nb < D / 16; ++nb) acc[qb][nb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   float m_run[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.f, 0.f};
 
+  // the block's range of tiles: from the window's start of its first row to its last row's position
+  const int blk_first_tok = tile * tokens_per_block;
+  const int blk_last_tok = min(q_len, blk_first_tok + tokens_per_block) - 1;
   int tile_lo = 0;
-  if (window > 0) tile_lo = max(0, pos_min - window + 1) / FAST_TILE;
-  const int tile_hi = pos_max / FAST_TILE + 1;
+  if (window > 0) tile_lo = max(0, first_pos + blk_first_tok - window + 1) / FAST_TILE;
+  const int tile_hi = (first_pos + blk_last_tok) / FAST_TILE + 1;
+  // and this wavefront's own (a wavefront whose rows do not exist has none)
+  int my_lo = tile_lo, my_hi = pos_max >= 0 ? pos_max / FAST_TILE + 1 : 0;
+  if (window > 0 && pos_max >= 0) my_lo = max(0, pos_min - window + 1) / FAST_TILE;
   const int* bt_row = block_table + (size_t)b * bt_stride;
-  for (int t = tile_lo; t < tile_hi; ++t)
-    attend_tile<D, 2>(qreg, k_cache, v_cache, num_pages, bt_row, Hkv, g_kv, page, t * FAST_TILE, kv_len, row_pos,
-                      window, scale_log2, acc, m_run, l_run);
+
+  constexpr int CHUNKS = D / 64;  // 16-byte chunks of K, and of V, per thread and tile
+  uint4 kreg[CHUNKS], vreg[CHUNKS];
+  int page_base = 0;  // sh_pages[i] is the table's entry page_base + i
+
+  // per-thread constants of the copy: which 16-key block, which row and chunk of it
+  const int page_shift = 31 - __clz(page);  // the page size is a power of two here
+  int c_kb[CHUNKS], c_koff[CHUNKS], c_voff[CHUNKS], c_h[CHUNKS];
+#pragma unroll
+  for (int u = 0; u < CHUNKS; ++u) {
+    const int idx = tid + 256 * u;
+    c_kb[u] = idx / (2 * D);
+    c_koff[u] = ((idx / (D / 8)) % 16) * D + 8 * (idx % (D / 8));
+    c_h[u] = idx & 1;
+    c_voff[u] = ((idx >> 1) % D) * page + 8 * c_h[u];
+  }
+
+  const size_t page_elems = (size_t)page * D;  // elements of one (page, head) in either cache
+  auto fetch = [&](int t) {
+    const int key0 = t * FAST_TILE;
+    if (key0 + FAST_TILE <= kv_len && window == 0) {
+      // the whole tile lies inside the sequence and no page has been given back: no checks
+#pragma unroll
+      for (int u = 0; u < CHUNKS; ++u) {
+        const int kbase = key0 + 16 * c_kb[u];
+        int pg = sh_pages[(kbase >> page_shift) - page_base];
+        pg = min(max(pg, 0), num_pages - 1);
+        const size_t base = (size_t)(pg * Hkv + g_kv) * page_elems;
+        const int slot0 = kbase & (page - 1);
+        kreg[u] = *reinterpret_cast<const uint4*>(k_cache + base + (slot0 * D + c_koff[u]));
+        vreg[u] = *reinterpret_cast<const uint4*>(v_cache + base + (c_voff[u] + slot0));
+      }
+      return;
+    }
+#pragma unroll
+    for (int u = 0; u < CHUNKS; ++u) {
+      const int kbase = key0 + 16 * c_kb[u];
+      kreg[u] = make_uint4(0, 0, 0, 0);
+      vreg[u] = make_uint4(0, 0, 0, 0);
+      if (kbase < kv_len) {
+        const int pg = sh_pages[(kbase >> page_shift) - page_base];
+        if (pg >= 0 && pg < num_pages) {
+          const size_t base = (size_t)(pg * Hkv + g_kv) * page_elems;
+          const int slot0 = kbase & (page - 1);
+          // K: chunk c of key row r of the block (rows past the end are zero)
+          if (kbase + (c_koff[u] / D) < kv_len)
+            kreg[u] = *reinterpret_cast<const uint4*>(k_cache + base + (slot0 * D + c_koff[u]));
+          // V^T: half h (8 slots) of row d of the block
+          if (kbase + 8 * c_h[u] < kv_len) {
+            Pack16 v;
+            v.u = *reinterpret_cast<const uint4*>(v_cache + base + (c_voff[u] + slot0));
+            if (kbase + 8 * c_h[u] + 8 > kv_len) {  // slots past the end hold anything: zero them (0 * NaN is NaN)
+#pragma unroll
+              for (int j = 0; j < 8; ++j)
+                if (kbase + 8 * c_h[u] + j >= kv_len) v.e[j] = (__bf16)0.f;
+            }
+            vreg[u] = v.u;
+          }
+        }
+      }
+    }
+  };
+  auto stash = [&](int stage) {
+    unsigned char* ks = smem + stage * SM::STAGE;
+    unsigned char* vs = ks + SM::K_BYTES;
+#pragma unroll
+    for (int u = 0; u < CHUNKS; ++u) {
+      const int idx = tid + 256 * u;
+      const int r = idx / (D / 8), c = idx % (D / 8);
+      *reinterpret_cast<uint4*>(ks + r * SM::K_ROW + 16 * c) = kreg[u];
+      const int h = idx & 1, d = (idx >> 1) % D, kb = idx / (2 * D);
+      // keys 8h..8h+3 belong to lane group 2h, keys 8h+4..8h+7 to group 2h+1; within a group's
+      // 16 bytes the first block's four keys come first
+      unsigned char* row = vs + d * SM::V_ROW + 8 * kb;
+      *reinterpret_cast<uint2*>(row + 16 * (2 * h)) = make_uint2(vreg[u].x, vreg[u].y);
+      *reinterpret_cast<uint2*>(row + 16 * (2 * h + 1)) = make_uint2(vreg[u].z, vreg[u].w);
+    }
+  };
+
+  // tiles are worked through in spans whose table entries fit sh_pages
+  const int tiles_per_span = max(1, (PREFILL_PAGES - 2) * (page / 16) / 2);
+  for (int span_lo = tile_lo; span_lo < tile_hi; span_lo += tiles_per_span) {
+  const int span_hi = min(tile_hi, span_lo + tiles_per_span);
+  __syncthreads();
+  page_base = (span_lo * FAST_TILE) >> page_shift;
+  {
+    const int last_page = min((kv_len - 1) >> page_shift, (span_hi * FAST_TILE - 1) >> page_shift);
+    for (int i = tid; page_base + i <= last_page; i += 256) sh_pages[i] = bt_row[page_base + i];
+  }
+  __syncthreads();
+  fetch(span_lo);
+  stash(0);
+  __syncthreads();
+  for (int t = span_lo; t < span_hi; ++t) {
+    const int stage = (t - span_lo) & 1;
+    const bool more = t + 1 < span_hi;
+    if (more) fetch(t + 1);
+    if (t >= my_lo && t < my_hi) {
+      const unsigned char* ks = smem + stage * SM::STAGE;
+      const unsigned char* vs = ks + SM::K_BYTES;
+      const int key0 = t * FAST_TILE;
+      f32x4_t sc[2][2];
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) {
+        Pack16 a[D / 32];
+#pragma unroll
+        for (int i = 0; i < D / 32; ++i)
+          a[i].u = *reinterpret_cast<const uint4*>(ks + (16 * kb + col) * SM::K_ROW + 64 * i + 16 * grp);
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb) {
+          f32x4_t c = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int i = 0; i < D / 32; ++i)
+            c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i].v, qreg[qb][i].v, c, 0, 0, 0);
+          sc[qb][kb] = c;
+        }
+      }
+      // no key of the tile is hidden from any row of this wavefront?
+      const bool full = key0 + FAST_TILE - 1 <= pos_min && (window == 0 || pos_max - key0 < window);
+      Pack16 p[2];
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb)
+        p[qb] = softmax_step<D / 16>(sc[qb], full, key0, grp, row_pos[qb], window, scale_log2, m_run[qb], l_run[qb],
+                                     acc[qb]);
+#pragma unroll
+      for (int nb = 0; nb < D / 16; ++nb) {
+        Pack16 vt;
+        vt.u = *reinterpret_cast<const uint4*>(vs + (16 * nb + col) * SM::V_ROW + 16 * grp);
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb)
+          acc[qb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt.v, p[qb].v, acc[qb][nb], 0, 0, 0);
+      }
+    }
+    if (more) stash(stage ^ 1);
+    __syncthreads();
+  }
+  }
 #pragma unroll
   for (int qb = 0; qb < 2; ++qb) {
     float l = l_run[qb];
@@ -555,7 +792,7 @@ static int launch_fast(const void* q, int q_stride, void* out, const void* k_cac
 extern "C" int q3_paged_attention_fast_path(int Hq, int Hkv, int D, int page, int dtype) {
   if (dtype != Q3_BF16) return 0;
   if (D != 64 && D != 128) return 0;
-  if (page % 16) return 0;
+  if (page < 16 || (page & (page - 1))) return 0;  // a power of two, at least 16
   if (Hq % Hkv || Hq / Hkv > 16) return 0;
   return 1;
 }

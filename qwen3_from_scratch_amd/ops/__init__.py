@@ -203,7 +203,7 @@ def paged_attention(q, num_q_heads, k_cache, v_cache, block_table, cu_seqlens_q,
     `max_q_len` and `min_q_len` bound the sequences' row counts (they choose
     between the kernels for few and for many rows; loose bounds cost time only).
 
-    bfloat16 with head size 64 or 128 and a page size that is a multiple of 16
+    bfloat16 with head size 64 or 128 and a page size that is a power of two from 16
     runs on the matrix cores; everything else (float32, other head sizes in
     steps of 16 up to 256, other page sizes) takes the general kernel.
     """

@@ -137,8 +137,8 @@ def decoder_layer(x, w, i, cfg, positions):
     return x + swiglu_mlp(h, w, p + ".mlp")
 
 
-def logits_of_sequence(cfg, w, token_ids, first_position=0):
-    """Logits (T, V) at every position of one whole sequence.
+def logits_of_sequence(cfg, w, token_ids, first_position=0, rows=None):
+    """Logits (T, V) at every position of one whole sequence (or at `rows` only).
 
     Embedding gather without scaling, the layers, the final norm, the output
     matrix, which is the embedding itself when tie_word_embeddings is set
@@ -151,6 +151,8 @@ def logits_of_sequence(cfg, w, token_ids, first_position=0):
     positions = torch.arange(first_position, first_position + len(token_ids))
     for i in range(cfg["num_hidden_layers"]):
         x = decoder_layer(x, w, i, cfg, positions)
+    if rows is not None:
+        x = x[torch.as_tensor(rows, dtype=torch.long)]
     x = rms_norm(x, w["model.norm.weight"], cfg["rms_norm_eps"])
     head = emb if cfg.get("tie_word_embeddings", False) else w["lm_head.weight"]
     return x @ head.T

@@ -1,0 +1,53 @@
+"""Layers of the Qwen3-8B configuration's sizes (hidden 4096, 32 query and 8 key
+heads of 128, feed-forward 12288, vocabulary 151936) with random weights, two of
+them instead of 36 so that the plain implementation finishes on the CPU: the
+sizes at which the matrix-core kernels, the weight-streaming GEMM and the
+vocabulary-wide head actually run."""
+
+import pytest
+import torch
+
+import plain_qwen3
+from helpers import max_live_tokens, random_tokens, run_trace, trace_mixed, trace_tail_decoded
+from qwen3_from_scratch_amd.config import ModelConfig
+from qwen3_from_scratch_amd.engine import StepEntry, load_runner
+from qwen3_from_scratch_amd.weights import write_random_model
+
+pytestmark = pytest.mark.gpu
+
+CONFIG = dict(architectures=["Qwen3ForCausalLM"], vocab_size=151936, hidden_size=4096, hidden_act="silu",
+              num_hidden_layers=2, max_position_embeddings=40960, num_attention_heads=32,
+              num_key_value_heads=8, head_dim=128, intermediate_size=12288, rms_norm_eps=1e-6,
+              rope_theta=1000000.0, tie_word_embeddings=False)
+
+
+@pytest.fixture(scope="module")
+def folder(tmp_path_factory):
+    path = str(tmp_path_factory.mktemp("real") / "two_layers")
+    write_random_model(path, ModelConfig.from_dict(CONFIG), seed=5, std=0.02, norm_jitter=0.1)
+    return path
+
+
+@pytest.fixture(scope="module")
+def truth(folder):
+    cfg, w = plain_qwen3.read_model_folder(folder)
+    requests = {"a": random_tokens(150, 151936, 1), "b": random_tokens(70, 151936, 2),
+                "c": random_tokens(33, 151936, 3)}
+    rows = {rid: sorted({0, 1, len(t) // 2, len(t) - 2, len(t) - 1}) for rid, t in requests.items()}
+    want = {rid: plain_qwen3.logits_of_sequence(cfg, w, toks, rows=rows[rid]) for rid, toks in requests.items()}
+    return requests, rows, want
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 3e-4), ("bfloat16", 6e-2)])
+@pytest.mark.parametrize("family", ["tail", "mixed"])
+def test_real_layer_sizes_match_plain(folder, truth, dtype, tol, family):
+    requests, rows, want = truth
+    steps = (trace_tail_decoded(requests, tail=32) if family == "tail" else trace_mixed(requests, seed=2))
+    runner = load_runner(folder, dtype=dtype, page_size=16, max_tokens=max_live_tokens(steps, page=16),
+                         max_requests=4)
+    got = run_trace(runner, steps)
+    for rid, logits in want.items():
+        scale = max(1.0, float(logits.abs().max()))
+        for i, p in enumerate(rows[rid]):
+            diff = float((got[(rid, p)] - logits[i]).abs().max())
+            assert diff <= tol * scale, (rid, p, diff, scale)

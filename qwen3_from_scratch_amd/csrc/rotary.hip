@@ -119,6 +119,175 @@ __global__ void qk_norm_rope_store_kernel(T* __restrict__ qkv, const W* __restri
   }
 }
 
+// ---------------------------------------------------------------------------
+// The same work for bfloat16 with 16-byte accesses, for head sizes 16, 32, 64,
+// 128 and 256 with full or no rotation: a query or key head is served by D / 16
+// lanes, each holding eight elements of the head's first half and the eight
+// that pair with them in the second half; values are transposed page by page
+// through shared memory by a second kernel.
+// ---------------------------------------------------------------------------
+union Half8 {
+  uint4 u;
+  bf16_t e[8];
+};
+
+template <typename W>
+__device__ inline void load_weights8(const W* w, float (&o)[8]);
+template <>
+__device__ inline void load_weights8<float>(const float* w, float (&o)[8]) {
+  const float4 a = *reinterpret_cast<const float4*>(w), b = *reinterpret_cast<const float4*>(w + 4);
+  o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w; o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+}
+template <>
+__device__ inline void load_weights8<bf16_t>(const bf16_t* w, float (&o)[8]) {
+  Half8 h;
+  h.u = *reinterpret_cast<const uint4*>(w);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) o[i] = bf16_to_float(h.e[i]);
+}
+
+// grid (T, ceil(heads / heads_per_block)), 256 threads; LPH = D / 16 lanes per head. With
+// STORE_V the value heads are handled here too, element by element into the transposed
+// cache (for steps of few tokens, where a second launch would cost more than it saves).
+template <typename W, int LPH, bool STORE_V>
+__global__ __launch_bounds__(256) void qk_norm_rope_store_vec_kernel(
+    bf16_t* __restrict__ qkv, const W* __restrict__ q_weight, const W* __restrict__ k_weight, float eps,
+    const float* __restrict__ table, int max_pos, const int* __restrict__ positions,
+    const int* __restrict__ seq_index, const int* __restrict__ block_table, int bt_stride, int bt_rows,
+    bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache, int page_size, int num_pages, int Hq, int Hkv) {
+  constexpr int D = LPH * 16, HALF = D / 2;
+  const int t = blockIdx.x;
+  const int head = blockIdx.y * (256 / LPH) + threadIdx.x / LPH;
+  const int c = threadIdx.x % LPH;  // which eight of the half
+  if (head >= Hq + (STORE_V ? 2 : 1) * Hkv) return;
+  bf16_t* src = qkv + ((size_t)t * (Hq + 2 * Hkv) + head) * D;
+  const int pos = positions[t];
+  Half8 x1, x2;
+  x1.u = *reinterpret_cast<const uint4*>(src + 8 * c);
+  x2.u = *reinterpret_cast<const uint4*>(src + HALF + 8 * c);
+  if (STORE_V && head >= Hq + Hkv) {
+    if (v_cache == nullptr) return;
+    const int sq = seq_index[t];
+    const int blk = pos / page_size;
+    if (sq < 0 || sq >= bt_rows || blk >= bt_stride || pos < 0) return;
+    const int page = block_table[(size_t)sq * bt_stride + blk];
+    if (page < 0 || page >= num_pages) return;
+    bf16_t* o = v_cache + ((size_t)page * Hkv + (head - Hq - Hkv)) * D * page_size + (pos % page_size);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      o[(size_t)(8 * c + i) * page_size] = x1.e[i];
+      o[(size_t)(HALF + 8 * c + i) * page_size] = x2.e[i];
+    }
+    return;
+  }
+  float a[8], b[8];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    a[i] = bf16_to_float(x1.e[i]);
+    b[i] = bf16_to_float(x2.e[i]);
+    ss += a[i] * a[i] + b[i] * b[i];
+  }
+  const W* w = head < Hq ? q_weight : k_weight;
+  if (w != nullptr) {
+#pragma unroll
+    for (int off = LPH / 2; off > 0; off >>= 1) ss += __shfl_xor(ss, off, Q3_WAVE);
+    const float scale = rsqrtf(ss / (float)D + eps);
+    float wa[8], wb[8];
+    load_weights8<W>(w + 8 * c, wa);
+    load_weights8<W>(w + HALF + 8 * c, wb);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      a[i] = a[i] * scale * wa[i];
+      b[i] = b[i] * scale * wb[i];
+    }
+  }
+  if (table != nullptr && pos >= 0 && pos < max_pos) {
+    float cs[8], sn[8];
+    load_weights8<float>(table + (size_t)pos * D + 8 * c, cs);
+    load_weights8<float>(table + (size_t)pos * D + HALF + 8 * c, sn);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float ya = a[i] * cs[i] - b[i] * sn[i];
+      const float yb = b[i] * cs[i] + a[i] * sn[i];
+      a[i] = ya;
+      b[i] = yb;
+    }
+  }
+  bf16_t* dst = src;
+  if (head >= Hq) {
+    dst = nullptr;
+    if (k_cache != nullptr) {
+      const int sq = seq_index[t];
+      const int blk = pos / page_size;
+      if (sq >= 0 && sq < bt_rows && blk < bt_stride && pos >= 0) {
+        const int page = block_table[(size_t)sq * bt_stride + blk];
+        if (page >= 0 && page < num_pages)
+          dst = k_cache + (((size_t)page * Hkv + (head - Hq)) * page_size + (pos % page_size)) * D;
+      }
+    }
+  }
+  if (dst == nullptr) return;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    x1.e[i] = float_to_bf16(a[i]);
+    x2.e[i] = float_to_bf16(b[i]);
+  }
+  *reinterpret_cast<uint4*>(dst + 8 * c) = x1.u;
+  *reinterpret_cast<uint4*>(dst + HALF + 8 * c) = x2.u;
+}
+
+// Values of this step into the transposed value cache, one block per (logical
+// page j of the step's span, key head, sequence): the rows of the up to
+// `page_size` (<= 64) tokens that fall in the page are staged in shared memory and
+// written as rows of the page, 16 bytes at a time where eight neighbouring slots
+// are all written in this step, element by element otherwise.
+template <int D>
+__global__ __launch_bounds__(256) void store_values_kernel(
+    const bf16_t* __restrict__ qkv, const int* __restrict__ cu_q, const int* __restrict__ kv_lens,
+    const int* __restrict__ block_table, int bt_stride, bf16_t* __restrict__ v_cache, int page_size,
+    int num_pages, int Hq, int Hkv) {
+  __shared__ bf16_t tile[64][D + 8];
+  const int b = blockIdx.z, g = blockIdx.y;
+  const int q0 = cu_q[b];
+  const int q_len = cu_q[b + 1] - q0;
+  if (q_len <= 0) return;
+  const int first_pos = kv_lens[b] - q_len;
+  const int blk = first_pos / page_size + blockIdx.x;       // logical page
+  const int lo = max(first_pos, blk * page_size);           // positions written in it: [lo, hi)
+  const int hi = min(first_pos + q_len, (blk + 1) * page_size);
+  if (lo >= hi) return;
+  const int page = block_table[(size_t)b * bt_stride + blk];
+  if (page < 0 || page >= num_pages) return;
+  const int heads = Hq + 2 * Hkv;
+  const int n = hi - lo;
+  for (int idx = threadIdx.x; idx < n * (D / 8); idx += 256) {
+    const int r = idx / (D / 8), c = idx % (D / 8);
+    const bf16_t* row = qkv + ((size_t)(q0 + lo - first_pos + r) * heads + Hq + Hkv + g) * D;
+    *reinterpret_cast<uint4*>(&tile[r][8 * c]) = *reinterpret_cast<const uint4*>(row + 8 * c);
+  }
+  __syncthreads();
+  const int slot_lo = lo - blk * page_size;
+  bf16_t* base = v_cache + ((size_t)page * Hkv + g) * D * page_size;
+  const int groups = page_size / 8;  // 16-byte groups of slots per row (page_size is a multiple of 8 here)
+  for (int idx = threadIdx.x; idx < D * groups; idx += 256) {
+    const int d = idx / groups, s8 = (idx % groups) * 8;
+    if (s8 + 8 <= slot_lo || s8 >= slot_lo + n) continue;
+    bf16_t* o = base + (size_t)d * page_size + s8;
+    if (s8 >= slot_lo && s8 + 8 <= slot_lo + n) {
+      Half8 h;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) h.e[i] = tile[s8 - slot_lo + i][d];
+      *reinterpret_cast<uint4*>(o) = h.u;
+    } else {
+      for (int i = 0; i < 8; ++i) {
+        const int r = s8 + i - slot_lo;
+        if (r >= 0 && r < n) o[i] = tile[r][d];
+      }
+    }
+  }
+}
+
 extern "C" int q3_rope_table(const float* inv_freq, float* table, int max_pos, int half,
                              hipStream_t stream) {
   if (max_pos <= 0 || half <= 0) return Q3_ERR_BAD_ARGUMENT;
@@ -156,16 +325,76 @@ static int launch_qk(void* qkv, const void* qw, const void* kw, float eps, const
   return q3_launch_status();
 }
 
+template <typename W>
+static int launch_qk_vec(void* qkv, const void* qw, const void* kw, float eps, const float* table, int max_pos,
+                         const int* positions, const int* seq_index, const int* block_table, int bt_stride,
+                         int bt_rows, void* k_cache, void* v_cache, int page_size, int num_pages, int T_, int Hq,
+                         int Hkv, int D, const int* cu_q, const int* kv_lens, int B, int max_q_len,
+                         hipStream_t stream) {
+  const bool few = max_q_len < 8;  // values element by element in the same launch
+  const int nheads = Hq + (few ? 2 : 1) * Hkv;
+#define Q3_QKV_LAUNCH(LPH)                                                                                   \
+  do {                                                                                                       \
+    const dim3 grid(T_, (nheads + 256 / LPH - 1) / (256 / LPH));                                             \
+    if (few)                                                                                                 \
+      hipLaunchKernelGGL((qk_norm_rope_store_vec_kernel<W, LPH, true>), grid, dim3(256), 0, stream,          \
+                         (bf16_t*)qkv, (const W*)qw, (const W*)kw, eps, table, max_pos, positions, seq_index, \
+                         block_table, bt_stride, bt_rows, (bf16_t*)k_cache, (bf16_t*)v_cache, page_size,     \
+                         num_pages, Hq, Hkv);                                                                \
+    else                                                                                                     \
+      hipLaunchKernelGGL((qk_norm_rope_store_vec_kernel<W, LPH, false>), grid, dim3(256), 0, stream,         \
+                         (bf16_t*)qkv, (const W*)qw, (const W*)kw, eps, table, max_pos, positions, seq_index, \
+                         block_table, bt_stride, bt_rows, (bf16_t*)k_cache, (bf16_t*)v_cache, page_size,     \
+                         num_pages, Hq, Hkv);                                                                \
+  } while (0)
+  switch (D) {
+    case 16: Q3_QKV_LAUNCH(1); break;
+    case 32: Q3_QKV_LAUNCH(2); break;
+    case 64: Q3_QKV_LAUNCH(4); break;
+    case 128: Q3_QKV_LAUNCH(8); break;
+    case 256: Q3_QKV_LAUNCH(16); break;
+    default: return Q3_ERR_UNSUPPORTED;
+  }
+#undef Q3_QKV_LAUNCH
+  if (v_cache != nullptr && !few) {
+    const dim3 grid((max_q_len + page_size - 1) / page_size + 1, Hkv, B);
+#define Q3_V_LAUNCH(DD)                                                                                       \
+  hipLaunchKernelGGL(store_values_kernel<DD>, grid, dim3(256), 0, stream, (const bf16_t*)qkv, cu_q, kv_lens, \
+                     block_table, bt_stride, (bf16_t*)v_cache, page_size, num_pages, Hq, Hkv)
+    switch (D) {
+      case 16: Q3_V_LAUNCH(16); break;
+      case 32: Q3_V_LAUNCH(32); break;
+      case 64: Q3_V_LAUNCH(64); break;
+      case 128: Q3_V_LAUNCH(128); break;
+      case 256: Q3_V_LAUNCH(256); break;
+    }
+#undef Q3_V_LAUNCH
+  }
+  return q3_launch_status();
+}
+
+// `cu_q`, `kv_lens`, `B`, `max_q_len` describe the step's sequences (they may be null / 0: then
+// only the one-wavefront-per-head kernel is used).
 extern "C" int q3_qk_norm_rope_store(void* qkv, const void* q_weight, const void* k_weight, int w_dtype,
                                      float eps, const float* table, int rotary_dim, int max_pos,
                                      const int* positions, const int* seq_index, const int* block_table,
                                      int bt_stride, int bt_rows, void* k_cache, void* v_cache,
                                      int page_size, int num_pages, int T_, int Hq, int Hkv, int D,
-                                     int act_dtype, hipStream_t stream) {
+                                     int act_dtype, const int* cu_q, const int* kv_lens, int B, int max_q_len,
+                                     hipStream_t stream) {
   if (T_ <= 0 || Hq <= 0 || Hkv <= 0 || D <= 0 || (Hq + 2 * Hkv + 3) / 4 > 65535) return Q3_ERR_BAD_ARGUMENT;
   if (table && (rotary_dim <= 0 || rotary_dim % 2 || rotary_dim > D)) return Q3_ERR_BAD_ARGUMENT;
   if (k_cache && (!v_cache || !block_table || page_size <= 0)) return Q3_ERR_BAD_ARGUMENT;
   if ((q_weight == nullptr) != (k_weight == nullptr)) return Q3_ERR_BAD_ARGUMENT;
+  const bool pow2_head = D == 16 || D == 32 || D == 64 || D == 128 || D == 256;
+  const bool vec = act_dtype == Q3_BF16 && pow2_head && (!table || rotary_dim == D) &&
+                   (!k_cache || (cu_q && kv_lens && B > 0 && B <= 65535 && max_q_len > 0 && page_size % 8 == 0 &&
+                                 page_size <= 64));
+  if (vec) {
+    Q3_DISPATCH_DTYPE(w_dtype, WW, return (launch_qk_vec<WW>(
+        qkv, q_weight, k_weight, eps, table, max_pos, positions, seq_index, block_table, bt_stride, bt_rows,
+        k_cache, v_cache, page_size, num_pages, T_, Hq, Hkv, D, cu_q, kv_lens, B, max_q_len, stream)));
+  }
   Q3_DISPATCH_DTYPE(act_dtype, TT, Q3_DISPATCH_DTYPE(w_dtype, WW, return (launch_qk<TT, WW>(
       qkv, q_weight, k_weight, eps, table, rotary_dim, max_pos, positions, seq_index, block_table,
       bt_stride, bt_rows, k_cache, v_cache, page_size, num_pages, T_, Hq, Hkv, D, stream))));

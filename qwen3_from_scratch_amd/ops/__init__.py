@@ -137,7 +137,8 @@ def rope_table(inv_freq, max_positions):
 
 def qk_norm_rope_store(qkv, num_q_heads, num_kv_heads, head_dim, positions, seq_index,
                        q_weight=None, k_weight=None, eps=0.0, table=None,
-                       block_table=None, k_cache=None, v_cache=None):
+                       block_table=None, k_cache=None, v_cache=None,
+                       cu_seqlens_q=None, kv_lens=None, max_q_len=0):
     """Per-head RMSNorm of q and k, rotation by position, and the cache write, in one pass.
 
     qkv (T, (Hq + 2 Hkv) D) holds [q heads | k heads | v heads]. q heads are
@@ -149,8 +150,20 @@ def qk_norm_rope_store(qkv, num_q_heads, num_kv_heads, head_dim, positions, seq_
     nothing is stored when no cache is given. Norm and
     rotation are each skipped when their operand is None. The rotation pairs
     element i with i + R/2 over the first R = table.shape[1] elements.
+    `cu_seqlens_q`, `kv_lens` (after this step's write) and `max_q_len`
+    describe the step's sequences; with them, bfloat16 steps use kernels with
+    16-byte accesses that write values page by page. positions must then be
+    kv_lens[b] - q_len[b] + i for row i of sequence b, as the step function
+    makes them.
     """
-    _dev(qkv, positions, seq_index, q_weight, k_weight, table, block_table, k_cache, v_cache)
+    _dev(qkv, positions, seq_index, q_weight, k_weight, table, block_table, k_cache, v_cache,
+         cu_seqlens_q, kv_lens)
+    if (cu_seqlens_q is None) != (kv_lens is None):
+        raise OperandError("cu_seqlens_q and kv_lens are given together or not at all")
+    if kv_lens is not None:
+        _need(kv_lens.dtype == torch.int32 and cu_seqlens_q.dtype == torch.int32
+              and cu_seqlens_q.shape == (kv_lens.shape[0] + 1,) and max_q_len > 0,
+              "cu_seqlens_q int32 (B+1,), kv_lens int32 (B,), max_q_len > 0")
     Hq, Hkv, D = num_q_heads, num_kv_heads, head_dim
     _need(qkv.dim() == 2 and qkv.shape[1] == (Hq + 2 * Hkv) * D and qkv.dtype in _DT,
           "qkv must be (T, (Hq + 2 Hkv) D) bfloat16 or float32")
@@ -185,7 +198,8 @@ def qk_norm_rope_store(qkv, num_q_heads, num_kv_heads, head_dim, positions, seq_
             _ptr(table), rotary_dim, max_pos, _ptr(positions), _ptr(seq_index),
             _ptr(block_table), stride, 0 if block_table is None else block_table.shape[0],
             _ptr(k_cache), _ptr(v_cache), page, 0 if k_cache is None else k_cache.shape[0],
-            T, Hq, Hkv, D, _DT[qkv.dtype], _stream()), "qk_norm_rope_store")
+            T, Hq, Hkv, D, _DT[qkv.dtype], _ptr(cu_seqlens_q), _ptr(kv_lens),
+            0 if kv_lens is None else kv_lens.shape[0], int(max_q_len), _stream()), "qk_norm_rope_store")
     return qkv
 
 

@@ -82,6 +82,7 @@ class PagedAttention(Part):
             block_table=cache.block_table if cache.writes else None,
             k_cache=cache.keys if cache.writes else None,
             v_cache=cache.values if cache.writes else None,
+            cu_seqlens_q=batch.cu_seqlens_q, kv_lens=batch.kv_lens, max_q_len=batch.max_q_len,
         )
         q = qkv[:, : Hq * D].unflatten(1, (Hq, D))
         o = ops.paged_attention(

@@ -92,7 +92,8 @@ def test_rope_table_matches_closed_form():
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("Hq,Hkv,D,R,page", [(4, 2, 16, 16, 16), (6, 3, 48, 48, 8), (5, 1, 80, 32, 4),
-                                             (32, 8, 128, 128, 16), (2, 2, 256, 256, 16)])
+                                             (32, 8, 128, 128, 16), (2, 2, 256, 256, 16), (7, 1, 64, 64, 8),
+                                             (8, 4, 32, 32, 32), (3, 3, 128, 128, 64)])
 def test_qk_norm_rope_store(dtype, Hq, Hkv, D, R, page):
     ops = _ops()
     T, B, P = 23, 3, 300
@@ -114,7 +115,7 @@ def test_qk_norm_rope_store(dtype, Hq, Hkv, D, R, page):
     got = qkv.clone()
     ops.qk_norm_rope_store(got, Hq, Hkv, D, pos, seq, q_weight=qw, k_weight=kw, eps=1e-5, table=table,
                            block_table=bt, k_cache=kc, v_cache=vc)
-    want = qkv.float()
+    want = qkv.float().clone()
     torch_ops.qk_norm_rope_store(want, Hq, Hkv, D, pos, seq, q_weight=qw, k_weight=kw, eps=1e-5,
                                  table=table, block_table=bt, k_cache=kc2, v_cache=vc2)
     tol = _tol(dtype)
@@ -123,6 +124,33 @@ def test_qk_norm_rope_store(dtype, Hq, Hkv, D, R, page):
     torch.testing.assert_close(kc.float(), kc2, **tol)
     assert torch.equal(vc.float(), vc2)                             # values are copied bit for bit
     assert (kc2 == -7.0).any()                                      # untouched slots keep the sentinel
+    # the same step described by its sequences: the kernels with 16-byte accesses where they apply
+    cu = torch.tensor([0, 9, 10, 23], dtype=torch.int32).cuda()
+    kvl = torch.tensor([49, 78, 13], dtype=torch.int32).cuda()
+    kc3 = torch.full_like(kc, -7.0)
+    vc3 = torch.full_like(vc, -7.0)
+    got3 = qkv.clone()
+    ops.qk_norm_rope_store(got3, Hq, Hkv, D, pos, seq, q_weight=qw, k_weight=kw, eps=1e-5, table=table,
+                           block_table=bt, k_cache=kc3, v_cache=vc3, cu_seqlens_q=cu, kv_lens=kvl, max_q_len=13)
+    torch.testing.assert_close(got3.float()[:, :Hq * D], want[:, :Hq * D], **tol)
+    assert torch.equal(got3[:, Hq * D:], qkv[:, Hq * D:])
+    torch.testing.assert_close(kc3.float(), kc2, **tol)
+    assert torch.equal(vc3.float(), vc2)
+    # and a step of few tokens per sequence (values go with the same launch)
+    few_pos = torch.tensor([48, 77, 12], dtype=torch.int32).cuda()
+    few_seq = torch.tensor([0, 1, 2], dtype=torch.int32).cuda()
+    few = qkv[:3].clone()
+    few_want = few.float().clone()
+    kc4, vc4 = torch.full_like(kc, -7.0), torch.full_like(vc, -7.0)
+    kc5, vc5 = kc4.float(), vc4.float()
+    ops.qk_norm_rope_store(few, Hq, Hkv, D, few_pos, few_seq, q_weight=qw, k_weight=kw, eps=1e-5, table=table,
+                           block_table=bt, k_cache=kc4, v_cache=vc4,
+                           cu_seqlens_q=torch.tensor([0, 1, 2, 3], dtype=torch.int32).cuda(), kv_lens=kvl, max_q_len=1)
+    torch_ops.qk_norm_rope_store(few_want, Hq, Hkv, D, few_pos, few_seq, q_weight=qw, k_weight=kw, eps=1e-5,
+                                 table=table, block_table=bt, k_cache=kc5, v_cache=vc5)
+    torch.testing.assert_close(few.float()[:, :Hq * D], few_want[:, :Hq * D], **tol)
+    torch.testing.assert_close(kc4.float(), kc5, **tol)
+    assert torch.equal(vc4.float(), vc5)
     # without norm, without rotation, without cache: q comes back as it went in
     same = qkv.clone()
     ops.qk_norm_rope_store(same, Hq, Hkv, D, pos, seq)

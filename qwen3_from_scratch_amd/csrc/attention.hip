@@ -287,14 +287,9 @@ __device__ __forceinline__ void load_keys(Pack16 (&a)[2][D / 32], const TileAddr
 // position of this lane's row, below zero for a row that does not exist. m, l:
 // running maximum (log2 domain) and this lane's share of the running sum. The
 // value loads are issued first and meet the probabilities after the softmax.
-template <int D, int QB>
-__device__ __forceinline__ void attend_tile(const Pack16 (&qreg)[QB][D / 32], const Pack16 (&a)[2][D / 32],
-                                            const TileAddr& t, int page, int key0, int kv_len,
-                                            const int (&row_pos)[QB], int window, float scale_log2,
-                                            f32x4_t (&acc)[QB][D / 16], float (&m_run)[QB], float (&l_run)[QB]) {
-  const int lane = threadIdx.x & 63;
-  const int grp = lane >> 4;
-  Pack16 vt[D / 16];
+// The V^T operands of a tile, one per block of 16 output columns.
+template <int D>
+__device__ __forceinline__ void load_values(Pack16 (&vt)[D / 16], const TileAddr& t, int page) {
 #pragma unroll
   for (int nb = 0; nb < D / 16; ++nb)
 #pragma unroll
@@ -304,6 +299,15 @@ __device__ __forceinline__ void attend_tile(const Pack16 (&qreg)[QB][D / 32], co
       else
         vt[nb].h[kb] = make_uint2(0, 0);
     }
+}
+
+template <int D, int QB>
+__device__ __forceinline__ void attend_tile(const Pack16 (&qreg)[QB][D / 32], const Pack16 (&a)[2][D / 32],
+                                            Pack16 (&vt)[D / 16], int key0, int kv_len,
+                                            const int (&row_pos)[QB], int window, float scale_log2,
+                                            f32x4_t (&acc)[QB][D / 16], float (&m_run)[QB], float (&l_run)[QB]) {
+  const int lane = threadIdx.x & 63;
+  const int grp = lane >> 4;
   f32x4_t s[QB][2];
 #pragma unroll
   for (int kb = 0; kb < 2; ++kb)
@@ -334,8 +338,8 @@ __device__ __forceinline__ void attend_tile(const Pack16 (&qreg)[QB][D / 32], co
       acc[qb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt[nb].v, p[qb].v, acc[qb][nb], 0, 0, 0);
 }
 
-// All tiles first, first + step, ... below last for one wavefront: the K operands
-// of the next tile are fetched while the current one is worked on.
+// All tiles first, first + step, ... below last for one wavefront: the value loads of a
+// tile and the key loads of the next one are issued before the tile's arithmetic.
 template <int D, int QB>
 __device__ __forceinline__ void attend_tiles(const Pack16 (&qreg)[QB][D / 32], const bf16_t* __restrict__ k_cache,
                                              const bf16_t* __restrict__ v_cache, int num_pages,
@@ -344,20 +348,18 @@ __device__ __forceinline__ void attend_tiles(const Pack16 (&qreg)[QB][D / 32], c
                                              float scale_log2, f32x4_t (&acc)[QB][D / 16], float (&m_run)[QB],
                                              float (&l_run)[QB]) {
   if (first >= last) return;
-  Pack16 a_cur[2][D / 32], a_nxt[2][D / 32];
+  Pack16 a_cur[2][D / 32], a_nxt[2][D / 32], vt[D / 16];
   TileAddr t_cur = tile_addr(k_cache, v_cache, num_pages, bt_row, Hkv, g_kv, page, D, first * FAST_TILE, kv_len);
   load_keys<D>(a_cur, t_cur);
   for (int t = first; t < last; t += step) {
-    TileAddr t_nxt;
+    load_values<D>(vt, t_cur, page);
     const bool more = t + step < last;
     if (more) {
-      t_nxt = tile_addr(k_cache, v_cache, num_pages, bt_row, Hkv, g_kv, page, D, (t + step) * FAST_TILE, kv_len);
-      load_keys<D>(a_nxt, t_nxt);
+      t_cur = tile_addr(k_cache, v_cache, num_pages, bt_row, Hkv, g_kv, page, D, (t + step) * FAST_TILE, kv_len);
+      load_keys<D>(a_nxt, t_cur);
     }
-    attend_tile<D, QB>(qreg, a_cur, t_cur, page, t * FAST_TILE, kv_len, row_pos, window, scale_log2, acc, m_run,
-                       l_run);
+    attend_tile<D, QB>(qreg, a_cur, vt, t * FAST_TILE, kv_len, row_pos, window, scale_log2, acc, m_run, l_run);
     if (more) {
-      t_cur = t_nxt;
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll

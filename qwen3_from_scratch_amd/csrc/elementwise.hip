@@ -15,7 +15,8 @@ __global__ void embed_rows_kernel(const int* __restrict__ ids, const T* __restri
   for (int j = threadIdx.x; j < H; j += blockDim.x) dst[j] = ok ? to_float(row[j]) : 0.f;
 }
 
-// out[t, j] = silu(gate[t, j]) * up[t, j], gate = gate_up[:, :I], up = gate_up[:, I:],
+// out[t, j] = silu(gate[t, j]) * up[t, j] for rows that interleave the two:
+// gate_up[t, 2j] = gate[t, j], gate_up[t, 2j + 1] = up[t, j].
 // silu(g) = g / (1 + exp(-g)), evaluated in float32 and rounded once.
 template <typename T>
 __global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int I) {
@@ -23,27 +24,28 @@ __global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out
   const int j = blockIdx.x * blockDim.x + threadIdx.x;
   if (j >= I) return;
   const T* row = gate_up + (size_t)t * 2 * I;
-  const float g = to_float(row[j]);
-  const float u = to_float(row[I + j]);
+  const float g = to_float(row[2 * j]);
+  const float u = to_float(row[2 * j + 1]);
   out[(size_t)t * I + j] = from_float<T>(g / (1.f + expf(-g)) * u);
 }
 
-// The same, eight elements per thread with 16-byte loads and stores; bfloat16, I a multiple of 8.
+// The same, eight outputs per thread with 16-byte loads and stores; bfloat16, I a multiple of 8.
 __global__ void swiglu_vec8_kernel(const bf16_t* __restrict__ gate_up, bf16_t* __restrict__ out, int I) {
   const int t = blockIdx.y;
   const int j = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
   if (j >= I) return;
-  const bf16_t* row = gate_up + (size_t)t * 2 * I;
+  const bf16_t* row = gate_up + (size_t)t * 2 * I + 2 * j;
   union {
     uint4 u;
     bf16_t e[8];
-  } g, u, o;
-  g.u = *reinterpret_cast<const uint4*>(row + j);
-  u.u = *reinterpret_cast<const uint4*>(row + I + j);
+  } a, b, o;
+  a.u = *reinterpret_cast<const uint4*>(row);
+  b.u = *reinterpret_cast<const uint4*>(row + 8);
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const float gv = bf16_to_float(g.e[i]);
-    o.e[i] = float_to_bf16(gv / (1.f + expf(-gv)) * bf16_to_float(u.e[i]));
+  for (int i = 0; i < 4; ++i) {
+    const float g0 = bf16_to_float(a.e[2 * i]), g1 = bf16_to_float(b.e[2 * i]);
+    o.e[i] = float_to_bf16(g0 / (1.f + expf(-g0)) * bf16_to_float(a.e[2 * i + 1]));
+    o.e[4 + i] = float_to_bf16(g1 / (1.f + expf(-g1)) * bf16_to_float(b.e[2 * i + 1]));
   }
   *reinterpret_cast<uint4*>(out + (size_t)t * I + j) = o.u;
 }

@@ -112,7 +112,10 @@ union Pack16 {
   bf16x8_t v;
 };
 
-template <int CB, typename OUT>
+// With SWIGLU the weight's rows interleave a gate and an up matrix (row 2i gate, row 2i + 1
+// up) and the kernel writes silu(gate) * up, out (M, N / 2): a lane's four consecutive
+// outputs are two (gate, up) pairs.
+template <int CB, typename OUT, bool SWIGLU>
 __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restrict__ x,
                                                            const bf16_t* __restrict__ w, OUT* __restrict__ out,
                                                            int M, int N, int K, int kw, int k_per_wave) {
@@ -169,6 +172,24 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[cb][j] += red[(((wave + s) * CB + cb) * 64 + lane) * 4 + j];
   }
+  if constexpr (SWIGLU) {
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) {
+      const int m = 16 * cb + col;
+      if (m >= M) continue;
+      const int n = n0 + 4 * grp;  // even; pairs (n, n + 1) and (n + 2, n + 3)
+      OUT* o = out + (size_t)m * (N / 2) + n / 2;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        if (n + 2 * j + 1 < N) {
+          // the separate kernel sees gate and up rounded to the activation dtype: do the same
+          const float g = to_float(from_float<OUT>(acc[cb][2 * j])), u = to_float(from_float<OUT>(acc[cb][2 * j + 1]));
+          o[j] = from_float<OUT>(g / (1.f + expf(-g)) * u);
+        }
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int cb = 0; cb < CB; ++cb) {
     const int m = 16 * cb + col;
@@ -195,7 +216,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
   }
 }
 
-template <int CB, typename OUT>
+template <int CB, typename OUT, bool SWIGLU = false>
 static int launch_skinny(const void* x, const void* w, void* out, int M, int N, int K, hipStream_t stream) {
   const int slabs = (N + 15) / 16;
   // enough wavefronts to keep every CU's memory pipeline full, each with at least 4 k-steps
@@ -210,7 +231,7 @@ static int launch_skinny(const void* x, const void* w, void* out, int M, int N, 
   k_per_wave = (k_per_wave + step - 1) / step * step;
   const int blocks = (slabs + sw - 1) / sw;
   const size_t smem = kw > 1 ? (size_t)sw * kw * CB * 64 * 4 * sizeof(float) : 0;
-  hipLaunchKernelGGL((gemm_skinny_kernel<CB, OUT>), dim3(blocks), dim3(64 * sw * kw), smem, stream, (const bf16_t*)x,
+  hipLaunchKernelGGL((gemm_skinny_kernel<CB, OUT, SWIGLU>), dim3(blocks), dim3(64 * sw * kw), smem, stream, (const bf16_t*)x,
                      (const bf16_t*)w, (OUT*)out, M, N, K, kw, k_per_wave);
   return q3_launch_status();
 }
@@ -239,4 +260,13 @@ extern "C" int q3_linear(const void* x, const void* weight, void* out, int M, in
   if (M <= 32) return Q3_SKINNY(2);
   return Q3_SKINNY(4);
 #undef Q3_SKINNY
+}
+
+// out (M, N / 2) = silu(gate) * up where x @ weight^T interleaves gate and up columns
+// (weight row 2i is gate's row i, row 2i + 1 up's). bfloat16, M <= 16, N even.
+extern "C" int q3_linear_swiglu(const void* x, const void* weight, void* out, int M, int N, int K, int dtype,
+                                hipStream_t stream) {
+  if (M <= 0 || N <= 0 || K <= 0 || N % 2) return Q3_ERR_BAD_ARGUMENT;
+  if (!q3_linear_is_skinny(M, N, K, dtype)) return Q3_ERR_UNSUPPORTED;
+  return launch_skinny<1, bf16_t, true>(x, weight, out, M, N, K, stream);
 }

@@ -27,6 +27,7 @@ __all__ = [
     "paged_attention",
     "swiglu",
     "linear",
+    "linear_swiglu",
     "sample",
 ]
 
@@ -79,7 +80,7 @@ def embed_rows(ids, table, out=None):
 
 
 def swiglu(gate_up, out=None):
-    """out = silu(gate) * up for gate_up = [gate | up] of shape (T, 2I)."""
+    """out[:, j] = silu(gate_up[:, 2j]) * gate_up[:, 2j + 1]: gate and up interleaved, (T, 2I) -> (T, I)."""
     _dev(gate_up, out)
     _need(gate_up.dim() == 2 and gate_up.shape[1] % 2 == 0 and gate_up.dtype in _DT,
           "gate_up must be (T, 2I) bfloat16 or float32")
@@ -291,6 +292,24 @@ def linear(x, weight, out_dtype=None, out=None):
         _check(library("gemm").q3_linear(
             _ptr(x), _ptr(weight), _ptr(out), M, N, K, _DT[x.dtype], _DT[out_dtype], _stream()), "linear")
     return out
+
+
+def linear_swiglu(x, weight):
+    """swiglu(x @ weight^T) for a weight whose rows interleave gate and up (row 2i gate's, row
+    2i + 1 up's): (M, K) x (2I, K) -> (M, I). With few bfloat16 rows the activation is the
+    product kernel's epilogue; otherwise it is the product followed by `swiglu`."""
+    _dev(x, weight)
+    _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1] and weight.shape[0] % 2 == 0,
+          "x (M, K) and weight (2I, K)")
+    _need(x.dtype in _DT and weight.dtype == x.dtype, "x and weight must share bfloat16 or float32")
+    M, K = x.shape
+    N = weight.shape[0]
+    if M and library("gemm").q3_linear_is_skinny(M, N, K, _DT[x.dtype]):
+        out = torch.empty((M, N // 2), dtype=x.dtype, device=x.device)
+        _check(library("gemm").q3_linear_swiglu(_ptr(x), _ptr(weight), _ptr(out), M, N, K, _DT[x.dtype], _stream()),
+               "linear_swiglu")
+        return out
+    return swiglu(linear(x, weight))
 
 
 def sample(logits, temperature, top_k, seed, counter, out=None):

@@ -11,7 +11,10 @@ from .base import Part
 class SwiGLU(Part):
     """down(silu(gate(x)) * up(x)), no biases
     (src/qwen3_from_scratch/models/feedback.py:28-34). gate and up are kept as
-    one matrix [gate | up] so that one product feeds the activation kernel."""
+    one matrix with their rows interleaved (row 2i gate's, row 2i + 1 up's), so
+    that one product feeds the activation, which for few rows is the product
+    kernel's epilogue (the reference's fused variant concatenates them,
+    feedback.py:52-54)."""
 
     graph_safe = True
 
@@ -34,10 +37,9 @@ class SwiGLU(Part):
         act = self.precision.act
         I, H = self.intermediate_size, self.hidden_size
         self.gate_up = torch.empty((2 * I, H), dtype=act, device=self.device)
-        self.gate_up[:I].copy_(fetch(self._name("gate_proj.weight"), act, keep=False))
-        self.gate_up[I:].copy_(fetch(self._name("up_proj.weight"), act, keep=False))
+        self.gate_up[0::2].copy_(fetch(self._name("gate_proj.weight"), act, keep=False))
+        self.gate_up[1::2].copy_(fetch(self._name("up_proj.weight"), act, keep=False))
         self.down = fetch(self._name("down_proj.weight"), act)
 
     def forward(self, x, batch=None):
-        gate_up = ops.linear(x, self.gate_up)
-        return ops.linear(ops.swiglu(gate_up), self.down)
+        return ops.linear(ops.linear_swiglu(x, self.gate_up), self.down)

@@ -302,6 +302,22 @@ def test_linear_few_rows_streams_weights(M, N, K):
         assert torch.equal(alone[0], got[0])
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,I,K", [(1, 12288, 4096), (8, 100, 72), (16, 333, 200), (40, 64, 64)])
+def test_linear_swiglu(dtype, M, I, K):
+    ops = _ops()
+    x = _rand((M, K), dtype, 21)
+    w = _rand((2 * I, K), dtype, 22, scale=0.1)
+    got = ops.linear_swiglu(x, w)
+    assert got.shape == (M, I) and got.dtype == dtype
+    want = torch_ops.swiglu((x.double() @ w.double().T).float())
+    tol = dict(rtol=1e-4, atol=1e-4) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(got.float(), want, **tol)
+    if dtype == torch.bfloat16:
+        # fused or not, the result is the same to the bit
+        assert torch.equal(got, ops.swiglu(ops.linear(x, w)))
+
+
 def test_linear_float32_is_true_float32():
     """Inputs whose products need all 24 bits: a matrix mode of reduced precision
     (bf16 or tf32-like splitting) would be off by far more than float32 rounding."""

@@ -21,9 +21,8 @@ def embed_rows(ids, table, out=None):
 
 
 def swiglu(gate_up, out=None):
-    I = gate_up.shape[1] // 2
-    g = gate_up[:, :I].float()
-    u = gate_up[:, I:].float()
+    g = gate_up[:, 0::2].float()          # gate and up interleaved
+    u = gate_up[:, 1::2].float()
     res = (g / (1.0 + torch.exp(-g)) * u).to(gate_up.dtype)
     if out is not None:
         out.copy_(res)
@@ -133,6 +132,10 @@ def linear(x, weight, out_dtype=None, out=None):
     return res
 
 
+def linear_swiglu(x, weight):
+    return swiglu(linear(x, weight))
+
+
 def _uniform(seed, counter, n, device):
     # any fixed stream will do for the stand-in; the kernel's generator is tested on the GPU
     g = torch.Generator(device="cpu")
@@ -163,4 +166,4 @@ def sample(logits, temperature, top_k, seed, counter, out=None):
 
 
 ALL = ("embed_rows", "swiglu", "rmsnorm", "rope_table", "qk_norm_rope_store",
-       "paged_attention", "linear", "sample")
+       "paged_attention", "linear", "linear_swiglu", "sample")

@@ -463,6 +463,9 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
 }
 
 // Merge the splits' partial results: grid (Hkv, B), 256 threads; splits <= 64.
+// (A kernel of its own rather than the work of the decode kernel's last-arriving
+// block: the device-scope fences that needs write back and invalidate each XCD's
+// L2, which measured three times slower than this second launch.)
 // The weights of the splits are formed once per row in shared memory, then
 // every thread sums a few output elements over the splits with loads that are
 // contiguous across the block.

@@ -8,14 +8,16 @@ from .batch import StepEntry, pack_step, packed_size
 
 class _DecodeGraph:
     """A captured HIP graph of the model's forward pass for `B` requests with
-    one token each. The batch description lives in fixed device memory that is
-    refilled before every replay; sizes that the kernels' launches depend on
-    (the longest sequence, hence how keys are split over workgroups) are fixed
-    at the cache's capacity."""
+    one token each, none longer than `max_kv_len`. The batch description lives
+    in fixed device memory that is refilled before every replay; what the
+    kernels' launches depend on (the longest sequence, hence how keys are
+    split over workgroups) is fixed at `max_kv_len`, a power of two, so a
+    batch gets a new graph each time its longest request doubles."""
 
-    def __init__(self, runner, B):
+    def __init__(self, runner, B, max_kv_len):
         m = runner.manager
         self.B = B
+        self.max_kv_len = max_kv_len
         self.widths = [-(-runner.max_request_tokens // m.page_size)] * len(m.groups)
         n = packed_size(B, B, B, self.widths)
         self.host = torch.empty(n, dtype=torch.int32).pin_memory()
@@ -29,7 +31,7 @@ class _DecodeGraph:
         batch, block_tables = pack_step(entries, lengths, slots, tables, runner.device,
                                         fixed_widths=self.widths, buffers=(self.host, self.dev), all_rows=True)
         self.copied.record()
-        batch.max_kv_len = runner.max_request_tokens
+        batch.max_kv_len = self.max_kv_len
         runner.storage.bind(block_tables)
         if self.graph is None:
             # once eagerly on a side stream (libraries build and tune at first use), then capture
@@ -74,6 +76,7 @@ class ModelRunner:
             self.max_request_tokens = min(self.max_request_tokens, self.max_positions)
         self.use_graphs = bool(use_graphs) and self.device.type == "cuda" and model.graph_safe()
         self._graphs = {}
+        self.max_graphs = 32
 
     def step(self, entries):
         """entries: list of StepEntry. Returns logits (R, V) float32 on the
@@ -123,9 +126,17 @@ class ModelRunner:
 
     def _step_graph(self, entries, lengths, slots, tables):
         B = len(entries)
-        graph = self._graphs.get(B)
+        longest = max(lengths) + 1
+        bucket = 256
+        while bucket < longest:
+            bucket *= 2
+        bucket = min(bucket, self.max_request_tokens)
+        graph = self._graphs.pop((B, bucket), None)
         if graph is None:
-            graph = self._graphs[B] = _DecodeGraph(self, B)
+            if len(self._graphs) >= self.max_graphs:       # drop the one used longest ago
+                self._graphs.pop(next(iter(self._graphs)))
+            graph = _DecodeGraph(self, B, bucket)
+        self._graphs[(B, bucket)] = graph                   # most recently used last
         logits = graph.run(self, entries, lengths, slots, tables)
         wanted = [i for i, e in enumerate(entries) for _ in e.want]
         if wanted == list(range(B)):

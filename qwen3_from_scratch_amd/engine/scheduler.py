@@ -99,6 +99,15 @@ class Scheduler:
     def has_work(self):
         return bool(self.waiting or self.running)
 
+    def abort(self, request):
+        """Take a request out, wherever it is; what it holds is given back."""
+        if request in self.waiting:
+            self.waiting.remove(request)
+        if request in self.running:
+            self.running.remove(request)
+        self.release(request.request_id)
+        request.status = RequestStatus.FINISHED
+
     # ---- one step's plan ----
     def schedule(self):
         while True:

@@ -155,6 +155,10 @@ class SyncEngine:
         self.scheduler.add(request)
         return request
 
+    def abort(self, request):
+        """Stop a request before it has finished; its pages and slot are given back."""
+        self.scheduler.abort(request)
+
     # ---- the loop body ----
     def step(self):
         """Schedule, run the step function, sample, book-keep. Returns the plan

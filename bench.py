@@ -57,6 +57,8 @@ def main():
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration (0 = all)")
     ap.add_argument("--dtype", default="bfloat16")
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 points")
+    ap.add_argument("--skip-prefill", action="store_true",
+                    help="skip the prefill measurement (for profiles of decoding alone; the line then has no value for it)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this engine runs on one GPU; --gpus %d is not supported" % args.gpus)
@@ -91,7 +93,8 @@ def main():
 
     # ---- prefill: one prompt of 2,048 tokens in one step ----
     engine = engine_for(1)
-    for _ in range(2):                               # warm-up, then the timed one
+    prefill_s = None
+    for _ in range(0 if args.skip_prefill else 2):   # warm-up, then the timed one
         req = engine.add_request(prompts(1)[0], engine.default_params(1, temperature=0.0, ignore_eos=True))
         sync()
         t0 = time.perf_counter()
@@ -101,8 +104,10 @@ def main():
         assert len(plan) == 1 and plan[0].num_tokens == PROMPT
         while engine.scheduler.has_work():
             engine.step()
-    prefill = {"value": round(PROMPT / prefill_s, 1), "tokens": PROMPT, "ms": round(prefill_s * 1e3, 3),
-               "frac": round(prefill_flops(config, PROMPT) / prefill_s / PEAK_FLOPS[args.dtype], 4)}
+    prefill = None
+    if prefill_s is not None:
+        prefill = {"value": round(PROMPT / prefill_s, 1), "tokens": PROMPT, "ms": round(prefill_s * 1e3, 3),
+                   "frac": round(prefill_flops(config, PROMPT) / prefill_s / PEAK_FLOPS[args.dtype], 4)}
     del engine
 
     # ---- decode ----

@@ -90,19 +90,24 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
 
 
 // ---------------------------------------------------------------------------
-// bfloat16 with few rows (M <= 16 as dispatched; the kernel takes up to 64): a
-// weight-streaming kernel. Every weight is
+// bfloat16 with at most 16 rows: a weight-streaming kernel. Every weight is
 // read once from HBM and that read is the cost; the matrix cores do the sums
-// (v_mfma_f32_16x16x32_bf16) with 16 weight rows as the A operand and up to 16
-// rows of x as the B operand, so out^T tiles come out with x's row in the
-// lane's low bits: lane (m = lane % 16, g = lane / 16) ends with
-// out[m][n0 + 4g .. 4g+3], four consecutive outputs of one row.
+// (v_mfma_f32_16x16x32_bf16) with 16 weight rows as the A operand and the rows
+// of x as the B operand, so out^T tiles come out with x's row in the lane's low
+// bits: lane (m = lane % 16, g = lane / 16) ends with out[m][n0 + 4g .. 4g+3],
+// four consecutive outputs of one row.
 //
 // A wavefront owns a slab of 16 weight rows and a share of K; the `kw`
 // wavefronts that share a slab are summed through shared memory in a fixed
 // order, so the result does not depend on timing. Loads are 16 bytes per lane;
 // a lane's eight k-values are the same in A and B, which is all the product needs.
 // K must be a multiple of 8; rows of the weight beyond N and k beyond K read as zero.
+// (More rows of x per wavefront were tried, up to 64: the x operand loads then
+// compete with the weight loads and the vendor library's kernels are faster.)
+//
+// With SWIGLU the weight's rows interleave a gate and an up matrix (row 2i gate, row 2i + 1
+// up) and the kernel writes silu(gate) * up, out (M, N / 2): a lane's four consecutive
+// outputs are two (gate, up) pairs.
 // ---------------------------------------------------------------------------
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
@@ -112,14 +117,13 @@ union Pack16 {
   bf16x8_t v;
 };
 
-// With SWIGLU the weight's rows interleave a gate and an up matrix (row 2i gate, row 2i + 1
-// up) and the kernel writes silu(gate) * up, out (M, N / 2): a lane's four consecutive
-// outputs are two (gate, up) pairs.
-template <int CB, typename OUT, bool SWIGLU>
+#define SKINNY_U 8  // k-steps of 32 per loop iteration: eight 16-byte loads of each operand in flight
+
+template <typename OUT, bool SWIGLU>
 __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restrict__ x,
                                                            const bf16_t* __restrict__ w, OUT* __restrict__ out,
                                                            int M, int N, int K, int kw, int k_per_wave) {
-  extern __shared__ float red[];  // [waves][CB][64][4]
+  extern __shared__ float red[];  // [waves][64][4]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, grp = lane >> 4;
   const int sw = (blockDim.x >> 6) / kw;
@@ -128,111 +132,83 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
   const int n0 = slab * 16;
   const int k_begin = ksplit * k_per_wave;
   const int k_end = min(K, k_begin + k_per_wave);
-  f32x4_t acc[CB];
-#pragma unroll
-  for (int cb = 0; cb < CB; ++cb) acc[cb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 
   const bool row_ok = n0 + col < N;
+  const bool x_ok = col < M;
   const bf16_t* wp = w + (size_t)(row_ok ? n0 + col : 0) * K + 8 * grp;
-  const bf16_t* xp[CB];
-  bool x_ok[CB];
+  const bf16_t* xp = x + (size_t)(x_ok ? col : 0) * K + 8 * grp;
+  for (int k = k_begin; k < k_end; k += 32 * SKINNY_U) {
+    Pack16 a[SKINNY_U], b[SKINNY_U];
 #pragma unroll
-  for (int cb = 0; cb < CB; ++cb) {
-    x_ok[cb] = 16 * cb + col < M;
-    xp[cb] = x + (size_t)(x_ok[cb] ? 16 * cb + col : 0) * K + 8 * grp;
-  }
-  constexpr int U = CB == 1 ? 8 : (CB == 2 ? 4 : 2);
-  for (int k = k_begin; k < k_end; k += 32 * U) {
-    Pack16 a[U], b[CB][U];
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
+    for (int u = 0; u < SKINNY_U; ++u) {
       const int kk = k + 32 * u;
       const bool k_ok = kk + 8 * grp + 8 <= k_end;
       a[u].u = (row_ok && k_ok) ? *reinterpret_cast<const uint4*>(wp + kk) : make_uint4(0, 0, 0, 0);
-#pragma unroll
-      for (int cb = 0; cb < CB; ++cb)
-        b[cb][u].u = (x_ok[cb] && k_ok) ? *reinterpret_cast<const uint4*>(xp[cb] + kk) : make_uint4(0, 0, 0, 0);
+      b[u].u = (x_ok && k_ok) ? *reinterpret_cast<const uint4*>(xp + kk) : make_uint4(0, 0, 0, 0);
     }
 #pragma unroll
-    for (int u = 0; u < U; ++u)
-#pragma unroll
-      for (int cb = 0; cb < CB; ++cb)
-        acc[cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u].v, b[cb][u].v, acc[cb], 0, 0, 0);
+    for (int u = 0; u < SKINNY_U; ++u) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u].v, b[u].v, acc, 0, 0, 0);
   }
   if (kw > 1) {
 #pragma unroll
-    for (int cb = 0; cb < CB; ++cb)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) red[((wave * CB + cb) * 64 + lane) * 4 + j] = acc[cb][j];
+    for (int j = 0; j < 4; ++j) red[(wave * 64 + lane) * 4 + j] = acc[j];
     __syncthreads();
     if (ksplit != 0) return;
+    for (int s = 1; s < kw; ++s)
 #pragma unroll
-    for (int cb = 0; cb < CB; ++cb)
-      for (int s = 1; s < kw; ++s)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[cb][j] += red[(((wave + s) * CB + cb) * 64 + lane) * 4 + j];
+      for (int j = 0; j < 4; ++j) acc[j] += red[((wave + s) * 64 + lane) * 4 + j];
   }
+  if (col >= M) return;
+  const int n = n0 + 4 * grp;
   if constexpr (SWIGLU) {
+    OUT* o = out + (size_t)col * (N / 2) + n / 2;  // n is even: pairs (n, n + 1) and (n + 2, n + 3)
 #pragma unroll
-    for (int cb = 0; cb < CB; ++cb) {
-      const int m = 16 * cb + col;
-      if (m >= M) continue;
-      const int n = n0 + 4 * grp;  // even; pairs (n, n + 1) and (n + 2, n + 3)
-      OUT* o = out + (size_t)m * (N / 2) + n / 2;
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        if (n + 2 * j + 1 < N) {
-          // the separate kernel sees gate and up rounded to the activation dtype: do the same
-          const float g = to_float(from_float<OUT>(acc[cb][2 * j])), u = to_float(from_float<OUT>(acc[cb][2 * j + 1]));
-          o[j] = from_float<OUT>(g / (1.f + expf(-g)) * u);
-        }
+    for (int j = 0; j < 2; ++j) {
+      if (n + 2 * j + 1 < N) {
+        // the separate kernel sees gate and up rounded to the activation dtype: do the same
+        const float g = to_float(from_float<OUT>(acc[2 * j])), u = to_float(from_float<OUT>(acc[2 * j + 1]));
+        o[j] = from_float<OUT>(g / (1.f + expf(-g)) * u);
       }
     }
     return;
   }
-#pragma unroll
-  for (int cb = 0; cb < CB; ++cb) {
-    const int m = 16 * cb + col;
-    if (m >= M) continue;
-    const int n = n0 + 4 * grp;
-    OUT* o = out + (size_t)m * N + n;
-    if (n + 3 < N && (N % 4) == 0) {
-      if constexpr (sizeof(OUT) == 4) {
-        *reinterpret_cast<float4*>(o) = make_float4(acc[cb][0], acc[cb][1], acc[cb][2], acc[cb][3]);
-      } else {
-        union {
-          uint2 u;
-          bf16_t e[4];
-        } pk;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) pk.e[j] = float_to_bf16(acc[cb][j]);
-        *reinterpret_cast<uint2*>(o) = pk.u;
-      }
+  OUT* o = out + (size_t)col * N + n;
+  if (n + 3 < N && (N % 4) == 0) {
+    if constexpr (sizeof(OUT) == 4) {
+      *reinterpret_cast<float4*>(o) = make_float4(acc[0], acc[1], acc[2], acc[3]);
     } else {
+      union {
+        uint2 u;
+        bf16_t e[4];
+      } pk;
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-        if (n + j < N) o[j] = from_float<OUT>(acc[cb][j]);
+      for (int j = 0; j < 4; ++j) pk.e[j] = float_to_bf16(acc[j]);
+      *reinterpret_cast<uint2*>(o) = pk.u;
     }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (n + j < N) o[j] = from_float<OUT>(acc[j]);
   }
 }
 
-template <int CB, typename OUT, bool SWIGLU = false>
+template <typename OUT, bool SWIGLU>
 static int launch_skinny(const void* x, const void* w, void* out, int M, int N, int K, hipStream_t stream) {
   const int slabs = (N + 15) / 16;
-  // enough wavefronts to keep every CU's memory pipeline full, each with at least 4 k-steps
+  // enough wavefronts to keep every CU's memory pipeline full (about 4096), each with at
+  // least four k-steps
   int kw = 1;
-  while (kw < 16 && slabs * kw < 2048 && K / (kw * 2) >= 128 && kw * 2 * CB <= 32) kw *= 2;
+  while (kw < 16 && slabs * kw < 4096 && K / (kw * 2) >= 128) kw *= 2;
   int sw = 1;
   while (sw * kw < 4 && sw * 2 <= slabs) sw *= 2;
-  // k_per_wave: a multiple of the unrolled step, covering K
-  constexpr int U = CB == 1 ? 8 : (CB == 2 ? 4 : 2);
-  const int step = 32 * U;
+  const int step = 32 * SKINNY_U;
   int k_per_wave = (K + kw - 1) / kw;
   k_per_wave = (k_per_wave + step - 1) / step * step;
   const int blocks = (slabs + sw - 1) / sw;
-  const size_t smem = kw > 1 ? (size_t)sw * kw * CB * 64 * 4 * sizeof(float) : 0;
-  hipLaunchKernelGGL((gemm_skinny_kernel<CB, OUT, SWIGLU>), dim3(blocks), dim3(64 * sw * kw), smem, stream, (const bf16_t*)x,
-                     (const bf16_t*)w, (OUT*)out, M, N, K, kw, k_per_wave);
+  const size_t smem = kw > 1 ? (size_t)sw * kw * 64 * 4 * sizeof(float) : 0;
+  hipLaunchKernelGGL((gemm_skinny_kernel<OUT, SWIGLU>), dim3(blocks), dim3(64 * sw * kw), smem, stream,
+                     (const bf16_t*)x, (const bf16_t*)w, (OUT*)out, M, N, K, kw, k_per_wave);
   return q3_launch_status();
 }
 
@@ -253,13 +229,8 @@ extern "C" int q3_linear(const void* x, const void* weight, void* out, int M, in
     return q3_launch_status();
   }
   if (!q3_linear_is_skinny(M, N, K, in_dtype)) return Q3_ERR_UNSUPPORTED;
-#define Q3_SKINNY(CB)                                                                      \
-  (out_dtype == Q3_F32 ? launch_skinny<CB, float>(x, weight, out, M, N, K, stream)         \
-                       : launch_skinny<CB, bf16_t>(x, weight, out, M, N, K, stream))
-  if (M <= 16) return Q3_SKINNY(1);
-  if (M <= 32) return Q3_SKINNY(2);
-  return Q3_SKINNY(4);
-#undef Q3_SKINNY
+  return out_dtype == Q3_F32 ? launch_skinny<float, false>(x, weight, out, M, N, K, stream)
+                             : launch_skinny<bf16_t, false>(x, weight, out, M, N, K, stream);
 }
 
 // out (M, N / 2) = silu(gate) * up where x @ weight^T interleaves gate and up columns
@@ -268,5 +239,5 @@ extern "C" int q3_linear_swiglu(const void* x, const void* weight, void* out, in
                                 hipStream_t stream) {
   if (M <= 0 || N <= 0 || K <= 0 || N % 2) return Q3_ERR_BAD_ARGUMENT;
   if (!q3_linear_is_skinny(M, N, K, dtype)) return Q3_ERR_UNSUPPORTED;
-  return launch_skinny<1, bf16_t, true>(x, weight, out, M, N, K, stream);
+  return launch_skinny<bf16_t, true>(x, weight, out, M, N, K, stream);
 }

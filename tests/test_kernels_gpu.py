@@ -175,7 +175,8 @@ def _paged_case(dtype, B, Hq, Hkv, D, page, q_lens, kv_lens, seed, spread=True):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("Hq,Hkv,D,page", [(4, 2, 16, 16), (8, 2, 32, 8), (6, 3, 48, 16), (5, 5, 80, 4),
-                                           (32, 8, 128, 16), (3, 1, 256, 32), (16, 2, 64, 16)])
+                                           (32, 8, 128, 16), (3, 1, 256, 32), (16, 2, 64, 16),
+                                           (40, 8, 128, 16), (64, 8, 128, 16), (14, 2, 64, 64), (9, 3, 128, 32)])
 @pytest.mark.parametrize("window", [0, 19])
 def test_paged_attention_mixed_batch(dtype, Hq, Hkv, D, page, window):
     ops = _ops()

@@ -119,7 +119,13 @@ union Pack16 {
 
 #define SKINNY_U 8  // k-steps of 32 per loop iteration: eight 16-byte loads of each operand in flight
 
-template <typename OUT, bool SWIGLU>
+//
+// With TILED the weight is a copy laid out for this kernel, w[slab][k / 32][lane][8] with
+// lane = (n % 16) + 16 * ((k % 32) / 8): the A operand of one matrix instruction is then one
+// contiguous kilobyte instead of sixteen 64-byte pieces of sixteen rows, which the memory
+// system serves about a fifth faster. Rows are padded with zeros to a multiple of 16, and K
+// is a multiple of 32.
+template <typename OUT, bool SWIGLU, bool TILED>
 __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restrict__ x,
                                                            const bf16_t* __restrict__ w, OUT* __restrict__ out,
                                                            int M, int N, int K, int kw, int k_per_wave) {
@@ -134,9 +140,10 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
   const int k_end = min(K, k_begin + k_per_wave);
   f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 
-  const bool row_ok = n0 + col < N;
+  const bool row_ok = TILED ? n0 < N : n0 + col < N;
   const bool x_ok = col < M;
-  const bf16_t* wp = w + (size_t)(row_ok ? n0 + col : 0) * K + 8 * grp;
+  const bf16_t* wp = TILED ? w + (size_t)(row_ok ? slab : 0) * (K / 32) * 512 + lane * 8
+                           : w + (size_t)(row_ok ? n0 + col : 0) * K + 8 * grp;
   const bf16_t* xp = x + (size_t)(x_ok ? col : 0) * K + 8 * grp;
   for (int k = k_begin; k < k_end; k += 32 * SKINNY_U) {
     Pack16 a[SKINNY_U], b[SKINNY_U];
@@ -144,7 +151,10 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
     for (int u = 0; u < SKINNY_U; ++u) {
       const int kk = k + 32 * u;
       const bool k_ok = kk + 8 * grp + 8 <= k_end;
-      a[u].u = (row_ok && k_ok) ? *reinterpret_cast<const uint4*>(wp + kk) : make_uint4(0, 0, 0, 0);
+      if (TILED)
+        a[u].u = (row_ok && k_ok) ? *reinterpret_cast<const uint4*>(wp + (size_t)(kk / 32) * 512) : make_uint4(0, 0, 0, 0);
+      else
+        a[u].u = (row_ok && k_ok) ? *reinterpret_cast<const uint4*>(wp + kk) : make_uint4(0, 0, 0, 0);
       b[u].u = (x_ok && k_ok) ? *reinterpret_cast<const uint4*>(xp + kk) : make_uint4(0, 0, 0, 0);
     }
 #pragma unroll
@@ -193,7 +203,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
   }
 }
 
-template <typename OUT, bool SWIGLU>
+template <typename OUT, bool SWIGLU, bool TILED = false>
 static int launch_skinny(const void* x, const void* w, void* out, int M, int N, int K, hipStream_t stream) {
   const int slabs = (N + 15) / 16;
   // enough wavefronts to keep every CU's memory pipeline full (about 4096), each with at
@@ -207,7 +217,7 @@ static int launch_skinny(const void* x, const void* w, void* out, int M, int N, 
   k_per_wave = (k_per_wave + step - 1) / step * step;
   const int blocks = (slabs + sw - 1) / sw;
   const size_t smem = kw > 1 ? (size_t)sw * kw * 64 * 4 * sizeof(float) : 0;
-  hipLaunchKernelGGL((gemm_skinny_kernel<OUT, SWIGLU>), dim3(blocks), dim3(64 * sw * kw), smem, stream,
+  hipLaunchKernelGGL((gemm_skinny_kernel<OUT, SWIGLU, TILED>), dim3(blocks), dim3(64 * sw * kw), smem, stream,
                      (const bf16_t*)x, (const bf16_t*)w, (OUT*)out, M, N, K, kw, k_per_wave);
   return q3_launch_status();
 }
@@ -240,4 +250,18 @@ extern "C" int q3_linear_swiglu(const void* x, const void* weight, void* out, in
   if (M <= 0 || N <= 0 || K <= 0 || N % 2) return Q3_ERR_BAD_ARGUMENT;
   if (!q3_linear_is_skinny(M, N, K, dtype)) return Q3_ERR_UNSUPPORTED;
   return launch_skinny<bf16_t, true>(x, weight, out, M, N, K, stream);
+}
+
+// The same products from the tile-ordered copy of the weight (see gemm_skinny_kernel):
+// x (M, K) bfloat16, M <= 16, K a multiple of 32; `swiglu` selects the activation epilogue
+// (output (M, N / 2) bfloat16), otherwise output (M, N) in `out_dtype`.
+extern "C" int q3_linear_tiled(const void* x, const void* weight_tiled, void* out, int M, int N, int K,
+                               int out_dtype, int swiglu, hipStream_t stream) {
+  if (M <= 0 || M > 16 || N <= 0 || K <= 0 || K % 32) return Q3_ERR_BAD_ARGUMENT;
+  if (swiglu) {
+    if (N % 2 || out_dtype != Q3_BF16) return Q3_ERR_BAD_ARGUMENT;
+    return launch_skinny<bf16_t, true, true>(x, weight_tiled, out, M, N, K, stream);
+  }
+  return out_dtype == Q3_F32 ? launch_skinny<float, false, true>(x, weight_tiled, out, M, N, K, stream)
+                             : launch_skinny<bf16_t, false, true>(x, weight_tiled, out, M, N, K, stream);
 }

@@ -28,6 +28,7 @@ __all__ = [
     "swiglu",
     "linear",
     "linear_swiglu",
+    "tile_weight",
     "sample",
 ]
 
@@ -262,8 +263,34 @@ def paged_attention(q, num_q_heads, k_cache, v_cache, block_table, cu_seqlens_q,
     return out
 
 
-def linear(x, weight, out_dtype=None, out=None):
+def tile_weight(weight):
+    """A copy of a bfloat16 matrix (N, K) in the order the few-row product kernel reads it:
+    [N / 16 slabs][K / 32 steps][64 lanes][8], lane = (n % 16) + 16 * ((k % 32) // 8), rows
+    padded with zeros to a multiple of 16. None if the matrix is not bfloat16 or K is not a
+    multiple of 32 (the row-major kernel then serves it)."""
+    if weight.dtype != torch.bfloat16 or weight.dim() != 2 or weight.shape[1] % 32:
+        return None
+    N, K = weight.shape
+    N16 = -(-N // 16) * 16
+    if N16 != N:
+        weight = torch.cat((weight, weight.new_zeros((N16 - N, K))), dim=0)
+    tiles = weight.view(N16 // 16, 16, K // 32, 4, 8).permute(0, 2, 3, 1, 4)   # slab, step, group, row, 8
+    return tiles.contiguous().view(-1)
+
+
+def _tiled_ok(tiled, weight, M):
+    if tiled is None or not 1 <= M <= 16:
+        return False
+    N, K = weight.shape
+    _need(tiled.is_cuda and tiled.dtype == torch.bfloat16 and tiled.is_contiguous()
+          and tiled.numel() == (-(-N // 16) * 16) * K and K % 32 == 0,
+          "the tiled copy does not belong to this weight")
+    return True
+
+
+def linear(x, weight, out_dtype=None, out=None, tiled=None):
     """out = x @ weight^T with float32 accumulation. x (M, K), weight (N, K).
+    `tiled` is `tile_weight(weight)`, if the caller keeps one: few rows are then served from it.
 
     float32 operands take a float32 kernel with no reduced-precision mode;
     bfloat16 operands with at most 16 rows take a weight-streaming matrix-core
@@ -280,7 +307,10 @@ def linear(x, weight, out_dtype=None, out=None):
     if out is None:
         out = torch.empty((M, N), dtype=out_dtype, device=x.device)
     _need(out.shape == (M, N) and out.dtype == out_dtype, "out must be (M, N) of out_dtype")
-    if M and x.dtype == torch.bfloat16 and not library("gemm").q3_linear_is_skinny(M, N, K, 1):
+    if M and x.dtype == torch.bfloat16 and _tiled_ok(tiled, weight, M):
+        _check(library("gemm").q3_linear_tiled(
+            _ptr(x), _ptr(tiled), _ptr(out), M, N, K, _DT[out_dtype], 0, _stream()), "linear")
+    elif M and x.dtype == torch.bfloat16 and not library("gemm").q3_linear_is_skinny(M, N, K, 1):
         # bfloat16 products with many rows go to the vendor library (hipBLASLt through
         # torch), as the reference's engine uses its vendor library for them; accumulation
         # is float32. Few rows take the weight-streaming kernel below.
@@ -294,7 +324,7 @@ def linear(x, weight, out_dtype=None, out=None):
     return out
 
 
-def linear_swiglu(x, weight):
+def linear_swiglu(x, weight, tiled=None):
     """swiglu(x @ weight^T) for a weight whose rows interleave gate and up (row 2i gate's, row
     2i + 1 up's): (M, K) x (2I, K) -> (M, I). With few bfloat16 rows the activation is the
     product kernel's epilogue; otherwise it is the product followed by `swiglu`."""
@@ -304,12 +334,17 @@ def linear_swiglu(x, weight):
     _need(x.dtype in _DT and weight.dtype == x.dtype, "x and weight must share bfloat16 or float32")
     M, K = x.shape
     N = weight.shape[0]
+    if M and x.dtype == torch.bfloat16 and _tiled_ok(tiled, weight, M):
+        out = torch.empty((M, N // 2), dtype=x.dtype, device=x.device)
+        _check(library("gemm").q3_linear_tiled(_ptr(x), _ptr(tiled), _ptr(out), M, N, K, 1, 1, _stream()),
+               "linear_swiglu")
+        return out
     if M and library("gemm").q3_linear_is_skinny(M, N, K, _DT[x.dtype]):
         out = torch.empty((M, N // 2), dtype=x.dtype, device=x.device)
         _check(library("gemm").q3_linear_swiglu(_ptr(x), _ptr(weight), _ptr(out), M, N, K, _DT[x.dtype], _stream()),
                "linear_swiglu")
         return out
-    return swiglu(linear(x, weight))
+    return swiglu(linear(x, weight, tiled=tiled))
 
 
 def sample(logits, temperature, top_k, seed, counter, out=None):

@@ -5,6 +5,7 @@ import torch
 from .. import ops
 from ..config.registry import register_part
 from .base import CacheNeed, Part
+from .linear import LinearWeight
 
 
 @register_part("mixer", "attention")
@@ -63,18 +64,19 @@ class PagedAttention(Part):
     def load(self, fetch):
         act = self.precision.act
         Hq, Hkv, D = self.num_heads, self.num_kv_heads, self.head_dim
-        self.qkv = torch.empty(((Hq + 2 * Hkv) * D, self.hidden_size), dtype=act, device=self.device)
-        self.qkv[: Hq * D].copy_(fetch(self._name("q_proj.weight"), act, keep=False))
-        self.qkv[Hq * D: (Hq + Hkv) * D].copy_(fetch(self._name("k_proj.weight"), act, keep=False))
-        self.qkv[(Hq + Hkv) * D:].copy_(fetch(self._name("v_proj.weight"), act, keep=False))
-        self.out = fetch(self._name("o_proj.weight"), act)
+        qkv = torch.empty(((Hq + 2 * Hkv) * D, self.hidden_size), dtype=act, device=self.device)
+        qkv[: Hq * D].copy_(fetch(self._name("q_proj.weight"), act, keep=False))
+        qkv[Hq * D: (Hq + Hkv) * D].copy_(fetch(self._name("k_proj.weight"), act, keep=False))
+        qkv[(Hq + Hkv) * D:].copy_(fetch(self._name("v_proj.weight"), act, keep=False))
+        self.qkv = LinearWeight(qkv, self.precision)
+        self.out = LinearWeight(fetch(self._name("o_proj.weight"), act), self.precision)
         if self.qk_norm:
             self.q_weight = fetch(self._name("q_norm.weight"))
             self.k_weight = fetch(self._name("k_norm.weight"))
 
     def forward(self, x, batch, cache):
         Hq, Hkv, D = self.num_heads, self.num_kv_heads, self.head_dim
-        qkv = ops.linear(x, self.qkv)
+        qkv = self.qkv.forward(x)
         table = self.position.rotation_table() if self.position is not None else None
         ops.qk_norm_rope_store(
             qkv, Hq, Hkv, D, batch.positions, batch.seq_index,
@@ -90,4 +92,4 @@ class PagedAttention(Part):
             batch.max_q_len, batch.max_kv_len, self.scale, window=self.window,
             min_q_len=batch.min_q_len,
         )
-        return ops.linear(o, self.out)
+        return self.out.forward(o)

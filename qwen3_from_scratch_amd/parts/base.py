@@ -18,9 +18,12 @@ from ..config.registry import lookup_part
 @dataclass(frozen=True)
 class Precision:
     """Compute dtypes of one engine instance. Activations, matrices and the
-    cache share `act`; the residual stream and logits are float32."""
+    cache share `act`; the residual stream and logits are float32. `tiled`:
+    keep a second, tile-ordered copy of every bfloat16 matrix for the few-row
+    product kernel (decoding); it costs the matrices' memory once more."""
 
     act: torch.dtype
+    tiled: bool = True
 
     @classmethod
     def named(cls, name):

@@ -5,6 +5,7 @@ import torch
 from .. import ops
 from ..config.registry import register_part
 from .base import Part
+from .linear import LinearWeight
 
 
 @register_part("feed_forward", "swiglu")
@@ -36,10 +37,11 @@ class SwiGLU(Part):
     def load(self, fetch):
         act = self.precision.act
         I, H = self.intermediate_size, self.hidden_size
-        self.gate_up = torch.empty((2 * I, H), dtype=act, device=self.device)
-        self.gate_up[0::2].copy_(fetch(self._name("gate_proj.weight"), act, keep=False))
-        self.gate_up[1::2].copy_(fetch(self._name("up_proj.weight"), act, keep=False))
-        self.down = fetch(self._name("down_proj.weight"), act)
+        gate_up = torch.empty((2 * I, H), dtype=act, device=self.device)
+        gate_up[0::2].copy_(fetch(self._name("gate_proj.weight"), act, keep=False))
+        gate_up[1::2].copy_(fetch(self._name("up_proj.weight"), act, keep=False))
+        self.gate_up = LinearWeight(gate_up, self.precision)
+        self.down = LinearWeight(fetch(self._name("down_proj.weight"), act), self.precision)
 
     def forward(self, x, batch=None):
-        return ops.linear(ops.linear_swiglu(x, self.gate_up), self.down)
+        return self.down.forward(self.gate_up.forward_swiglu(x))

@@ -5,6 +5,7 @@ import torch
 from .. import ops
 from ..config.registry import register_part
 from .base import Part
+from .linear import LinearWeight
 
 
 @register_part("head", "linear")
@@ -26,7 +27,7 @@ class LinearHead(Part):
         return {self.weight_name: (self.vocab_size, self.hidden_size)}
 
     def load(self, fetch):
-        self.weight = fetch(self.weight_name, self.precision.act)
+        self.weight = LinearWeight(fetch(self.weight_name, self.precision.act), self.precision)
 
     def forward(self, h):
-        return ops.linear(h, self.weight, out_dtype=torch.float32)
+        return self.weight.forward(h, out_dtype=torch.float32)

@@ -303,6 +303,26 @@ def test_linear_few_rows_streams_weights(M, N, K):
         assert torch.equal(alone[0], got[0])
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 6144, 4096), (8, 4096, 12288), (16, 1000, 96), (3, 331, 64), (9, 24, 2048),
+                                   (5, 151936, 256)])
+def test_linear_from_the_tiled_copy(M, N, K):
+    """The tile-ordered copy gives the very sums of the row-major kernel: the same numbers
+    are added in the same order, only their addresses differ."""
+    ops = _ops()
+    x = _rand((M, K), torch.bfloat16, 23)
+    w = _rand((N, K), torch.bfloat16, 24, scale=0.05)
+    tiled = ops.tile_weight(w)
+    assert tiled is not None and tiled.numel() == -(-N // 16) * 16 * K
+    for out_dtype in (torch.bfloat16, torch.float32):
+        assert torch.equal(ops.linear(x, w, out_dtype=out_dtype, tiled=tiled), ops.linear(x, w, out_dtype=out_dtype))
+    if N % 2 == 0:
+        assert torch.equal(ops.linear_swiglu(x, w, tiled=tiled), ops.linear_swiglu(x, w))
+    assert ops.tile_weight(_rand((8, 72), torch.bfloat16, 1)) is None       # K not a multiple of 32
+    assert ops.tile_weight(w.float()) is None
+    many = _rand((40, K), torch.bfloat16, 25)                                 # many rows ignore the copy
+    assert torch.equal(ops.linear(many, w, tiled=tiled), ops.linear(many, w))
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,I,K", [(1, 12288, 4096), (8, 100, 72), (16, 333, 200), (40, 64, 64)])
 def test_linear_swiglu(dtype, M, I, K):

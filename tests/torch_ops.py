@@ -124,7 +124,11 @@ def paged_attention(q, num_q_heads, k_cache, v_cache, block_table, cu_seqlens_q,
     return res
 
 
-def linear(x, weight, out_dtype=None, out=None):
+def tile_weight(weight):
+    return None
+
+
+def linear(x, weight, out_dtype=None, out=None, tiled=None):
     res = (x.float() @ weight.float().T).to(out_dtype or x.dtype)
     if out is not None:
         out.copy_(res)
@@ -132,7 +136,7 @@ def linear(x, weight, out_dtype=None, out=None):
     return res
 
 
-def linear_swiglu(x, weight):
+def linear_swiglu(x, weight, tiled=None):
     return swiglu(linear(x, weight))
 
 
@@ -166,4 +170,4 @@ def sample(logits, temperature, top_k, seed, counter, out=None):
 
 
 ALL = ("embed_rows", "swiglu", "rmsnorm", "rope_table", "qk_norm_rope_store",
-       "paged_attention", "linear", "linear_swiglu", "sample")
+       "paged_attention", "linear", "linear_swiglu", "tile_weight", "sample")

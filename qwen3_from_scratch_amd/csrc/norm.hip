@@ -79,12 +79,13 @@ __global__ void rmsnorm_vec_kernel(float* __restrict__ x, const T* __restrict__ 
   float* xs = x + (size_t)s * H;
   const T* ds = delta ? delta + (size_t)s * H : nullptr;
   const int H4 = H >> 2;
-  float4 v[NORM_CHUNKS];
+  float4 v[NORM_CHUNKS], wv[NORM_CHUNKS];
   float acc = 0.f;
 #pragma unroll
   for (int c = 0; c < NORM_CHUNKS; ++c) {
     const int j = threadIdx.x + c * blockDim.x;
     if (j < H4) {
+      wv[c] = load4(weight + 4 * j);  // needed only after the sum; asked for now so that it has arrived by then
       v[c] = load4(xs + 4 * j);
       if (ds) {
         const float4 d = load4(ds + 4 * j);
@@ -101,7 +102,7 @@ __global__ void rmsnorm_vec_kernel(float* __restrict__ x, const T* __restrict__ 
     const int j = threadIdx.x + c * blockDim.x;
     if (j < H4) {
       if (write_back) store4(xs + 4 * j, v[c]);
-      const float4 w = load4(weight + 4 * j);
+      const float4 w = wv[c];
       store4(o + 4 * j, make_float4(v[c].x * scale * w.x, v[c].y * scale * w.y, v[c].z * scale * w.z,
                                     v[c].w * scale * w.w));
     }

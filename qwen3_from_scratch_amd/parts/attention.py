@@ -31,6 +31,9 @@ class PagedAttention(Part):
         if num_heads % num_kv_heads:
             raise ValueError("num_heads (%d) must be a multiple of num_kv_heads (%d)"
                              % (num_heads, num_kv_heads))
+        if head_dim % 16 or not 16 <= head_dim <= 256:
+            raise ValueError("the attention kernels take head sizes in steps of 16 from 16 to 256, not %d"
+                             % head_dim)
         self.hidden_size = hidden_size
         self.num_heads = num_heads
         self.num_kv_heads = num_kv_heads

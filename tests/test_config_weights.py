@@ -77,6 +77,12 @@ def test_spec_is_data_and_sizes_come_from_the_config():
         lookup_part("mixer", "nonesuch")
 
 
+def test_a_head_size_no_kernel_takes_is_refused_when_the_model_is_built():
+    raw = dict(TINY["A"]["config"], head_dim=24)
+    with pytest.raises(ValueError, match="steps of 16"):
+        build_model(ModelConfig.from_dict(raw), Precision(torch.float32), "cpu")
+
+
 def _rewrite(folder, out, change):
     tensors = load_file(os.path.join(folder, "model.safetensors"))
     change(tensors)

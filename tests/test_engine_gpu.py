@@ -96,3 +96,18 @@ def test_first_tokens(model_folders, dtype):
         runner = load_runner(model_folders[name], dtype=dtype, device="cuda",
                              page_size=TINY[name]["page_size"], max_tokens=64, max_requests=2)
         _compare(run_trace(runner, steps), want, dtype)
+
+
+def test_graph_replay_equals_eager_steps(model_folders):
+    """Single-token steps replay a captured graph; the same steps run eagerly give the same
+    logits up to the order of the splits' sums."""
+    name = "D"
+    requests = _requests(name, [70, 33, 150])
+    steps = trace_mixed(requests, seed=7, decode_tail=40)
+    kw = dict(dtype="bfloat16", device="cuda", page_size=16, max_tokens=max_live_tokens(steps, page=16),
+              max_requests=4)
+    a = run_trace(load_runner(model_folders[name], use_graphs=True, **kw), steps)
+    b = run_trace(load_runner(model_folders[name], use_graphs=False, **kw), steps)
+    assert a.keys() == b.keys()
+    worst = max(float((a[k] - b[k]).abs().max()) for k in a)
+    assert worst < 2e-2, worst

@@ -51,3 +51,32 @@ def test_real_layer_sizes_match_plain(folder, truth, dtype, tol, family):
         for i, p in enumerate(rows[rid]):
             diff = float((got[(rid, p)] - logits[i]).abs().max())
             assert diff <= tol * scale, (rid, p, diff, scale)
+
+
+def test_schedules_agree_at_real_sizes(folder):
+    """Sixteen requests through the engine twice, once with room for everything and once with
+    small portions, few sequences per step and so few pages that requests are preempted. In
+    float32 every kernel sums a row's numbers in an order that does not depend on the batch, so
+    the greedy tokens must be the same to the last one."""
+    from qwen3_from_scratch_amd.engine import SyncEngine
+
+    g = torch.Generator().manual_seed(9)
+    lengths = torch.randint(64, 600, (16,), generator=g).tolist()
+    news = torch.randint(8, 40, (16,), generator=g).tolist()
+    prompts = [random_tokens(n, 151936, 100 + i) for i, n in enumerate(lengths)]
+
+    def run(**kw):
+        engine = SyncEngine(path=folder, dtype="float32", block_size=16, **kw)
+        requests = [engine.add_request(p, engine.default_params(n, temperature=0.0, ignore_eos=True))
+                    for p, n in zip(prompts, news)]
+        while engine.scheduler.has_work():
+            engine.step()
+            engine.runner.manager.audit()
+        assert engine.runner.manager.num_free() == engine.runner.manager.num_pages()
+        return [r.generated for r in requests], sum(r.preemptions for r in requests)
+
+    roomy, _ = run(num_blocks=16 * 48, max_num_seqs=16, max_num_tokens=4096, chunked_prefill_size=512)
+    tight, preemptions = run(num_blocks=120, max_num_seqs=5, max_num_tokens=300, chunked_prefill_size=96)
+    assert [len(t) for t in roomy] == news
+    assert preemptions > 0
+    assert tight == roomy

@@ -517,25 +517,75 @@ __global__ __launch_bounds__(256) void attn_decode_reduce_kernel(
 // ---- sequences with many rows: portions of prompts ----------------------------
 // grid (row tiles, Hkv, B), 256 threads; a block owns 128 / G tokens x G heads,
 // each wavefront 32 rows of them (two blocks of 16). The block's threads bring
-// each 32-key tile from the cache into shared memory once, 16 bytes per load,
+// each 64-key tile from the cache into shared memory once, 16 bytes per load,
 // two tiles in flight (the next tile's loads are issued before the current
 // tile's arithmetic and stored after it); the wavefronts read their matrix-core
 // operands from there. K rows are padded by 16 bytes so that the sixteen rows a
-// read touches fall in different banks; V^T rows hold the tile's keys in the
-// order the P operand has them (for lane group g: keys 4g..4g+3 of the first
-// 16-key block, then of the second), so a V^T operand is one 16-byte read.
-// Row tiles are taken from the end of the sequence first: they have the most keys.
-// Block-table entries are copied to shared memory PREFILL_PAGES at a time, so
-// that no cache load waits for a table load.
-#define PREFILL_PAGES 2048
+// read touches fall in different banks; V^T rows hold each 32-key half of the
+// tile in the order the P operand has it (for lane group g: keys 4g..4g+3 of the
+// half's first 16-key block, then of its second), so a V^T operand is one
+// 16-byte read. Two stages of a 64-key tile take 72 KB of the CU's 160 KB, so two
+// blocks share a CU. The first half of the key heads takes its row tiles from the
+// sequence's end, the second half from its start, so that the blocks which come
+// to share a CU add up to about the same work. Block-table entries are copied to
+// shared memory PREFILL_PAGES at a time, so that no cache load waits for a table load.
+#define PREFILL_PAGES 1024
+#define PF_TILE 64
 template <int D>
 struct PrefillSmem {
-  static constexpr int K_ROW = D * 2 + 16;   // bytes
-  static constexpr int V_ROW = 64 + 16;      // 32 keys * 2 bytes + pad
-  static constexpr int K_BYTES = FAST_TILE * K_ROW;
+  static constexpr int K_ROW = D * 2 + 16;        // bytes
+  static constexpr int V_ROW = PF_TILE * 2 + 16;  // 64 keys * 2 bytes + pad
+  static constexpr int K_BYTES = PF_TILE * K_ROW;
   static constexpr int V_BYTES = D * V_ROW;
   static constexpr int STAGE = K_BYTES + V_BYTES;
 };
+
+// The softmax update of one block of 16 rows for one 64-key tile: as softmax_step, over
+// four 16-key blocks; the probabilities come back as the two P operands of the tile's halves.
+template <int NB>
+__device__ __forceinline__ void softmax_step64(const f32x4_t (&s)[4], bool full, int key0, int grp, int row_pos,
+                                               int window, float scale_log2, float& m_run, float& l_run,
+                                               f32x4_t (&acc)[NB], Pack16 (&p)[2]) {
+  float v[16];
+#pragma unroll
+  for (int j = 0; j < 16; ++j) v[j] = s[j >> 2][j & 3];
+  if (!full) {
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const int key = key0 + 16 * (j >> 2) + 4 * grp + (j & 3);
+      bool seen = key <= row_pos;
+      if (window > 0 && row_pos - key >= window) seen = false;
+      if (!seen) v[j] = -INFINITY;
+    }
+  }
+  float mx = v[0];
+#pragma unroll
+  for (int j = 1; j < 16; ++j) mx = fmaxf(mx, v[j]);
+  mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+  mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+  const float m_new = fmaxf(m_run, mx * scale_log2);
+  float sum = 0.f;
+  if (m_new > -INFINITY) {
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const float e = fast_exp2(fmaf(v[j], scale_log2, -m_new));
+      sum += e;
+      p[j >> 3].e[j & 7] = (__bf16)e;
+    }
+  } else {
+    p[0].u = make_uint4(0, 0, 0, 0);
+    p[1].u = make_uint4(0, 0, 0, 0);
+  }
+  const bool moved = m_new != m_run;
+  if (__builtin_amdgcn_ballot_w64(moved) != 0) {
+    const float alpha = m_new > -INFINITY ? fast_exp2(m_run - m_new) : 1.f;
+    l_run *= alpha;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) acc[nb] *= alpha;
+    m_run = m_new;
+  }
+  l_run += sum;
+}
 
 template <int D>
 __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
@@ -553,9 +603,6 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
   if (q_len * G <= 16) return;  // the other kernel's sequence
   const int n_tiles = (q_len + tokens_per_block - 1) / tokens_per_block;
   if ((int)blockIdx.x >= n_tiles) return;
-  // the first half of the key heads takes its row tiles from the sequence's end (most keys
-  // first), the second half from its start, so that blocks which come to share a CU add up
-  // to about the same work
   const int tile = (2 * (int)blockIdx.y < Hkv || Hkv == 1) ? n_tiles - 1 - blockIdx.x : blockIdx.x;
   const int kv_len = kv_lens[b];
   const int tid = threadIdx.x;
@@ -604,14 +651,14 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
   const int blk_first_tok = tile * tokens_per_block;
   const int blk_last_tok = min(q_len, blk_first_tok + tokens_per_block) - 1;
   int tile_lo = 0;
-  if (window > 0) tile_lo = max(0, first_pos + blk_first_tok - window + 1) / FAST_TILE;
-  const int tile_hi = (first_pos + blk_last_tok) / FAST_TILE + 1;
+  if (window > 0) tile_lo = max(0, first_pos + blk_first_tok - window + 1) / PF_TILE;
+  const int tile_hi = (first_pos + blk_last_tok) / PF_TILE + 1;
   // and this wavefront's own (a wavefront whose rows do not exist has none)
-  int my_lo = tile_lo, my_hi = pos_max >= 0 ? pos_max / FAST_TILE + 1 : 0;
-  if (window > 0 && pos_max >= 0) my_lo = max(0, pos_min - window + 1) / FAST_TILE;
+  int my_lo = tile_lo, my_hi = pos_max >= 0 ? pos_max / PF_TILE + 1 : 0;
+  if (window > 0 && pos_max >= 0) my_lo = max(0, pos_min - window + 1) / PF_TILE;
   const int* bt_row = block_table + (size_t)b * bt_stride;
 
-  constexpr int CHUNKS = D / 64;  // 16-byte chunks of K, and of V, per thread and tile
+  constexpr int CHUNKS = D / 32;  // 16-byte chunks of K, and of V, per thread and tile
   uint4 kreg[CHUNKS], vreg[CHUNKS];
   int page_base = 0;  // sh_pages[i] is the table's entry page_base + i
 
@@ -626,11 +673,11 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
     c_h[u] = idx & 1;
     c_voff[u] = ((idx >> 1) % D) * page + 8 * c_h[u];
   }
-
   const size_t page_elems = (size_t)page * D;  // elements of one (page, head) in either cache
+
   auto fetch = [&](int t) {
-    const int key0 = t * FAST_TILE;
-    if (key0 + FAST_TILE <= kv_len && window == 0) {
+    const int key0 = t * PF_TILE;
+    if (key0 + PF_TILE <= kv_len && window == 0) {
       // the whole tile lies inside the sequence and no page has been given back: no checks
 #pragma unroll
       for (int u = 0; u < CHUNKS; ++u) {
@@ -680,72 +727,74 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
       const int idx = tid + 256 * u;
       const int r = idx / (D / 8), c = idx % (D / 8);
       *reinterpret_cast<uint4*>(ks + r * SM::K_ROW + 16 * c) = kreg[u];
-      const int h = idx & 1, d = (idx >> 1) % D, kb = idx / (2 * D);
-      // keys 8h..8h+3 belong to lane group 2h, keys 8h+4..8h+7 to group 2h+1; within a group's
-      // 16 bytes the first block's four keys come first
-      unsigned char* row = vs + d * SM::V_ROW + 8 * kb;
+      const int h = idx & 1, d = (idx >> 1) % D, kb4 = idx / (2 * D);
+      // within a 32-key half: keys 8h..8h+3 of a 16-key block belong to lane group 2h, keys
+      // 8h+4..8h+7 to group 2h+1; within a group's 16 bytes the half's first block comes first
+      unsigned char* row = vs + d * SM::V_ROW + 64 * (kb4 >> 1) + 8 * (kb4 & 1);
       *reinterpret_cast<uint2*>(row + 16 * (2 * h)) = make_uint2(vreg[u].x, vreg[u].y);
       *reinterpret_cast<uint2*>(row + 16 * (2 * h + 1)) = make_uint2(vreg[u].z, vreg[u].w);
     }
   };
 
   // tiles are worked through in spans whose table entries fit sh_pages
-  const int tiles_per_span = max(1, (PREFILL_PAGES - 2) * (page / 16) / 2);
+  const int tiles_per_span = max(1, (PREFILL_PAGES - 4) * (page / 16) / 4);
   for (int span_lo = tile_lo; span_lo < tile_hi; span_lo += tiles_per_span) {
-  const int span_hi = min(tile_hi, span_lo + tiles_per_span);
-  __syncthreads();
-  page_base = (span_lo * FAST_TILE) >> page_shift;
-  {
-    const int last_page = min((kv_len - 1) >> page_shift, (span_hi * FAST_TILE - 1) >> page_shift);
-    for (int i = tid; page_base + i <= last_page; i += 256) sh_pages[i] = bt_row[page_base + i];
-  }
-  __syncthreads();
-  fetch(span_lo);
-  stash(0);
-  __syncthreads();
-  for (int t = span_lo; t < span_hi; ++t) {
-    const int stage = (t - span_lo) & 1;
-    const bool more = t + 1 < span_hi;
-    if (more) fetch(t + 1);
-    if (t >= my_lo && t < my_hi) {
-      const unsigned char* ks = smem + stage * SM::STAGE;
-      const unsigned char* vs = ks + SM::K_BYTES;
-      const int key0 = t * FAST_TILE;
-      f32x4_t sc[2][2];
+    const int span_hi = min(tile_hi, span_lo + tiles_per_span);
+    __syncthreads();
+    page_base = (span_lo * PF_TILE) >> page_shift;
+    {
+      const int last_page = min((kv_len - 1) >> page_shift, (span_hi * PF_TILE - 1) >> page_shift);
+      for (int i = tid; page_base + i <= last_page; i += 256) sh_pages[i] = bt_row[page_base + i];
+    }
+    __syncthreads();
+    fetch(span_lo);
+    stash(0);
+    __syncthreads();
+    for (int t = span_lo; t < span_hi; ++t) {
+      const int stage = (t - span_lo) & 1;
+      const bool more = t + 1 < span_hi;
+      if (more) fetch(t + 1);
+      if (t >= my_lo && t < my_hi) {
+        const unsigned char* ks = smem + stage * SM::STAGE;
+        const unsigned char* vs = ks + SM::K_BYTES;
+        const int key0 = t * PF_TILE;
+        f32x4_t sc[2][4];
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
-        Pack16 a[D / 32];
-#pragma unroll
-        for (int i = 0; i < D / 32; ++i)
-          a[i].u = *reinterpret_cast<const uint4*>(ks + (16 * kb + col) * SM::K_ROW + 64 * i + 16 * grp);
-#pragma unroll
-        for (int qb = 0; qb < 2; ++qb) {
-          f32x4_t c = {0.f, 0.f, 0.f, 0.f};
+        for (int kb4 = 0; kb4 < 4; ++kb4) {
+          Pack16 a[D / 32];
 #pragma unroll
           for (int i = 0; i < D / 32; ++i)
-            c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i].v, qreg[qb][i].v, c, 0, 0, 0);
-          sc[qb][kb] = c;
+            a[i].u = *reinterpret_cast<const uint4*>(ks + (16 * kb4 + col) * SM::K_ROW + 64 * i + 16 * grp);
+#pragma unroll
+          for (int qb = 0; qb < 2; ++qb) {
+            f32x4_t c = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int i = 0; i < D / 32; ++i)
+              c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i].v, qreg[qb][i].v, c, 0, 0, 0);
+            sc[qb][kb4] = c;
+          }
         }
-      }
-      // no key of the tile is hidden from any row of this wavefront?
-      const bool full = key0 + FAST_TILE - 1 <= pos_min && (window == 0 || pos_max - key0 < window);
-      Pack16 p[2];
-#pragma unroll
-      for (int qb = 0; qb < 2; ++qb)
-        p[qb] = softmax_step<D / 16>(sc[qb], full, key0, grp, row_pos[qb], window, scale_log2, m_run[qb], l_run[qb],
-                                     acc[qb]);
-#pragma unroll
-      for (int nb = 0; nb < D / 16; ++nb) {
-        Pack16 vt;
-        vt.u = *reinterpret_cast<const uint4*>(vs + (16 * nb + col) * SM::V_ROW + 16 * grp);
+        // no key of the tile is hidden from any row of this wavefront?
+        const bool full = key0 + PF_TILE - 1 <= pos_min && (window == 0 || pos_max - key0 < window);
+        Pack16 p[2][2];
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb)
-          acc[qb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt.v, p[qb].v, acc[qb][nb], 0, 0, 0);
+          softmax_step64<D / 16>(sc[qb], full, key0, grp, row_pos[qb], window, scale_log2, m_run[qb], l_run[qb],
+                                 acc[qb], p[qb]);
+#pragma unroll
+        for (int nb = 0; nb < D / 16; ++nb)
+#pragma unroll
+          for (int half = 0; half < 2; ++half) {
+            Pack16 vt;
+            vt.u = *reinterpret_cast<const uint4*>(vs + (16 * nb + col) * SM::V_ROW + 64 * half + 16 * grp);
+#pragma unroll
+            for (int qb = 0; qb < 2; ++qb)
+              acc[qb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt.v, p[qb][half].v, acc[qb][nb], 0, 0, 0);
+          }
       }
+      if (more) stash(stage ^ 1);
+      __syncthreads();
     }
-    if (more) stash(stage ^ 1);
-    __syncthreads();
-  }
   }
 #pragma unroll
   for (int qb = 0; qb < 2; ++qb) {

@@ -474,7 +474,7 @@ template <int D>
 __global__ __launch_bounds__(256) void attn_decode_reduce_kernel(
     bf16_t* __restrict__ out, const int* __restrict__ cu_q, int Hq, int Hkv, int splits,
     const float* __restrict__ ws_acc, const float* __restrict__ ws_ml) {
-  __shared__ float sh_w[16][MAX_SPLITS];
+  __shared__ float sh_w[16][MAX_SPLITS], sh_l[16][MAX_SPLITS];
   const int b = blockIdx.y, g_kv = blockIdx.x;
   const int G = Hq / Hkv;
   const int q0 = cu_q[b];
@@ -482,9 +482,20 @@ __global__ __launch_bounds__(256) void attn_decode_reduce_kernel(
   if (q_len <= 0 || q_len * G > 16) return;
   const int rows = q_len * G;
   const size_t base = ((size_t)b * Hkv + g_kv) * splits;
+  // every load of the kernel is issued before anything waits: maxima and sums here, and
+  // this thread's first accumulator elements
+  const int n_elems = rows * D;
+  float first[4] = {0.f, 0.f, 0.f, 0.f};
+  const int e0 = threadIdx.x;
+  if (splits <= 4 && e0 < n_elems) {
+    const int r = e0 / D, d = e0 - r * D;
+    for (int s = 0; s < splits; ++s) first[s] = ws_acc[((base + s) * 16 + r) * D + d];
+  }
   for (int idx = threadIdx.x; idx < rows * splits; idx += blockDim.x) {
     const int r = idx / splits, s = idx - r * splits;
-    sh_w[r][s] = ws_ml[((base + s) * 16 + r) * 2];  // the split's maximum, for now
+    const float2 ml = *reinterpret_cast<const float2*>(ws_ml + ((base + s) * 16 + r) * 2);
+    sh_w[r][s] = ml.x;
+    sh_l[r][s] = ml.y;
   }
   __syncthreads();
   if ((int)threadIdx.x < rows) {
@@ -495,22 +506,30 @@ __global__ __launch_bounds__(256) void attn_decode_reduce_kernel(
     for (int s = 0; s < splits; ++s) {
       const float ms = sh_w[r][s];
       const float e = ms > -INFINITY ? exp2f(ms - m_all) : 0.f;
-      l_all += ws_ml[((base + s) * 16 + r) * 2 + 1] * e;
+      l_all += sh_l[r][s] * e;
       sh_w[r][s] = e;
     }
     const float inv = 1.f / l_all;
     for (int s = 0; s < splits; ++s) sh_w[r][s] *= inv;
   }
   __syncthreads();
-  for (int idx = threadIdx.x; idx < rows * D; idx += blockDim.x) {
+  for (int idx = threadIdx.x; idx < n_elems; idx += blockDim.x) {
     const int r = idx / D, d = idx - r * D;
     float o = 0.f;
-    for (int s = 0; s < splits; ++s) {
-      const float wgt = sh_w[r][s];
-      if (wgt != 0.f) o += ws_acc[((base + s) * 16 + r) * D + d] * wgt;
+    if (splits <= 4 && idx == e0) {
+      for (int s = 0; s < splits; ++s) o += first[s] * sh_w[r][s];
+    } else {
+      const float* src = ws_acc + (base * 16 + r) * D + d;
+      int s = 0;
+      for (; s + 4 <= splits; s += 4) {  // four loads in flight at a time; an empty split's partial is zero
+        const float a0 = src[(size_t)(s + 0) * 16 * D], a1 = src[(size_t)(s + 1) * 16 * D];
+        const float a2 = src[(size_t)(s + 2) * 16 * D], a3 = src[(size_t)(s + 3) * 16 * D];
+        o += a0 * sh_w[r][s] + a1 * sh_w[r][s + 1] + a2 * sh_w[r][s + 2] + a3 * sh_w[r][s + 3];
+      }
+      for (; s < splits; ++s) o += src[(size_t)s * 16 * D] * sh_w[r][s];
     }
     const int token = q0 + r / G, head = g_kv * G + r % G;
-    out[(size_t)token * Hq * D + (size_t)head * D + d] = float_to_bf16(o * 1.f);
+    out[(size_t)token * Hq * D + (size_t)head * D + d] = float_to_bf16(o);
   }
 }
 

@@ -249,8 +249,9 @@ def paged_attention(q, num_q_heads, k_cache, v_cache, block_table, cu_seqlens_q,
         lib = library("attention")
         splits, workspace = 1, None
         if lib.q3_paged_attention_fast_path(Hq, Hkv, D, page, _DT[q.dtype]) and min_q_len * (Hq // Hkv) <= 16:
-            # few rows per sequence: split the keys over blocks until the chip is full
-            splits = max(1, min(max_kv_len // 256, -(-512 // (B * Hkv)), 64))
+            # few rows per sequence: split the keys over blocks until the chip is full (about two
+            # blocks a compute unit; beyond 32 parts the merge costs more than the split gains)
+            splits = max(1, min(max_kv_len // 64, -(-512 // (B * Hkv)), 32))
             if splits > 1:
                 lib.q3_paged_attention_workspace.restype = ctypes.c_long
                 n = lib.q3_paged_attention_workspace(B, Hkv, D, splits)

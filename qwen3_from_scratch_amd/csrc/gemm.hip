@@ -125,20 +125,76 @@ union Pack16 {
 // contiguous kilobyte instead of sixteen 64-byte pieces of sixteen rows, which the memory
 // system serves about a fifth faster. Rows are padded with zeros to a multiple of 16, and K
 // is a multiple of 32.
-template <typename OUT, bool SWIGLU, bool TILED>
+//
+// Two fusions with the norm between two products, both for TILED weights only (`SkinnyFusion`):
+// * EPI_RESIDUAL: the product is a residual stream's next addend. The epilogue rounds it to
+//   bfloat16 (what a separate addition would have read), adds it into `residual` (M, N) float32
+//   in place, writes (residual * norm_weight) as bfloat16 to out: the next norm's rows, weighted
+//   but not yet divided by their root mean square; and leaves, per slab of 16 columns, each
+//   row's sum of squares in `sums_out` (slabs, 16). A slab's columns belong to one wavefront,
+//   so nothing is added twice and no order depends on timing.
+// * `row_sums`: the rows of x are such weighted, unscaled rows. The block adds the partial sums
+//   (`sums_rows` slabs of 16 rows) in a fixed order and multiplies row m of the product by
+//   rsqrt(sum_m * inv_width + eps) before any other epilogue: (x / rms) @ W^T = (x @ W^T) / rms.
+enum { EPI_PLAIN = 0, EPI_SWIGLU = 1, EPI_RESIDUAL = 2 };
+
+struct SkinnyFusion {
+  const float* row_sums;
+  int sums_rows;
+  float eps, inv_width;
+  float* residual;
+  const void* norm_weight;
+  int norm_weight_f32;
+  float* sums_out;
+};
+
+#define SKINNY_PRE 4  // float4 loads of partial sums a thread has in flight beside the main loop's
+
+template <typename OUT, int EPI, bool TILED, bool SCALED>
 __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restrict__ x,
                                                            const bf16_t* __restrict__ w, OUT* __restrict__ out,
-                                                           int M, int N, int K, int kw, int k_per_wave) {
-  extern __shared__ float red[];  // [waves][64][4]
+                                                           int M, int N, int K, int kw, int k_per_wave,
+                                                           SkinnyFusion fu) {
+  extern __shared__ float red[];  // [waves][64][4], then [waves][16] for the rows' sums
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, grp = lane >> 4;
-  const int sw = (blockDim.x >> 6) / kw;
+  const int nwaves = blockDim.x >> 6;
+  const int sw = nwaves / kw;
   const int slab = blockIdx.x * sw + wave / kw;
   const int ksplit = wave % kw;
   const int n0 = slab * 16;
   const int k_begin = ksplit * k_per_wave;
   const int k_end = min(K, k_begin + k_per_wave);
   f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+
+  // partial sums of the rows' squares: thread -> (rows 4q .. 4q + 3, slabs i0, i0 + stride, ...)
+  constexpr bool scaled = SCALED;
+  float4 pre[SKINNY_PRE];
+  if (scaled) {
+    const int q = threadIdx.x & 3, i0 = threadIdx.x >> 2, stride = blockDim.x >> 2;
+#pragma unroll
+    for (int u = 0; u < SKINNY_PRE; ++u) {
+      const int i = i0 + u * stride;
+      pre[u] = i < fu.sums_rows ? reinterpret_cast<const float4*>(fu.row_sums)[i * 4 + q] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+  }
+  // the residual and the norm's weights of this lane's four outputs, asked for before the products
+  const int n = n0 + 4 * grp;
+  float4 res = make_float4(0.f, 0.f, 0.f, 0.f), nw = res;
+  const bool owner = EPI == EPI_RESIDUAL && ksplit == 0 && col < M && n + 3 < N;
+  if (EPI == EPI_RESIDUAL && owner) {
+    res = *reinterpret_cast<const float4*>(fu.residual + (size_t)col * N + n);
+    if (fu.norm_weight_f32) {
+      nw = *reinterpret_cast<const float4*>(static_cast<const float*>(fu.norm_weight) + n);
+    } else {
+      union {
+        uint2 u;
+        bf16_t e[4];
+      } pk;
+      pk.u = *reinterpret_cast<const uint2*>(static_cast<const bf16_t*>(fu.norm_weight) + n);
+      nw = make_float4(bf16_to_float(pk.e[0]), bf16_to_float(pk.e[1]), bf16_to_float(pk.e[2]), bf16_to_float(pk.e[3]));
+    }
+  }
 
   const bool row_ok = TILED ? n0 < N : n0 + col < N;
   const bool x_ok = col < M;
@@ -160,18 +216,69 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
 #pragma unroll
     for (int u = 0; u < SKINNY_U; ++u) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u].v, b[u].v, acc, 0, 0, 0);
   }
+  float* sums = red + (size_t)nwaves * 256;
+  if (scaled) {
+    float4 s = pre[0];
+#pragma unroll
+    for (int u = 1; u < SKINNY_PRE; ++u) {
+      s.x += pre[u].x; s.y += pre[u].y; s.z += pre[u].z; s.w += pre[u].w;
+    }
+    const int q = threadIdx.x & 3, stride = blockDim.x >> 2;
+    for (int i = (threadIdx.x >> 2) + SKINNY_PRE * stride; i < fu.sums_rows; i += stride) {
+      const float4 v = reinterpret_cast<const float4*>(fu.row_sums)[i * 4 + q];
+      s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+    }
+#pragma unroll
+    for (int off = 4; off < 64; off <<= 1) {
+      s.x += __shfl_xor(s.x, off, 64); s.y += __shfl_xor(s.y, off, 64);
+      s.z += __shfl_xor(s.z, off, 64); s.w += __shfl_xor(s.w, off, 64);
+    }
+    if (lane < 4) *reinterpret_cast<float4*>(sums + wave * 16 + 4 * lane) = s;
+  }
   if (kw > 1) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) red[(wave * 64 + lane) * 4 + j] = acc[j];
-    __syncthreads();
+  }
+  if (kw > 1 || scaled) __syncthreads();
+  if (kw > 1) {
     if (ksplit != 0) return;
     for (int s = 1; s < kw; ++s)
 #pragma unroll
       for (int j = 0; j < 4; ++j) acc[j] += red[((wave + s) * 64 + lane) * 4 + j];
   }
+  if (scaled) {
+    float total = 0.f;
+    for (int wv = 0; wv < nwaves; ++wv) total += sums[wv * 16 + col];
+    const float r = rsqrtf(total * fu.inv_width + fu.eps);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[j] *= r;
+  }
+  if constexpr (EPI == EPI_RESIDUAL) {
+    // N is a multiple of 16 here: a slab is whole or absent
+    float ss = 0.f;
+    if (owner) {
+      const float xn[4] = {res.x + bf16_to_float(float_to_bf16(acc[0])), res.y + bf16_to_float(float_to_bf16(acc[1])),
+                           res.z + bf16_to_float(float_to_bf16(acc[2])), res.w + bf16_to_float(float_to_bf16(acc[3]))};
+      *reinterpret_cast<float4*>(fu.residual + (size_t)col * N + n) = make_float4(xn[0], xn[1], xn[2], xn[3]);
+      const float wn[4] = {nw.x, nw.y, nw.z, nw.w};
+      union {
+        uint2 u;
+        bf16_t e[4];
+      } pk;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        ss += xn[j] * xn[j];
+        pk.e[j] = float_to_bf16(xn[j] * wn[j]);
+      }
+      *reinterpret_cast<uint2*>(reinterpret_cast<bf16_t*>(out) + (size_t)col * N + n) = pk.u;
+    }
+    ss += __shfl_xor(ss, 16, 64);
+    ss += __shfl_xor(ss, 32, 64);
+    if (grp == 0 && n0 < N) fu.sums_out[slab * 16 + col] = ss;
+    return;
+  }
   if (col >= M) return;
-  const int n = n0 + 4 * grp;
-  if constexpr (SWIGLU) {
+  if constexpr (EPI == EPI_SWIGLU) {
     OUT* o = out + (size_t)col * (N / 2) + n / 2;  // n is even: pairs (n, n + 1) and (n + 2, n + 3)
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
@@ -203,8 +310,9 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
   }
 }
 
-template <typename OUT, bool SWIGLU, bool TILED = false>
-static int launch_skinny(const void* x, const void* w, void* out, int M, int N, int K, hipStream_t stream) {
+template <typename OUT, int EPI, bool TILED = false, bool SCALED = false>
+static int launch_skinny(const void* x, const void* w, void* out, int M, int N, int K, hipStream_t stream,
+                         SkinnyFusion fu = SkinnyFusion{}) {
   const int slabs = (N + 15) / 16;
   // enough wavefronts to keep every CU's memory pipeline full (about 4096), each with at
   // least four k-steps
@@ -216,9 +324,9 @@ static int launch_skinny(const void* x, const void* w, void* out, int M, int N, 
   int k_per_wave = (K + kw - 1) / kw;
   k_per_wave = (k_per_wave + step - 1) / step * step;
   const int blocks = (slabs + sw - 1) / sw;
-  const size_t smem = kw > 1 ? (size_t)sw * kw * 64 * 4 * sizeof(float) : 0;
-  hipLaunchKernelGGL((gemm_skinny_kernel<OUT, SWIGLU, TILED>), dim3(blocks), dim3(64 * sw * kw), smem, stream,
-                     (const bf16_t*)x, (const bf16_t*)w, (OUT*)out, M, N, K, kw, k_per_wave);
+  const size_t smem = (size_t)sw * kw * (64 * 4 + 16) * sizeof(float);
+  hipLaunchKernelGGL((gemm_skinny_kernel<OUT, EPI, TILED, SCALED>), dim3(blocks), dim3(64 * sw * kw), smem, stream,
+                     (const bf16_t*)x, (const bf16_t*)w, (OUT*)out, M, N, K, kw, k_per_wave, fu);
   return q3_launch_status();
 }
 
@@ -239,8 +347,8 @@ extern "C" int q3_linear(const void* x, const void* weight, void* out, int M, in
     return q3_launch_status();
   }
   if (!q3_linear_is_skinny(M, N, K, in_dtype)) return Q3_ERR_UNSUPPORTED;
-  return out_dtype == Q3_F32 ? launch_skinny<float, false>(x, weight, out, M, N, K, stream)
-                             : launch_skinny<bf16_t, false>(x, weight, out, M, N, K, stream);
+  return out_dtype == Q3_F32 ? launch_skinny<float, EPI_PLAIN>(x, weight, out, M, N, K, stream)
+                             : launch_skinny<bf16_t, EPI_PLAIN>(x, weight, out, M, N, K, stream);
 }
 
 // out (M, N / 2) = silu(gate) * up where x @ weight^T interleaves gate and up columns
@@ -249,19 +357,49 @@ extern "C" int q3_linear_swiglu(const void* x, const void* weight, void* out, in
                                 hipStream_t stream) {
   if (M <= 0 || N <= 0 || K <= 0 || N % 2) return Q3_ERR_BAD_ARGUMENT;
   if (!q3_linear_is_skinny(M, N, K, dtype)) return Q3_ERR_UNSUPPORTED;
-  return launch_skinny<bf16_t, true>(x, weight, out, M, N, K, stream);
+  return launch_skinny<bf16_t, EPI_SWIGLU>(x, weight, out, M, N, K, stream);
 }
 
 // The same products from the tile-ordered copy of the weight (see gemm_skinny_kernel):
-// x (M, K) bfloat16, M <= 16, K a multiple of 32; `swiglu` selects the activation epilogue
-// (output (M, N / 2) bfloat16), otherwise output (M, N) in `out_dtype`.
+// x (M, K) bfloat16, M <= 16, K a multiple of 32. `epilogue`: 0 output (M, N) in `out_dtype`;
+// 1 the activation (output (M, N / 2) bfloat16); 2 the residual addition and the next norm's
+// preparation (N a multiple of 16; `residual` (M, N) float32 updated in place, `norm_weight`
+// (N,) of `norm_w_dtype`, output (M, N) bfloat16 = residual * norm_weight, `sums_out`
+// (N / 16, 16) float32). `row_sums` (sums_rows, 16) float32, if not null, says that x's rows
+// still lack the factor rsqrt(sum / width + eps), which the product's rows then receive.
 extern "C" int q3_linear_tiled(const void* x, const void* weight_tiled, void* out, int M, int N, int K,
-                               int out_dtype, int swiglu, hipStream_t stream) {
+                               int out_dtype, int epilogue, const float* row_sums, int sums_rows, float eps,
+                               int width, float* residual, const void* norm_weight, int norm_w_dtype,
+                               float* sums_out, hipStream_t stream) {
   if (M <= 0 || M > 16 || N <= 0 || K <= 0 || K % 32) return Q3_ERR_BAD_ARGUMENT;
-  if (swiglu) {
-    if (N % 2 || out_dtype != Q3_BF16) return Q3_ERR_BAD_ARGUMENT;
-    return launch_skinny<bf16_t, true, true>(x, weight_tiled, out, M, N, K, stream);
+  SkinnyFusion fu{};
+  if (row_sums) {
+    if (sums_rows <= 0 || width <= 0) return Q3_ERR_BAD_ARGUMENT;
+    fu.row_sums = row_sums;
+    fu.sums_rows = sums_rows;
+    fu.eps = eps;
+    fu.inv_width = 1.f / (float)width;
   }
-  return out_dtype == Q3_F32 ? launch_skinny<float, false, true>(x, weight_tiled, out, M, N, K, stream)
-                             : launch_skinny<bf16_t, false, true>(x, weight_tiled, out, M, N, K, stream);
+  if (epilogue == EPI_SWIGLU) {
+    if (N % 2 || out_dtype != Q3_BF16) return Q3_ERR_BAD_ARGUMENT;
+    return row_sums ? launch_skinny<bf16_t, EPI_SWIGLU, true, true>(x, weight_tiled, out, M, N, K, stream, fu)
+                    : launch_skinny<bf16_t, EPI_SWIGLU, true>(x, weight_tiled, out, M, N, K, stream, fu);
+  }
+  if (epilogue == EPI_RESIDUAL) {
+    if (row_sums || N % 16 || out_dtype != Q3_BF16 || !residual || !norm_weight || !sums_out ||
+        (norm_w_dtype != Q3_F32 && norm_w_dtype != Q3_BF16))
+      return Q3_ERR_BAD_ARGUMENT;
+    fu.residual = residual;
+    fu.norm_weight = norm_weight;
+    fu.norm_weight_f32 = norm_w_dtype == Q3_F32;
+    fu.sums_out = sums_out;
+    return launch_skinny<bf16_t, EPI_RESIDUAL, true>(x, weight_tiled, out, M, N, K, stream, fu);
+  }
+  if (epilogue != EPI_PLAIN) return Q3_ERR_BAD_ARGUMENT;
+  if (row_sums)
+    return out_dtype == Q3_F32
+               ? launch_skinny<float, EPI_PLAIN, true, true>(x, weight_tiled, out, M, N, K, stream, fu)
+               : launch_skinny<bf16_t, EPI_PLAIN, true, true>(x, weight_tiled, out, M, N, K, stream, fu);
+  return out_dtype == Q3_F32 ? launch_skinny<float, EPI_PLAIN, true>(x, weight_tiled, out, M, N, K, stream, fu)
+                             : launch_skinny<bf16_t, EPI_PLAIN, true>(x, weight_tiled, out, M, N, K, stream, fu);
 }

@@ -100,9 +100,13 @@ class DecoderModel:
         x = self.embedding.forward(batch.token_ids)
         x = self.position.on_embeddings(x, batch)
         pending = None
-        for i, step in enumerate(self.spec.order):
+        order = self.spec.order
+        for i, step in enumerate(order):
             view = cache.view(self.plane_of_step[i], writes=step.reads_cache_of is None)
-            x, pending = self.layers[step.layer].block.forward(x, pending, batch, view)
+            # the norm at the next block's entry, if that block can take over its division
+            entry = getattr(self.layers[order[i + 1].layer].block, "entry_norm", None) if i + 1 < len(order) else None
+            x, pending = self.layers[step.layer].block.forward(x, pending, batch, view,
+                                                               next_norm=entry() if entry else None)
         h = self.final_norm.forward(x, delta=pending, rows=batch.logits_rows)
         return self.head.forward(h)
 

@@ -28,6 +28,7 @@ __all__ = [
     "swiglu",
     "linear",
     "linear_swiglu",
+    "linear_residual_norm",
     "tile_weight",
     "sample",
 ]
@@ -289,9 +290,24 @@ def _tiled_ok(tiled, weight, M):
     return True
 
 
-def linear(x, weight, out_dtype=None, out=None, tiled=None):
+def _row_sums_args(unscaled, M, K):
+    """The kernel's arguments for rows that still lack their 1 / rms factor:
+    `unscaled` = (sums (P, 16) float32, eps, width) as `linear_residual_norm` leaves them."""
+    if unscaled is None:
+        return None, 0, ctypes.c_float(0.0), 0
+    sums, eps, width = unscaled
+    _dev(sums)
+    _need(sums.dtype == torch.float32 and sums.dim() == 2 and sums.shape[1] == 16 and sums.shape[0] > 0
+          and sums.is_contiguous(), "row sums must be float32 (P, 16)")
+    _need(width == K, "the rows' width must be the product's inner size")
+    return _ptr(sums), sums.shape[0], ctypes.c_float(eps), int(width)
+
+
+def linear(x, weight, out_dtype=None, out=None, tiled=None, unscaled=None):
     """out = x @ weight^T with float32 accumulation. x (M, K), weight (N, K).
     `tiled` is `tile_weight(weight)`, if the caller keeps one: few rows are then served from it.
+    `unscaled` (see `linear_residual_norm`) says that x's rows still lack their 1 / rms factor;
+    the product's rows receive it. Only the few-row kernel on a tiled weight does this.
 
     float32 operands take a float32 kernel with no reduced-precision mode;
     bfloat16 operands with at most 16 rows take a weight-streaming matrix-core
@@ -309,9 +325,13 @@ def linear(x, weight, out_dtype=None, out=None, tiled=None):
         out = torch.empty((M, N), dtype=out_dtype, device=x.device)
     _need(out.shape == (M, N) and out.dtype == out_dtype, "out must be (M, N) of out_dtype")
     if M and x.dtype == torch.bfloat16 and _tiled_ok(tiled, weight, M):
+        sums, sums_rows, eps, width = _row_sums_args(unscaled, M, K)
         _check(library("gemm").q3_linear_tiled(
-            _ptr(x), _ptr(tiled), _ptr(out), M, N, K, _DT[out_dtype], 0, _stream()), "linear")
-    elif M and x.dtype == torch.bfloat16 and not library("gemm").q3_linear_is_skinny(M, N, K, 1):
+            _ptr(x), _ptr(tiled), _ptr(out), M, N, K, _DT[out_dtype], 0, sums, sums_rows, eps, width,
+            None, None, 0, None, _stream()), "linear")
+        return out
+    _need(unscaled is None, "unscaled rows need the few-row kernel: bfloat16, at most 16 rows, a tiled weight")
+    if M and x.dtype == torch.bfloat16 and not library("gemm").q3_linear_is_skinny(M, N, K, 1):
         # bfloat16 products with many rows go to the vendor library (hipBLASLt through
         # torch), as the reference's engine uses its vendor library for them; accumulation
         # is float32. Few rows take the weight-streaming kernel below.
@@ -325,10 +345,11 @@ def linear(x, weight, out_dtype=None, out=None, tiled=None):
     return out
 
 
-def linear_swiglu(x, weight, tiled=None):
+def linear_swiglu(x, weight, tiled=None, unscaled=None):
     """swiglu(x @ weight^T) for a weight whose rows interleave gate and up (row 2i gate's, row
     2i + 1 up's): (M, K) x (2I, K) -> (M, I). With few bfloat16 rows the activation is the
-    product kernel's epilogue; otherwise it is the product followed by `swiglu`."""
+    product kernel's epilogue; otherwise it is the product followed by `swiglu`.
+    `unscaled`: as for `linear`."""
     _dev(x, weight)
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1] and weight.shape[0] % 2 == 0,
           "x (M, K) and weight (2I, K)")
@@ -337,15 +358,46 @@ def linear_swiglu(x, weight, tiled=None):
     N = weight.shape[0]
     if M and x.dtype == torch.bfloat16 and _tiled_ok(tiled, weight, M):
         out = torch.empty((M, N // 2), dtype=x.dtype, device=x.device)
-        _check(library("gemm").q3_linear_tiled(_ptr(x), _ptr(tiled), _ptr(out), M, N, K, 1, 1, _stream()),
-               "linear_swiglu")
+        sums, sums_rows, eps, width = _row_sums_args(unscaled, M, K)
+        _check(library("gemm").q3_linear_tiled(
+            _ptr(x), _ptr(tiled), _ptr(out), M, N, K, 1, 1, sums, sums_rows, eps, width,
+            None, None, 0, None, _stream()), "linear_swiglu")
         return out
+    _need(unscaled is None, "unscaled rows need the few-row kernel: bfloat16, at most 16 rows, a tiled weight")
     if M and library("gemm").q3_linear_is_skinny(M, N, K, _DT[x.dtype]):
         out = torch.empty((M, N // 2), dtype=x.dtype, device=x.device)
         _check(library("gemm").q3_linear_swiglu(_ptr(x), _ptr(weight), _ptr(out), M, N, K, _DT[x.dtype], _stream()),
                "linear_swiglu")
         return out
     return swiglu(linear(x, weight, tiled=tiled))
+
+
+def linear_residual_norm(x, weight, tiled, residual, norm_weight):
+    """residual += x @ weight^T, and the next norm's input prepared in the same kernel.
+
+    x (M, K) bfloat16 with M <= 16, weight (N, K) with its tiled copy, N a multiple of 16;
+    residual (M, N) float32 is updated in place (the product is rounded to bfloat16 before the
+    addition, as a product written out and added by the norm kernel would be). Returns
+    (values, sums): values (M, N) bfloat16 = residual * norm_weight, and sums (N / 16, 16)
+    float32, the rows' sums of squares of the new residual in partial sums of 16 columns (row m
+    of the stream in column m). The norm's result is values * rsqrt(sum / N + eps) row by row;
+    `linear` and `linear_swiglu` apply that factor to their products when given
+    `unscaled=(sums, eps, N)`."""
+    _dev(x, weight, tiled, residual, norm_weight)
+    _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1], "x (M, K) and weight (N, K)")
+    M, K = x.shape
+    N = weight.shape[0]
+    _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and _tiled_ok(tiled, weight, M) and N % 16 == 0,
+          "bfloat16, 1 to 16 rows, a tiled weight and a width that is a multiple of 16")
+    _need(residual.shape == (M, N) and residual.dtype == torch.float32 and residual.is_contiguous(),
+          "residual must be float32 (M, N)")
+    _need(norm_weight.shape == (N,) and norm_weight.dtype in _DT and norm_weight.is_contiguous(), "norm weight (N,)")
+    values = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    sums = torch.empty((N // 16, 16), dtype=torch.float32, device=x.device)
+    _check(library("gemm").q3_linear_tiled(
+        _ptr(x), _ptr(tiled), _ptr(values), M, N, K, 1, 2, None, 0, ctypes.c_float(0.0), 0,
+        _ptr(residual), _ptr(norm_weight), _DT[norm_weight.dtype], _ptr(sums), _stream()), "linear_residual_norm")
+    return values, sums
 
 
 def sample(logits, temperature, top_k, seed, counter, out=None):

@@ -24,6 +24,7 @@ class PagedAttention(Part):
     """
 
     graph_safe = True
+    feeds_sink = True
 
     def __init__(self, prefix, precision, device, hidden_size, num_heads, num_kv_heads, head_dim,
                  qk_norm=True, qk_norm_eps=1e-6, window=0, scale=None):
@@ -77,7 +78,11 @@ class PagedAttention(Part):
             self.q_weight = fetch(self._name("q_norm.weight"))
             self.k_weight = fetch(self._name("k_norm.weight"))
 
-    def forward(self, x, batch, cache):
+    @property
+    def takes_unscaled(self):
+        return self.qkv is not None and self.qkv.fuses
+
+    def forward(self, x, batch, cache, sink=None):
         Hq, Hkv, D = self.num_heads, self.num_kv_heads, self.head_dim
         qkv = self.qkv.forward(x)
         table = self.position.rotation_table() if self.position is not None else None
@@ -95,4 +100,4 @@ class PagedAttention(Part):
             batch.max_q_len, batch.max_kv_len, self.scale, window=self.window,
             min_q_len=batch.min_q_len,
         )
-        return self.out.forward(o)
+        return self.out.forward(o) if sink is None else self.out.forward_into(o, sink)

@@ -65,6 +65,10 @@ class Part:
     # never synchronises with the host, and sizes nothing by a tensor's values.
     # A model with a part that does not declare this is run without graphs.
     graph_safe = False
+    # the norm fusion of steps with few rows (see NormSink, UnscaledRows): whether forward()
+    # takes `sink=`, and whether it takes UnscaledRows for its input
+    feeds_sink = False
+    takes_unscaled = False
 
     def __init__(self, prefix, precision, device):
         self.prefix = prefix
@@ -81,6 +85,35 @@ class Part:
 
     def _name(self, leaf):
         return self.prefix + "." + leaf if self.prefix else leaf
+
+
+@dataclass
+class NormSink:
+    """Where a part's last product may go instead of being returned: added into
+    `residual` (float32 (T, width), in place) and prepared for `norm`, the norm
+    that reads the residual next. A part whose class sets `feeds_sink` takes it
+    as `forward(..., sink=...)` and then returns `UnscaledRows`; it may also
+    ignore the sink and return its result as always."""
+
+    residual: torch.Tensor
+    norm: object
+
+
+@dataclass
+class UnscaledRows:
+    """A norm's output before the division by the root mean square: `values`
+    (T, width) hold residual * weight in the activation dtype, `sums` (P, 16)
+    float32 hold the rows' sums of squares in P partial sums (row t in column
+    t). A part whose `takes_unscaled` is true accepts this in place of its
+    input tensor and applies rsqrt(sum / width + eps) to its first product."""
+
+    values: torch.Tensor
+    sums: torch.Tensor
+    eps: float
+    width: int
+
+    def scale_args(self):
+        return (self.sums, self.eps, self.width)
 
 
 def build_part(spec, prefix, precision, device):

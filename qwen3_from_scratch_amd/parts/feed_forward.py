@@ -18,6 +18,7 @@ class SwiGLU(Part):
     feedback.py:52-54)."""
 
     graph_safe = True
+    feeds_sink = True
 
     def __init__(self, prefix, precision, device, hidden_size, intermediate_size):
         super().__init__(prefix, precision, device)
@@ -43,5 +44,10 @@ class SwiGLU(Part):
         self.gate_up = LinearWeight(gate_up, self.precision)
         self.down = LinearWeight(fetch(self._name("down_proj.weight"), act), self.precision)
 
-    def forward(self, x, batch=None):
-        return self.down.forward(self.gate_up.forward_swiglu(x))
+    @property
+    def takes_unscaled(self):
+        return self.gate_up is not None and self.gate_up.fuses
+
+    def forward(self, x, batch=None, sink=None):
+        h = self.gate_up.forward_swiglu(x)
+        return self.down.forward(h) if sink is None else self.down.forward_into(h, sink)

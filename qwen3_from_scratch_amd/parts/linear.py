@@ -4,6 +4,7 @@ in the order the few-row product kernel streams it."""
 import torch
 
 from .. import ops
+from .base import UnscaledRows
 
 
 class LinearWeight:
@@ -18,8 +19,28 @@ class LinearWeight:
         self.tiled = ops.tile_weight(weight) if precision.tiled else None
 
     def forward(self, x, out_dtype=None):
+        """x @ W^T; x may be UnscaledRows (see `fuses`)."""
+        if isinstance(x, UnscaledRows):
+            return ops.linear(x.values, self.weight, out_dtype=out_dtype, tiled=self.tiled, unscaled=x.scale_args())
         return ops.linear(x, self.weight, out_dtype=out_dtype, tiled=self.tiled)
 
     def forward_swiglu(self, x):
         """swiglu(x @ W^T) for a W whose rows interleave gate and up."""
+        if isinstance(x, UnscaledRows):
+            return ops.linear_swiglu(x.values, self.weight, tiled=self.tiled, unscaled=x.scale_args())
         return ops.linear_swiglu(x, self.weight, tiled=self.tiled)
+
+    @property
+    def fuses(self):
+        """Whether steps of at most 16 rows go through the few-row kernel, whose
+        epilogues carry the norm fusion: UnscaledRows in, a NormSink out."""
+        return self.tiled is not None
+
+    def forward_into(self, x, sink):
+        """x @ W^T added into the sink's residual and prepared for its norm, as
+        UnscaledRows; or, where the kernel does not take the case, returned."""
+        norm = sink.norm
+        if not self.fuses or x.shape[0] > 16 or self.weight.shape[0] % 16:
+            return self.forward(x)
+        values, sums = ops.linear_residual_norm(x, self.weight, self.tiled, sink.residual, norm.weight)
+        return UnscaledRows(values, sums, norm.eps, norm.size)

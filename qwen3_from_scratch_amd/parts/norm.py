@@ -4,7 +4,7 @@ import torch
 
 from .. import ops
 from ..config.registry import register_part
-from .base import Part
+from .base import NormSink, Part
 
 
 @register_part("norm", "rms")
@@ -34,3 +34,13 @@ class RMSNorm(Part):
         first (in place, unless `rows` selects a subset: then x is left alone)."""
         return ops.rmsnorm(x, self.weight, self.eps, self.precision.act, delta=delta,
                            rows=rows, write_back=rows is None)
+
+    def sink_for(self, x):
+        """A NormSink for the residual `x` if this step may have the addition
+        and this norm fused into the neighbouring products (bfloat16 with
+        tiled matrices, at most 16 rows), else None."""
+        if self.precision.act != torch.bfloat16 or not self.precision.tiled or not 1 <= x.shape[0] <= 16:
+            return None
+        if self.size % 16 or self.weight is None:
+            return None
+        return NormSink(x, self)

@@ -339,6 +339,59 @@ def test_linear_swiglu(dtype, M, I, K):
         assert torch.equal(got, ops.swiglu(ops.linear(x, w)))
 
 
+@pytest.mark.parametrize("norm_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,H,K,N2", [(1, 4096, 4096, 6144), (8, 4096, 12288, 24576), (16, 96, 224, 160),
+                                      (5, 992, 64, 330), (3, 32, 32, 48)])
+def test_linear_residual_norm_and_unscaled_rows(M, H, K, N2, norm_dtype):
+    """A product that adds itself into the residual stream and prepares the next norm, and the
+    product after it, which applies the norm's division: together they give what the product,
+    the norm kernel and the next product give one after the other."""
+    ops = _ops()
+    x = _rand((M, K), torch.bfloat16, 31)
+    w1 = _rand((H, K), torch.bfloat16, 32, scale=0.05)
+    w2 = _rand((N2, H), torch.bfloat16, 33, scale=0.05)
+    nw = (1.0 + _rand((H,), torch.float32, 34, scale=0.2)).to(norm_dtype)
+    residual = _rand((M, H), torch.float32, 35, scale=2.0)
+    eps = 1e-5
+    t1, t2 = ops.tile_weight(w1), ops.tile_weight(w2)
+
+    # one after the other
+    stream = residual.clone()
+    delta = ops.linear(x, w1, tiled=t1)
+    h = ops.rmsnorm(stream, nw, eps, torch.bfloat16, delta=delta)
+    want = ops.linear(h, w2, out_dtype=torch.float32, tiled=t2)
+    want_act = ops.linear_swiglu(h, w2, tiled=t2)
+
+    fused_stream = residual.clone()
+    values, sums = ops.linear_residual_norm(x, w1, t1, fused_stream, nw)
+    assert torch.equal(fused_stream, stream)                      # the stream itself is the same to the bit
+    assert sums.shape == (H // 16, 16)
+    ms = (stream.double() ** 2).sum(dim=1)
+    torch.testing.assert_close(sums.double().sum(dim=0)[:M], ms, rtol=1e-5, atol=1e-6)
+    assert float(sums[:, M:].abs().max()) == 0.0 if M < 16 else True
+    torch.testing.assert_close(values.float(), (stream * nw.float()), rtol=8e-3, atol=1e-6)
+    got = ops.linear(values, w2, out_dtype=torch.float32, tiled=t2, unscaled=(sums, eps, H))
+    # both roundings of the norm's output are to bfloat16, of numbers that differ by the row's factor
+    scale = float(want.abs().max())
+    assert float((got - want).abs().max()) <= 6e-3 * scale
+    exact = (stream.double() * torch.rsqrt((stream.double() ** 2).mean(dim=1, keepdim=True) + eps) * nw.double()) @ w2.double().T
+    assert float((got.double() - exact).abs().max()) <= 6e-3 * scale
+    got_act = ops.linear_swiglu(values, w2, tiled=t2, unscaled=(sums, eps, H))
+    assert float((got_act.float() - want_act.float()).abs().max()) <= 2e-2 * max(1.0, float(want_act.float().abs().max()))
+    # rows do not depend on their neighbours
+    if M > 1:
+        alone_stream = residual[:1].clone()
+        v1, s1 = ops.linear_residual_norm(x[:1].contiguous(), w1, t1, alone_stream, nw)
+        assert torch.equal(v1[0], values[0]) and torch.equal(s1[:, 0], sums[:, 0])
+        a = ops.linear(v1, w2, out_dtype=torch.float32, tiled=t2, unscaled=(s1, eps, H))
+        assert torch.equal(a[0], got[0])
+    # what the kernel does not take is refused
+    with pytest.raises(ops.OperandError):
+        ops.linear(_rand((17, H), torch.bfloat16, 1), w2, tiled=t2, unscaled=(sums, eps, H))
+    with pytest.raises(ops.OperandError):
+        ops.linear(values, w2, unscaled=(sums, eps, H))
+
+
 def test_linear_float32_is_true_float32():
     """Inputs whose products need all 24 bits: a matrix mode of reduced precision
     (bf16 or tf32-like splitting) would be off by far more than float32 rounding."""

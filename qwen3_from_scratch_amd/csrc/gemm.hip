@@ -314,10 +314,13 @@ template <typename OUT, int EPI, bool TILED = false, bool SCALED = false>
 static int launch_skinny(const void* x, const void* w, void* out, int M, int N, int K, hipStream_t stream,
                          SkinnyFusion fu = SkinnyFusion{}) {
   const int slabs = (N + 15) / 16;
-  // enough wavefronts to keep every CU's memory pipeline full (about 4096), each with at
-  // least four k-steps
+  // One slab per block, its K shared by up to eight wavefronts, each with at least four
+  // k-steps (measured on the 8B model's products at 1, 8 and 16 rows: eight beat four and
+  // sixteen by a few percent each, and blocks of several slabs are slower); sixteen where
+  // there are too few slabs to give every CU a block otherwise.
+  const int kw_max = slabs < 256 ? 16 : 8;
   int kw = 1;
-  while (kw < 16 && slabs * kw < 4096 && K / (kw * 2) >= 128) kw *= 2;
+  while (kw < kw_max && K / (kw * 2) >= 128) kw *= 2;
   int sw = 1;
   while (sw * kw < 4 && sw * 2 <= slabs) sw *= 2;
   const int step = 32 * SKINNY_U;

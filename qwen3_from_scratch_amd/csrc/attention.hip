@@ -6,6 +6,7 @@
 // rows and kv_len keys sits at position kv_len - q_len + i and sees keys at
 // positions <= its own, and, with a window w > 0, only those fewer than w behind.
 #include "common.h"
+#include "qk_prepare.h"
 
 #include <math.h>
 
@@ -373,22 +374,153 @@ __device__ __forceinline__ void attend_tiles(const Pack16 (&qreg)[QB][D / 32], c
 // tiles of the block's share of the keys in turn and are merged through shared
 // memory; with more than one split the block leaves an unnormalised partial
 // result (maximum, sum, accumulator) in the workspace for the reduction kernel.
-template <int D>
+// With PREP the kernel also does what the preparation kernel does for a step of single
+// tokens (q_len = 1 everywhere): `q` is then the step's raw [q | k | v] rows. Every block
+// normalises and rotates its own query rows on the way into the registers; the block whose
+// share of the keys holds the sequence's last position first normalises and rotates the new
+// key, writes it and the new value into the cache (if `prep.store`), and waits at a barrier
+// before any of its wavefronts reads keys: a block's own writes are visible to it after that.
+struct DecodePrep {
+  const void* q_weight;  // (D,) or null: no norm
+  const void* k_weight;
+  float eps;
+  const float* table;    // (max_pos, D): cos | sin, or null: no rotation
+  int max_pos;
+  bf16_t* k_cache;       // writable views of the caches, or null: nothing is stored
+  bf16_t* v_cache;
+};
+
+// One query row's operand registers from its raw values: lane (col, grp) holds elements
+// 32 i + 8 grp + j; the pairs (d, d + D / 2) are registers i and i + D / 64 of the same lane.
+// The sums take the order of the preparation kernel's butterfly (its lane c = 4 i + grp).
+template <int D, typename W>
+__device__ __forceinline__ void prepare_query(Pack16 (&qreg)[D / 32], const W* weight, float eps,
+                                              const float* table_row, int grp) {
+  constexpr int HI = D / 64;
+  float a[HI][8], b[HI][8];
+#pragma unroll
+  for (int i = 0; i < HI; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      a[i][j] = (float)qreg[i].e[j];
+      b[i][j] = (float)qreg[i + HI].e[j];
+    }
+  if (weight != nullptr) {
+    float ss = pairs_sum_of_squares(a[0], b[0]);
+    if constexpr (HI == 2) ss += pairs_sum_of_squares(a[1], b[1]);
+    ss += __shfl_xor(ss, 32, 64);
+    ss += __shfl_xor(ss, 16, 64);
+    const float scale = head_norm_scale(ss, D, eps);
+#pragma unroll
+    for (int i = 0; i < HI; ++i) {
+      float wa[8], wb[8];
+      load_weights8<W>(weight + 32 * i + 8 * grp, wa);
+      load_weights8<W>(weight + D / 2 + 32 * i + 8 * grp, wb);
+      pairs_normalise(a[i], b[i], scale, wa, wb);
+    }
+  }
+  if (table_row != nullptr) {
+#pragma unroll
+    for (int i = 0; i < HI; ++i) {
+      float cs[8], sn[8];
+      load_weights8<float>(table_row + 32 * i + 8 * grp, cs);
+      load_weights8<float>(table_row + D / 2 + 32 * i + 8 * grp, sn);
+      pairs_rotate(a[i], b[i], cs, sn);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < HI; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      qreg[i].e[j] = (__bf16)a[i][j];
+      qreg[i + HI].e[j] = (__bf16)b[i][j];
+    }
+}
+
+// The new key of head g_kv (threads 0 .. D / 16 - 1, as the preparation kernel's lanes) and
+// the new value (threads 64 .. 64 + D / 16 - 1) of the token whose raw row is `row`, into
+// slot pos % page of `pg`.
+template <int D, typename W>
+__device__ __forceinline__ void store_new_key_value(const bf16_t* row, int Hq, int Hkv, int g_kv, const W* k_weight,
+                                                    float eps, const float* table_row, bf16_t* k_cache,
+                                                    bf16_t* v_cache, int pg, int page, int slot) {
+  constexpr int LPH = D / 16, HALF = D / 2;
+  const int t = threadIdx.x;
+  if (t < LPH) {
+    const int c = t;
+    const bf16_t* src = row + (size_t)(Hq + g_kv) * D;
+    Half8 x1, x2;
+    x1.u = *reinterpret_cast<const uint4*>(src + 8 * c);
+    x2.u = *reinterpret_cast<const uint4*>(src + HALF + 8 * c);
+    float a[8], b[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      a[i] = bf16_to_float(x1.e[i]);
+      b[i] = bf16_to_float(x2.e[i]);
+    }
+    if (k_weight != nullptr) {
+      float ss = pairs_sum_of_squares(a, b);
+#pragma unroll
+      for (int off = LPH / 2; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+      float wa[8], wb[8];
+      load_weights8<W>(k_weight + 8 * c, wa);
+      load_weights8<W>(k_weight + HALF + 8 * c, wb);
+      pairs_normalise(a, b, head_norm_scale(ss, D, eps), wa, wb);
+    }
+    if (table_row != nullptr) {
+      float cs[8], sn[8];
+      load_weights8<float>(table_row + 8 * c, cs);
+      load_weights8<float>(table_row + HALF + 8 * c, sn);
+      pairs_rotate(a, b, cs, sn);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      x1.e[i] = float_to_bf16(a[i]);
+      x2.e[i] = float_to_bf16(b[i]);
+    }
+    bf16_t* dst = k_cache + (((size_t)pg * Hkv + g_kv) * page + slot) * D;
+    *reinterpret_cast<uint4*>(dst + 8 * c) = x1.u;
+    *reinterpret_cast<uint4*>(dst + HALF + 8 * c) = x2.u;
+  } else if (t >= 64 && t < 64 + LPH) {
+    const int c = t - 64;
+    const bf16_t* src = row + (size_t)(Hq + Hkv + g_kv) * D;
+    Half8 x1, x2;
+    x1.u = *reinterpret_cast<const uint4*>(src + 8 * c);
+    x2.u = *reinterpret_cast<const uint4*>(src + HALF + 8 * c);
+    bf16_t* o = v_cache + ((size_t)pg * Hkv + g_kv) * D * page + slot;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      o[(size_t)(8 * c + i) * page] = x1.e[i];
+      o[(size_t)(HALF + 8 * c + i) * page] = x2.e[i];
+    }
+  }
+}
+
+template <int D, bool PREP, typename W>
 __global__ __launch_bounds__(256) void attn_decode_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, int num_pages, const int* __restrict__ block_table, int bt_stride,
     const int* __restrict__ cu_q, const int* __restrict__ kv_lens, int Hq, int Hkv, int page, float scale_log2,
-    int window, int splits, float* __restrict__ ws_acc, float* __restrict__ ws_ml) {
+    int window, int splits, float* __restrict__ ws_acc, float* __restrict__ ws_ml, DecodePrep prep) {
   const int b = blockIdx.z, g_kv = blockIdx.y, split = blockIdx.x;
   const int G = Hq / Hkv;
   const int q0 = cu_q[b];
   const int q_len = cu_q[b + 1] - q0;
   if (q_len <= 0 || q_len * G > 16) return;  // the other kernel's sequence
+  if (PREP && q_len != 1) return;            // the host sends single tokens only
   const int kv_len = kv_lens[b];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, grp = lane >> 4;
   const int rows = q_len * G;
   const int first_pos = kv_len - q_len;
+  const int* bt_row = block_table + (size_t)b * bt_stride;
+
+  int tile_lo = 0;
+  if (window > 0) tile_lo = max(0, first_pos - window + 1) / FAST_TILE;
+  const int tile_hi = (kv_len + FAST_TILE - 1) / FAST_TILE;
+  const int per_split = (tile_hi - tile_lo + splits - 1) / splits;
+  const int t0 = tile_lo + split * per_split;
+  const int t1 = min(tile_hi, t0 + per_split);
 
   int row_pos[1];
   row_pos[0] = col < rows ? first_pos + col / G : -1;
@@ -401,18 +533,24 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     else
       qreg[0][i].u = make_uint4(0, 0, 0, 0);
   }
+  if constexpr (PREP) {
+    const float* table_row =
+        (prep.table != nullptr && first_pos >= 0 && first_pos < prep.max_pos) ? prep.table + (size_t)first_pos * D : nullptr;
+    if (prep.k_cache != nullptr && first_pos >= 0 && t0 <= tile_hi - 1 && tile_hi - 1 < t1) {  // uniform in the block
+      const int blk = first_pos / page;
+      const int pg = blk < bt_stride ? bt_row[blk] : -1;
+      if (pg >= 0 && pg < num_pages)
+        store_new_key_value<D, W>(q + (size_t)q0 * q_stride, Hq, Hkv, g_kv, static_cast<const W*>(prep.k_weight),
+                                  prep.eps, table_row, prep.k_cache, prep.v_cache, pg, page, first_pos % page);
+      __syncthreads();
+    }
+    prepare_query<D, W>(qreg[0], static_cast<const W*>(prep.q_weight), prep.eps, table_row, grp);
+  }
   f32x4_t acc[1][D / 16];
 #pragma unroll
   for (int nb = 0; nb < D / 16; ++nb) acc[0][nb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   float m_run[1] = {-INFINITY}, l_run[1] = {0.f};
 
-  int tile_lo = 0;
-  if (window > 0) tile_lo = max(0, first_pos - window + 1) / FAST_TILE;
-  const int tile_hi = (kv_len + FAST_TILE - 1) / FAST_TILE;
-  const int per_split = (tile_hi - tile_lo + splits - 1) / splits;
-  const int t0 = tile_lo + split * per_split;
-  const int t1 = min(tile_hi, t0 + per_split);
-  const int* bt_row = block_table + (size_t)b * bt_stride;
   attend_tiles<D, 1>(qreg, k_cache, v_cache, num_pages, bt_row, Hkv, g_kv, page, t0 + wave, t1, 4, kv_len, row_pos,
                      window, scale_log2, acc, m_run, l_run);
 
@@ -844,9 +982,10 @@ static int launch_fast(const void* q, int q_stride, void* out, const void* k_cac
   const int G = Hq / Hkv;
   const float scale_log2 = scale * 1.4426950408889634f;
   if (min_q_len * G <= 16) {
-    hipLaunchKernelGGL(attn_decode_kernel<D>, dim3(splits, Hkv, B), dim3(256), 0, stream, (const bf16_t*)q, q_stride,
-                       (bf16_t*)out, (const bf16_t*)k_cache, (const bf16_t*)v_cache, num_pages, block_table,
-                       bt_stride, cu_q, kv_lens, Hq, Hkv, page, scale_log2, window, splits, ws_acc, ws_ml);
+    hipLaunchKernelGGL((attn_decode_kernel<D, false, float>), dim3(splits, Hkv, B), dim3(256), 0, stream,
+                       (const bf16_t*)q, q_stride, (bf16_t*)out, (const bf16_t*)k_cache, (const bf16_t*)v_cache,
+                       num_pages, block_table, bt_stride, cu_q, kv_lens, Hq, Hkv, page, scale_log2, window, splits,
+                       ws_acc, ws_ml, DecodePrep{});
     if (splits > 1)
       hipLaunchKernelGGL(attn_decode_reduce_kernel<D>, dim3(Hkv, B), dim3(256), 0, stream, (bf16_t*)out, cu_q, Hq,
                          Hkv, splits, ws_acc, ws_ml);
@@ -858,6 +997,22 @@ static int launch_fast(const void* q, int q_stride, void* out, const void* k_cac
                        (bf16_t*)out, (const bf16_t*)k_cache, (const bf16_t*)v_cache, num_pages, block_table,
                        bt_stride, cu_q, kv_lens, Hq, Hkv, page, scale_log2, window, tokens_per_block);
   }
+  return q3_launch_status();
+}
+
+template <int D, typename W>
+static int launch_decode_prep(const void* qkv, void* out, const void* k_cache, const void* v_cache, int num_pages,
+                              const int* block_table, int bt_stride, const int* cu_q, const int* kv_lens, int B,
+                              int Hq, int Hkv, int page, float scale, int window, int splits, float* ws_acc,
+                              float* ws_ml, const DecodePrep& prep, hipStream_t stream) {
+  const float scale_log2 = scale * 1.4426950408889634f;
+  hipLaunchKernelGGL((attn_decode_kernel<D, true, W>), dim3(splits, Hkv, B), dim3(256), 0, stream,
+                     (const bf16_t*)qkv, (Hq + 2 * Hkv) * D, (bf16_t*)out, (const bf16_t*)k_cache,
+                     (const bf16_t*)v_cache, num_pages, block_table, bt_stride, cu_q, kv_lens, Hq, Hkv, page,
+                     scale_log2, window, splits, ws_acc, ws_ml, prep);
+  if (splits > 1)
+    hipLaunchKernelGGL(attn_decode_reduce_kernel<D>, dim3(Hkv, B), dim3(256), 0, stream, (bf16_t*)out, cu_q, Hq, Hkv,
+                       splits, ws_acc, ws_ml);
   return q3_launch_status();
 }
 
@@ -901,4 +1056,49 @@ extern "C" int q3_paged_attention(const void* q, int q_stride, void* out, const 
                                                         block_table, bt_stride, cu_q, kv_lens, B, Hq, Hkv,
                                                         D, page, scale, window, max_q_len, stream));
   return Q3_ERR_BAD_ARGUMENT;
+}
+
+// Whether `q3_decode_attention` takes a step of single tokens with these sizes: what the
+// matrix-core kernels take, with a rotation (if any) over the whole head.
+extern "C" int q3_decode_attention_takes(int Hq, int Hkv, int D, int page, int dtype, int rotary_dim) {
+  return q3_paged_attention_fast_path(Hq, Hkv, D, page, dtype) && (rotary_dim == 0 || rotary_dim == D);
+}
+
+// A step in which every sequence brings one token, from the raw projections: qkv (B, (Hq +
+// 2 Hkv) D) bfloat16 holds [q | k | v] of token b in row b (cu_q[b] = b). Per-head RMSNorm
+// of q and k (weights of `w_dtype`, both or neither), rotation by `table` (or null), the new
+// key and value written to the caches at position kv_lens[b] - 1 (if `store`), and attention
+// over the cache, in one kernel and the merge of its splits. out (B, Hq D) bfloat16.
+extern "C" int q3_decode_attention(const void* qkv, void* out, void* k_cache, void* v_cache, int num_pages,
+                                   const int* block_table, int bt_stride, const int* cu_q, const int* kv_lens,
+                                   int B, int Hq, int Hkv, int D, int page, float scale, int window, int splits,
+                                   float* workspace, const void* q_weight, const void* k_weight, int w_dtype,
+                                   float eps, const float* table, int rotary_dim, int max_pos, int store,
+                                   hipStream_t stream) {
+  if (B <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || page <= 0) return Q3_ERR_BAD_ARGUMENT;
+  if (B > 65535) return Q3_ERR_UNSUPPORTED;
+  if (!q3_decode_attention_takes(Hq, Hkv, D, page, Q3_BF16, table ? rotary_dim : 0)) return Q3_ERR_UNSUPPORTED;
+  if ((q_weight == nullptr) != (k_weight == nullptr)) return Q3_ERR_BAD_ARGUMENT;
+  if (q_weight && w_dtype != Q3_F32 && w_dtype != Q3_BF16) return Q3_ERR_BAD_ARGUMENT;
+  if (splits < 1 || splits > MAX_SPLITS || (splits > 1 && workspace == nullptr)) return Q3_ERR_BAD_ARGUMENT;
+  float* ws_acc = workspace;
+  float* ws_ml = workspace ? workspace + (size_t)B * Hkv * splits * 16 * D : nullptr;
+  DecodePrep prep{};
+  prep.q_weight = q_weight;
+  prep.k_weight = k_weight;
+  prep.eps = eps;
+  prep.table = table;
+  prep.max_pos = max_pos;
+  prep.k_cache = store ? (bf16_t*)k_cache : nullptr;
+  prep.v_cache = store ? (bf16_t*)v_cache : nullptr;
+#define Q3_DECODE_PREP(DD, WW)                                                                                    \
+  return launch_decode_prep<DD, WW>(qkv, out, k_cache, v_cache, num_pages, block_table, bt_stride, cu_q, kv_lens, \
+                                    B, Hq, Hkv, page, scale, window, splits, ws_acc, ws_ml, prep, stream)
+  if (D == 64) {
+    if (w_dtype == Q3_F32) Q3_DECODE_PREP(64, float);
+    Q3_DECODE_PREP(64, bf16_t);
+  }
+  if (w_dtype == Q3_F32) Q3_DECODE_PREP(128, float);
+  Q3_DECODE_PREP(128, bf16_t);
+#undef Q3_DECODE_PREP
 }

@@ -1,6 +1,7 @@
 // Rotary position encoding: the [cos | sin] table, and the fused pass over a
 // step's qkv rows: per-head RMSNorm of q and k, rotation, and the cache write.
 #include "common.h"
+#include "qk_prepare.h"
 
 // table[p, i] = cos(p * inv_freq[i]), table[p, half + i] = sin(p * inv_freq[i]).
 // The angle is the float32 product, as a float32 outer product would give it;
@@ -126,26 +127,6 @@ __global__ void qk_norm_rope_store_kernel(T* __restrict__ qkv, const W* __restri
 // that pair with them in the second half; values are transposed page by page
 // through shared memory by a second kernel.
 // ---------------------------------------------------------------------------
-union Half8 {
-  uint4 u;
-  bf16_t e[8];
-};
-
-template <typename W>
-__device__ inline void load_weights8(const W* w, float (&o)[8]);
-template <>
-__device__ inline void load_weights8<float>(const float* w, float (&o)[8]) {
-  const float4 a = *reinterpret_cast<const float4*>(w), b = *reinterpret_cast<const float4*>(w + 4);
-  o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w; o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
-}
-template <>
-__device__ inline void load_weights8<bf16_t>(const bf16_t* w, float (&o)[8]) {
-  Half8 h;
-  h.u = *reinterpret_cast<const uint4*>(w);
-#pragma unroll
-  for (int i = 0; i < 8; ++i) o[i] = bf16_to_float(h.e[i]);
-}
-
 // grid (T, ceil(heads / heads_per_block)), 256 threads; LPH = D / 16 lanes per head. With
 // STORE_V the value heads are handled here too, element by element into the transposed
 // cache (for steps of few tokens, where a second launch would cost more than it saves).
@@ -181,38 +162,26 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_vec_kernel(
     return;
   }
   float a[8], b[8];
-  float ss = 0.f;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     a[i] = bf16_to_float(x1.e[i]);
     b[i] = bf16_to_float(x2.e[i]);
-    ss += a[i] * a[i] + b[i] * b[i];
   }
   const W* w = head < Hq ? q_weight : k_weight;
   if (w != nullptr) {
+    float ss = pairs_sum_of_squares(a, b);
 #pragma unroll
     for (int off = LPH / 2; off > 0; off >>= 1) ss += __shfl_xor(ss, off, Q3_WAVE);
-    const float scale = rsqrtf(ss / (float)D + eps);
     float wa[8], wb[8];
     load_weights8<W>(w + 8 * c, wa);
     load_weights8<W>(w + HALF + 8 * c, wb);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      a[i] = a[i] * scale * wa[i];
-      b[i] = b[i] * scale * wb[i];
-    }
+    pairs_normalise(a, b, head_norm_scale(ss, D, eps), wa, wb);
   }
   if (table != nullptr && pos >= 0 && pos < max_pos) {
     float cs[8], sn[8];
     load_weights8<float>(table + (size_t)pos * D + 8 * c, cs);
     load_weights8<float>(table + (size_t)pos * D + HALF + 8 * c, sn);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const float ya = a[i] * cs[i] - b[i] * sn[i];
-      const float yb = b[i] * cs[i] + a[i] * sn[i];
-      a[i] = ya;
-      b[i] = yb;
-    }
+    pairs_rotate(a, b, cs, sn);
   }
   bf16_t* dst = src;
   if (head >= Hq) {

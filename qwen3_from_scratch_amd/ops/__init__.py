@@ -25,6 +25,8 @@ __all__ = [
     "rope_table",
     "qk_norm_rope_store",
     "paged_attention",
+    "decode_attention",
+    "decode_attention_takes",
     "swiglu",
     "linear",
     "linear_swiglu",
@@ -250,9 +252,7 @@ def paged_attention(q, num_q_heads, k_cache, v_cache, block_table, cu_seqlens_q,
         lib = library("attention")
         splits, workspace = 1, None
         if lib.q3_paged_attention_fast_path(Hq, Hkv, D, page, _DT[q.dtype]) and min_q_len * (Hq // Hkv) <= 16:
-            # few rows per sequence: split the keys over blocks until the chip is full (about two
-            # blocks a compute unit; beyond 32 parts the merge costs more than the split gains)
-            splits = max(1, min(max_kv_len // 64, -(-512 // (B * Hkv)), 32))
+            splits = _splits(B, Hkv, max_kv_len)       # few rows per sequence: the keys go over several blocks
             if splits > 1:
                 lib.q3_paged_attention_workspace.restype = ctypes.c_long
                 n = lib.q3_paged_attention_workspace(B, Hkv, D, splits)
@@ -262,6 +262,67 @@ def paged_attention(q, num_q_heads, k_cache, v_cache, block_table, cu_seqlens_q,
             _ptr(block_table), block_table.shape[1], _ptr(cu_seqlens_q), _ptr(kv_lens),
             B, T, Hq, Hkv, D, page, ctypes.c_float(scale), int(window), int(max_q_len), int(min_q_len),
             int(max_kv_len), _DT[q.dtype], splits, _ptr(workspace), _stream()), "paged_attention")
+    return out
+
+
+def _splits(B, Hkv, max_kv_len):
+    """Into how many blocks a sequence's keys are split when a step has few rows per sequence:
+    until the chip is full, about two blocks a compute unit; beyond 32 parts the merge costs
+    more than the split gains."""
+    return max(1, min(max_kv_len // 64, -(-512 // (B * Hkv)), 32))
+
+
+def decode_attention_takes(num_q_heads, num_kv_heads, head_dim, page_size, dtype, rotary_dim=0):
+    """Whether `decode_attention` serves these sizes (the caller then skips `qk_norm_rope_store`)."""
+    if dtype != torch.bfloat16:
+        return False
+    return bool(library("attention").q3_decode_attention_takes(
+        num_q_heads, num_kv_heads, head_dim, page_size, _DT[dtype], int(rotary_dim)))
+
+
+def decode_attention(qkv, num_q_heads, num_kv_heads, head_dim, k_cache, v_cache, block_table, cu_seqlens_q,
+                     kv_lens, max_kv_len, scale, window=0, q_weight=None, k_weight=None, eps=0.0, table=None,
+                     store=True):
+    """`qk_norm_rope_store` and `paged_attention` of a step in which every sequence brings one
+    token, in one kernel: qkv (B, (Hq + 2 Hkv) D) bfloat16 holds the raw projections of
+    sequence b's token in row b; the new key and value go to position kv_lens[b] - 1 of the
+    caches (unless `store` is false: a layer that reads another layer's cache) and the
+    attention output (B, Hq D) is returned. qkv is left as it was."""
+    _dev(qkv, k_cache, v_cache, block_table, cu_seqlens_q, kv_lens, q_weight, k_weight, table)
+    Hq, Hkv, D = num_q_heads, num_kv_heads, head_dim
+    B = kv_lens.shape[0]
+    _need(qkv.dtype == torch.bfloat16 and qkv.shape == (B, (Hq + 2 * Hkv) * D), "qkv must be bfloat16 (B, (Hq + 2 Hkv) D)")
+    _need(k_cache.dtype == torch.bfloat16 and v_cache.dtype == torch.bfloat16 and k_cache.dim() == 4
+          and k_cache.shape[1] == Hkv and k_cache.shape[3] == D, "key cache must be bfloat16 (pages, Hkv, page, D)")
+    page = k_cache.shape[2]
+    _need(v_cache.shape == (k_cache.shape[0], Hkv, D, page), "value cache must be (pages, Hkv, D, page)")
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.shape[0] >= B, "block table int32 (B, blocks)")
+    _need(cu_seqlens_q.dtype == torch.int32 and cu_seqlens_q.shape == (B + 1,), "cu_seqlens_q int32 (B + 1,)")
+    _need(kv_lens.dtype == torch.int32, "kv_lens int32 (B,)")
+    _need((q_weight is None) == (k_weight is None), "q and k norm weights come together")
+    w_dtype = 0
+    if q_weight is not None:
+        _need(q_weight.shape == (D,) and k_weight.shape == (D,) and q_weight.dtype == k_weight.dtype
+              and q_weight.dtype in _DT, "norm weights (D,) of one dtype")
+        w_dtype = _DT[q_weight.dtype]
+    rotary_dim = max_pos = 0
+    if table is not None:
+        _need(table.dtype == torch.float32 and table.dim() == 2, "rotation table float32 (positions, rotary_dim)")
+        max_pos, rotary_dim = table.shape
+    _need(decode_attention_takes(Hq, Hkv, D, page, qkv.dtype, rotary_dim), "sizes the decoding kernel does not take")
+    out = torch.empty((B, Hq * D), dtype=qkv.dtype, device=qkv.device)
+    if B:
+        lib = library("attention")
+        splits, workspace = _splits(B, Hkv, max_kv_len), None
+        if splits > 1:
+            lib.q3_paged_attention_workspace.restype = ctypes.c_long
+            workspace = torch.empty((lib.q3_paged_attention_workspace(B, Hkv, D, splits),), dtype=torch.float32,
+                                    device=qkv.device)
+        _check(lib.q3_decode_attention(
+            _ptr(qkv), _ptr(out), _ptr(k_cache), _ptr(v_cache), k_cache.shape[0], _ptr(block_table),
+            block_table.shape[1], _ptr(cu_seqlens_q), _ptr(kv_lens), B, Hq, Hkv, D, page, ctypes.c_float(scale),
+            int(window), splits, _ptr(workspace), _ptr(q_weight), _ptr(k_weight), w_dtype, ctypes.c_float(eps),
+            _ptr(table), int(rotary_dim), int(max_pos), 1 if store else 0, _stream()), "decode_attention")
     return out
 
 

@@ -86,6 +86,14 @@ class PagedAttention(Part):
         Hq, Hkv, D = self.num_heads, self.num_kv_heads, self.head_dim
         qkv = self.qkv.forward(x)
         table = self.position.rotation_table() if self.position is not None else None
+        if batch.max_q_len == 1 and qkv.shape[0] == batch.kv_lens.shape[0] and ops.decode_attention_takes(
+                Hq, Hkv, D, cache.keys.shape[2], qkv.dtype, 0 if table is None else table.shape[1]):
+            # every sequence brings one token: preparation, cache write and attention are one kernel
+            o = ops.decode_attention(
+                qkv, Hq, Hkv, D, cache.keys, cache.values, cache.block_table, batch.cu_seqlens_q, batch.kv_lens,
+                batch.max_kv_len, self.scale, window=self.window, q_weight=self.q_weight, k_weight=self.k_weight,
+                eps=self.qk_norm_eps, table=table, store=cache.writes)
+            return self.out.forward(o) if sink is None else self.out.forward_into(o, sink)
         ops.qk_norm_rope_store(
             qkv, Hq, Hkv, D, batch.positions, batch.seq_index,
             q_weight=self.q_weight, k_weight=self.k_weight, eps=self.qk_norm_eps, table=table,

@@ -206,6 +206,52 @@ def test_paged_attention_decoding_batches(Hq, Hkv, D, page, window):
         torch.testing.assert_close(got.float(), want, rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("Hq,Hkv,D,page", [(32, 8, 128, 16), (16, 2, 64, 16), (14, 2, 64, 64), (9, 3, 128, 32),
+                                           (16, 1, 128, 16)])
+@pytest.mark.parametrize("w_dtype", [torch.float32, torch.bfloat16, None])
+@pytest.mark.parametrize("window,rotate,store", [(0, True, True), (23, True, True), (0, False, True), (0, True, False)])
+def test_decode_attention_is_its_two_halves(Hq, Hkv, D, page, w_dtype, window, rotate, store):
+    """A step of single tokens in one kernel gives, to the bit, what the preparation kernel
+    followed by the attention kernel gives: the prepared queries and keys, the caches after
+    the step, and the output. Lengths are chosen so that the new key is a page's first and
+    last slot, a tile's first key, and far into many splits."""
+    ops = _ops()
+    kv_lens = [1, page, page + 1, 33, 64, 65, 700, 2500]
+    B = len(kv_lens)
+    _, kc, vc, bt, cu, kvl = _paged_case(torch.bfloat16, B, Hq, Hkv, D, page, [1] * B, kv_lens, 77)
+    qkv = _rand((B, (Hq + 2 * Hkv) * D), torch.bfloat16, 78, scale=1.5)
+    qw = kw = None
+    if w_dtype is not None:
+        qw = (1.0 + _rand((D,), torch.float32, 79, scale=0.3)).to(w_dtype)
+        kw = (1.0 + _rand((D,), torch.float32, 80, scale=0.3)).to(w_dtype)
+    inv_freq = (1.0 / (10000.0 ** (torch.arange(0, D, 2, dtype=torch.float32) / D))).cuda()
+    table = ops.rope_table(inv_freq, 4096) if rotate else None
+    positions = (kvl - 1).to(torch.int32)
+    seq_index = torch.arange(B, dtype=torch.int32, device="cuda")
+    scale = D ** -0.5
+    assert ops.decode_attention_takes(Hq, Hkv, D, page, torch.bfloat16, D if rotate else 0)
+
+    k1, v1, qkv1 = kc.clone(), vc.clone(), qkv.clone()
+    ops.qk_norm_rope_store(qkv1, Hq, Hkv, D, positions, seq_index, q_weight=qw, k_weight=kw, eps=1e-6, table=table,
+                           block_table=bt if store else None, k_cache=k1 if store else None,
+                           v_cache=v1 if store else None, cu_seqlens_q=cu, kv_lens=kvl, max_q_len=1)
+    q = qkv1[:, : Hq * D].unflatten(1, (Hq, D))
+    want = ops.paged_attention(q, Hq, k1, v1, bt, cu, kvl, 1, max(kv_lens), scale, window=window)
+
+    k2, v2, qkv2 = kc.clone(), vc.clone(), qkv.clone()
+    got = ops.decode_attention(qkv2, Hq, Hkv, D, k2, v2, bt, cu, kvl, max(kv_lens), scale, window=window,
+                               q_weight=qw, k_weight=kw, eps=1e-6, table=table, store=store)
+    assert torch.equal(qkv2, qkv)                              # the raw projections are left alone
+    assert torch.equal(k2, k1) and torch.equal(v2, v1)
+    if not store:
+        assert torch.equal(k2, kc) and torch.equal(v2, vc)
+    assert torch.equal(got, want)
+    # and against plain arithmetic
+    ref = torch_ops.paged_attention(q.float(), Hq, k1.float(), v1.float(), bt, cu, kvl, 1, max(kv_lens), scale,
+                                    window=window)
+    torch.testing.assert_close(got.float().view(B, Hq, D), ref.view(B, Hq, D), rtol=2e-2, atol=2e-2)
+
+
 def test_paged_attention_portions_over_long_prefixes():
     """Portions of prompts with hundreds of cached keys before them, beside single tokens."""
     ops = _ops()

@@ -124,6 +124,10 @@ def paged_attention(q, num_q_heads, k_cache, v_cache, block_table, cu_seqlens_q,
     return res
 
 
+def decode_attention_takes(*args, **kwargs):
+    return False            # the fused decoding kernel has no twin: its two halves above are the reference
+
+
 def tile_weight(weight):
     return None
 
@@ -170,4 +174,4 @@ def sample(logits, temperature, top_k, seed, counter, out=None):
 
 
 ALL = ("embed_rows", "swiglu", "rmsnorm", "rope_table", "qk_norm_rope_store",
-       "paged_attention", "linear", "linear_swiglu", "tile_weight", "sample")
+       "paged_attention", "decode_attention_takes", "linear", "linear_swiglu", "tile_weight", "sample")

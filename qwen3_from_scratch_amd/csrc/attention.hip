@@ -340,18 +340,31 @@ __device__ __forceinline__ void attend_tile(const Pack16 (&qreg)[QB][D / 32], co
 }
 
 // All tiles first, first + step, ... below last for one wavefront: the value loads of a
-// tile and the key loads of the next one are issued before the tile's arithmetic.
+// tile and the key loads of the next one are issued before the tile's arithmetic. The
+// first tile's keys are loaded by the caller (`first_tile_keys`), who may have other work
+// to do while they travel.
+template <int D>
+__device__ __forceinline__ TileAddr first_tile_keys(Pack16 (&a_cur)[2][D / 32], const bf16_t* __restrict__ k_cache,
+                                                    const bf16_t* __restrict__ v_cache, int num_pages,
+                                                    const int* __restrict__ bt_row, int Hkv, int g_kv, int page,
+                                                    int first, int last, int kv_len) {
+  TileAddr t{};
+  if (first >= last) return t;
+  t = tile_addr(k_cache, v_cache, num_pages, bt_row, Hkv, g_kv, page, D, first * FAST_TILE, kv_len);
+  load_keys<D>(a_cur, t);
+  return t;
+}
+
 template <int D, int QB>
-__device__ __forceinline__ void attend_tiles(const Pack16 (&qreg)[QB][D / 32], const bf16_t* __restrict__ k_cache,
+__device__ __forceinline__ void attend_tiles(const Pack16 (&qreg)[QB][D / 32], Pack16 (&a_cur)[2][D / 32],
+                                             TileAddr t_cur, const bf16_t* __restrict__ k_cache,
                                              const bf16_t* __restrict__ v_cache, int num_pages,
                                              const int* __restrict__ bt_row, int Hkv, int g_kv, int page, int first,
                                              int last, int step, int kv_len, const int (&row_pos)[QB], int window,
                                              float scale_log2, f32x4_t (&acc)[QB][D / 16], float (&m_run)[QB],
                                              float (&l_run)[QB]) {
   if (first >= last) return;
-  Pack16 a_cur[2][D / 32], a_nxt[2][D / 32], vt[D / 16];
-  TileAddr t_cur = tile_addr(k_cache, v_cache, num_pages, bt_row, Hkv, g_kv, page, D, first * FAST_TILE, kv_len);
-  load_keys<D>(a_cur, t_cur);
+  Pack16 a_nxt[2][D / 32], vt[D / 16];
   for (int t = first; t < last; t += step) {
     load_values<D>(vt, t_cur, page);
     const bool more = t + step < last;
@@ -376,10 +389,13 @@ __device__ __forceinline__ void attend_tiles(const Pack16 (&qreg)[QB][D / 32], c
 // result (maximum, sum, accumulator) in the workspace for the reduction kernel.
 // With PREP the kernel also does what the preparation kernel does for a step of single
 // tokens (q_len = 1 everywhere): `q` is then the step's raw [q | k | v] rows. Every block
-// normalises and rotates its own query rows on the way into the registers; the block whose
-// share of the keys holds the sequence's last position first normalises and rotates the new
-// key, writes it and the new value into the cache (if `prep.store`), and waits at a barrier
-// before any of its wavefronts reads keys: a block's own writes are visible to it after that.
+// normalises and rotates its own query rows on the way into the registers. If the step's
+// key and value are to be stored (`prep.k_cache`), the block of the last split (the one
+// with the fewest tiles) normalises and rotates the new key, writes it and the new value
+// into the cache for later steps, and adds the new key's share of the result itself, from
+// shared memory (one score per row, the value as it is) when it merges its wavefronts. No
+// block reads the new position from the cache: they read what earlier steps wrote, so no
+// read waits for a write.
 struct DecodePrep {
   const void* q_weight;  // (D,) or null: no norm
   const void* k_weight;
@@ -437,17 +453,20 @@ __device__ __forceinline__ void prepare_query(Pack16 (&qreg)[D / 32], const W* w
     }
 }
 
-// The new key of head g_kv (threads 0 .. D / 16 - 1, as the preparation kernel's lanes) and
-// the new value (threads 64 .. 64 + D / 16 - 1) of the token whose raw row is `row`, into
-// slot pos % page of `pg`.
+// The new key of head g_kv (the first D / 16 lanes of the block's last wavefront, as the
+// preparation kernel's lanes) and the new value (the first D / 16 lanes of the wavefront
+// before it) of the token whose raw row is `row`, into
+// slot pos % page of `pg` (if there is such a page) and, as the cache's rounded numbers, into
+// shared memory.
 template <int D, typename W>
 __device__ __forceinline__ void store_new_key_value(const bf16_t* row, int Hq, int Hkv, int g_kv, const W* k_weight,
                                                     float eps, const float* table_row, bf16_t* k_cache,
-                                                    bf16_t* v_cache, int pg, int page, int slot) {
+                                                    bf16_t* v_cache, int pg, int page, int slot, float* sh_k,
+                                                    float* sh_v) {
   constexpr int LPH = D / 16, HALF = D / 2;
   const int t = threadIdx.x;
-  if (t < LPH) {
-    const int c = t;
+  if (t >= 192 && t < 192 + LPH) {
+    const int c = t - 192;
     const bf16_t* src = row + (size_t)(Hq + g_kv) * D;
     Half8 x1, x2;
     x1.u = *reinterpret_cast<const uint4*>(src + 8 * c);
@@ -477,21 +496,32 @@ __device__ __forceinline__ void store_new_key_value(const bf16_t* row, int Hq, i
     for (int i = 0; i < 8; ++i) {
       x1.e[i] = float_to_bf16(a[i]);
       x2.e[i] = float_to_bf16(b[i]);
+      sh_k[8 * c + i] = bf16_to_float(x1.e[i]);
+      sh_k[HALF + 8 * c + i] = bf16_to_float(x2.e[i]);
     }
-    bf16_t* dst = k_cache + (((size_t)pg * Hkv + g_kv) * page + slot) * D;
-    *reinterpret_cast<uint4*>(dst + 8 * c) = x1.u;
-    *reinterpret_cast<uint4*>(dst + HALF + 8 * c) = x2.u;
-  } else if (t >= 64 && t < 64 + LPH) {
-    const int c = t - 64;
+    if (pg >= 0) {
+      bf16_t* dst = k_cache + (((size_t)pg * Hkv + g_kv) * page + slot) * D;
+      *reinterpret_cast<uint4*>(dst + 8 * c) = x1.u;
+      *reinterpret_cast<uint4*>(dst + HALF + 8 * c) = x2.u;
+    }
+  } else if (t >= 128 && t < 128 + LPH) {
+    const int c = t - 128;
     const bf16_t* src = row + (size_t)(Hq + Hkv + g_kv) * D;
     Half8 x1, x2;
     x1.u = *reinterpret_cast<const uint4*>(src + 8 * c);
     x2.u = *reinterpret_cast<const uint4*>(src + HALF + 8 * c);
-    bf16_t* o = v_cache + ((size_t)pg * Hkv + g_kv) * D * page + slot;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      o[(size_t)(8 * c + i) * page] = x1.e[i];
-      o[(size_t)(HALF + 8 * c + i) * page] = x2.e[i];
+      sh_v[8 * c + i] = bf16_to_float(x1.e[i]);
+      sh_v[HALF + 8 * c + i] = bf16_to_float(x2.e[i]);
+    }
+    if (pg >= 0) {
+      bf16_t* o = v_cache + ((size_t)pg * Hkv + g_kv) * D * page + slot;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        o[(size_t)(8 * c + i) * page] = x1.e[i];
+        o[(size_t)(HALF + 8 * c + i) * page] = x2.e[i];
+      }
     }
   }
 }
@@ -514,16 +544,16 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   const int rows = q_len * G;
   const int first_pos = kv_len - q_len;
   const int* bt_row = block_table + (size_t)b * bt_stride;
+  // the new key is not in the cache yet: the last split's block brings it
+  const bool fresh = PREP && prep.k_cache != nullptr;
+  const bool brings_new = fresh && split == splits - 1;  // uniform in the block
+  const float* table_row = nullptr;
+  if constexpr (PREP) {
+    if (first_pos < 0) return;
+    if (prep.table != nullptr && first_pos < prep.max_pos) table_row = prep.table + (size_t)first_pos * D;
+  }
+  __shared__ float sh_k[PREP ? D : 1], sh_v[PREP ? D : 1];
 
-  int tile_lo = 0;
-  if (window > 0) tile_lo = max(0, first_pos - window + 1) / FAST_TILE;
-  const int tile_hi = (kv_len + FAST_TILE - 1) / FAST_TILE;
-  const int per_split = (tile_hi - tile_lo + splits - 1) / splits;
-  const int t0 = tile_lo + split * per_split;
-  const int t1 = min(tile_hi, t0 + per_split);
-
-  int row_pos[1];
-  row_pos[0] = col < rows ? first_pos + col / G : -1;
   Pack16 qreg[1][D / 32];
 #pragma unroll
   for (int i = 0; i < D / 32; ++i) {
@@ -533,40 +563,74 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     else
       qreg[0][i].u = make_uint4(0, 0, 0, 0);
   }
+
+  // with a fresh key the cache is read up to the position before it: the rows then stand one
+  // position earlier for the masks, and the window, which counts the new key, is one shorter
+  const int kv_seen = fresh ? kv_len - 1 : kv_len;
+  const int win = (fresh && window > 0) ? window - 1 : window;
+  int row_pos[1];
+  row_pos[0] = col < rows ? first_pos + col / G - (fresh ? 1 : 0) : -1;
+  int tile_lo = 0;
+  if (window > 0) tile_lo = max(0, first_pos - window + 1) / FAST_TILE;
+  int tile_hi = (kv_seen + FAST_TILE - 1) / FAST_TILE;
+  if (fresh && window == 1) tile_hi = tile_lo;  // the new key alone is visible
+  const int per_split = (max(tile_hi - tile_lo, 0) + splits - 1) / splits;
+  const int t0 = tile_lo + split * per_split;
+  const int t1 = min(tile_hi, t0 + per_split);
+  // the first tile's keys are on their way while the query rows are prepared
+  Pack16 a_first[2][D / 32];
+  const TileAddr t_first = first_tile_keys<D>(a_first, k_cache, v_cache, num_pages, bt_row, Hkv, g_kv, page, t0 + wave,
+                                              t1, kv_seen);
+  float m_new = -INFINITY;  // in the last wavefront: the new key's score for this lane's row
   if constexpr (PREP) {
-    const float* table_row =
-        (prep.table != nullptr && first_pos >= 0 && first_pos < prep.max_pos) ? prep.table + (size_t)first_pos * D : nullptr;
-    if (prep.k_cache != nullptr && first_pos >= 0 && t0 <= tile_hi - 1 && tile_hi - 1 < t1) {  // uniform in the block
-      const int blk = first_pos / page;
-      const int pg = blk < bt_stride ? bt_row[blk] : -1;
-      if (pg >= 0 && pg < num_pages)
-        store_new_key_value<D, W>(q + (size_t)q0 * q_stride, Hq, Hkv, g_kv, static_cast<const W*>(prep.k_weight),
-                                  prep.eps, table_row, prep.k_cache, prep.v_cache, pg, page, first_pos % page);
-      __syncthreads();
-    }
     prepare_query<D, W>(qreg[0], static_cast<const W*>(prep.q_weight), prep.eps, table_row, grp);
+    if (brings_new) {
+      // the last two wavefronts, which have the fewest tiles, lend a few lanes: the key and the
+      // value into the cache for later steps, and into shared memory for this one (the value
+      // is read after the barriers of the merge, the key by the wavefront that wrote it)
+      const int blk = first_pos / page;
+      int pg = blk < bt_stride ? bt_row[blk] : -1;
+      if (pg >= num_pages) pg = -1;
+      store_new_key_value<D, W>(q + (size_t)q0 * q_stride, Hq, Hkv, g_kv, static_cast<const W*>(prep.k_weight),
+                                prep.eps, table_row, prep.k_cache, prep.v_cache, pg, page, first_pos % page, sh_k,
+                                sh_v);
+      if (wave == 3) {
+        float dot = 0.f;
+#pragma unroll
+        for (int i = 0; i < D / 32; ++i)
+#pragma unroll
+          for (int j = 0; j < 8; ++j) dot = fmaf((float)qreg[0][i].e[j], sh_k[32 * i + 8 * grp + j], dot);
+        dot += __shfl_xor(dot, 16, 64);
+        dot += __shfl_xor(dot, 32, 64);
+        if (col < rows) m_new = dot * scale_log2;
+      }
+    }
   }
+
   f32x4_t acc[1][D / 16];
 #pragma unroll
   for (int nb = 0; nb < D / 16; ++nb) acc[0][nb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   float m_run[1] = {-INFINITY}, l_run[1] = {0.f};
-
-  attend_tiles<D, 1>(qreg, k_cache, v_cache, num_pages, bt_row, Hkv, g_kv, page, t0 + wave, t1, 4, kv_len, row_pos,
-                     window, scale_log2, acc, m_run, l_run);
+  attend_tiles<D, 1>(qreg, a_first, t_first, k_cache, v_cache, num_pages, bt_row, Hkv, g_kv, page, t0 + wave, t1, 4,
+                     kv_seen, row_pos, win, scale_log2, acc, m_run, l_run);
 
   // this lane's sum covers its own keys only
   float l = l_run[0];
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
 
-  __shared__ float sh_m[4][16], sh_l[4][16];
+  // the merge of the four wavefronts, and of the new key as a fifth contribution of one key:
+  // its score is its maximum, its sum is one, its accumulator is the value itself
+  __shared__ float sh_m[5][16], sh_l[4][16];
   __shared__ float sh_acc[4][16][D + 4];
   if (grp == 0) {
     sh_m[wave][col] = m_run[0];
     sh_l[wave][col] = l;
   }
+  if (wave == 3 && grp == 0) sh_m[4][col] = m_new;
   __syncthreads();
   float m_all = fmaxf(fmaxf(sh_m[0][col], sh_m[1][col]), fmaxf(sh_m[2][col], sh_m[3][col]));
+  m_all = fmaxf(m_all, sh_m[4][col]);
   const float w_mine = m_run[0] > -INFINITY ? exp2f(m_run[0] - m_all) : 0.f;
   if (col < rows) {
 #pragma unroll
@@ -578,21 +642,27 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   // 256 threads: thread -> (row = t / 16, d = t % 16 + 16 k)
   const int r = threadIdx.x >> 4, dd = threadIdx.x & 15;
   if (r >= rows) return;
-  const float mr = fmaxf(fmaxf(sh_m[0][r], sh_m[1][r]), fmaxf(sh_m[2][r], sh_m[3][r]));
-  float lr = 0.f;
+  const float m5 = sh_m[4][r];
+  const float mr = fmaxf(fmaxf(fmaxf(sh_m[0][r], sh_m[1][r]), fmaxf(sh_m[2][r], sh_m[3][r])), m5);
+  const float w5 = m5 > -INFINITY ? exp2f(m5 - mr) : 0.f;
+  float lr = w5;
 #pragma unroll
   for (int w = 0; w < 4; ++w) lr += sh_m[w][r] > -INFINITY ? sh_l[w][r] * exp2f(sh_m[w][r] - mr) : 0.f;
   const int token = q0 + r / G, head = g_kv * G + r % G;
   if (splits == 1) {
     const float inv = 1.f / lr;
     for (int d = dd; d < D; d += 16) {
-      const float o = sh_acc[0][r][d] + sh_acc[1][r][d] + sh_acc[2][r][d] + sh_acc[3][r][d];
+      float o = sh_acc[0][r][d] + sh_acc[1][r][d] + sh_acc[2][r][d] + sh_acc[3][r][d];
+      if (PREP && w5 > 0.f) o += sh_v[d] * w5;
       out[(size_t)token * Hq * D + (size_t)head * D + d] = float_to_bf16(o * inv);
     }
   } else {
     const size_t slot = (((size_t)b * Hkv + g_kv) * splits + split) * 16 + r;
-    for (int d = dd; d < D; d += 16)
-      ws_acc[slot * D + d] = sh_acc[0][r][d] + sh_acc[1][r][d] + sh_acc[2][r][d] + sh_acc[3][r][d];
+    for (int d = dd; d < D; d += 16) {
+      float o = sh_acc[0][r][d] + sh_acc[1][r][d] + sh_acc[2][r][d] + sh_acc[3][r][d];
+      if (PREP && w5 > 0.f) o += sh_v[d] * w5;
+      ws_acc[slot * D + d] = o;
+    }
     if (dd == 0) {
       ws_ml[slot * 2] = mr;
       ws_ml[slot * 2 + 1] = lr;
@@ -1068,7 +1138,8 @@ extern "C" int q3_decode_attention_takes(int Hq, int Hkv, int D, int page, int d
 // 2 Hkv) D) bfloat16 holds [q | k | v] of token b in row b (cu_q[b] = b). Per-head RMSNorm
 // of q and k (weights of `w_dtype`, both or neither), rotation by `table` (or null), the new
 // key and value written to the caches at position kv_lens[b] - 1 (if `store`), and attention
-// over the cache, in one kernel and the merge of its splits. out (B, Hq D) bfloat16.
+// over the cache, in one kernel and, with more than one split, the merge of its partial
+// results (workspace as for q3_paged_attention). out (B, Hq D) bfloat16.
 extern "C" int q3_decode_attention(const void* qkv, void* out, void* k_cache, void* v_cache, int num_pages,
                                    const int* block_table, int bt_stride, const int* cu_q, const int* kv_lens,
                                    int B, int Hq, int Hkv, int D, int page, float scale, int window, int splits,

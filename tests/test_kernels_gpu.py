@@ -211,10 +211,11 @@ def test_paged_attention_decoding_batches(Hq, Hkv, D, page, window):
 @pytest.mark.parametrize("w_dtype", [torch.float32, torch.bfloat16, None])
 @pytest.mark.parametrize("window,rotate,store", [(0, True, True), (23, True, True), (0, False, True), (0, True, False)])
 def test_decode_attention_is_its_two_halves(Hq, Hkv, D, page, w_dtype, window, rotate, store):
-    """A step of single tokens in one kernel gives, to the bit, what the preparation kernel
-    followed by the attention kernel gives: the prepared queries and keys, the caches after
-    the step, and the output. Lengths are chosen so that the new key is a page's first and
-    last slot, a tile's first key, and far into many splits."""
+    """A step of single tokens in one kernel gives what the preparation kernel followed by the
+    attention kernel gives: the caches after the step to the bit, and the output to the bit
+    where nothing is stored, else to the order in which the new key's share is added.
+    Lengths are chosen so that the new key is a page's first and last slot, a tile's first
+    key, and far into many splits."""
     ops = _ops()
     kv_lens = [1, page, page + 1, 33, 64, 65, 700, 2500]
     B = len(kv_lens)
@@ -245,7 +246,12 @@ def test_decode_attention_is_its_two_halves(Hq, Hkv, D, page, w_dtype, window, r
     assert torch.equal(k2, k1) and torch.equal(v2, v1)
     if not store:
         assert torch.equal(k2, kc) and torch.equal(v2, vc)
-    assert torch.equal(got, want)
+    if store:
+        # the two-kernel path rounds the new key's probability to bfloat16 with all the others, the
+        # fused one keeps it in float32: half a bfloat16 step of a probability times a value of size ~1
+        torch.testing.assert_close(got.float(), want.float(), rtol=8e-3, atol=6e-3)
+    else:
+        assert torch.equal(got, want)
     # and against plain arithmetic
     ref = torch_ops.paged_attention(q.float(), Hq, k1.float(), v1.float(), bt, cu, kvl, 1, max(kv_lens), scale,
                                     window=window)

@@ -43,6 +43,7 @@ class _Held:
     reserved: int = 0                    # tokens beyond `length` that pages are held for
     tables: list = field(default_factory=list)   # per group: page of each block, -1 once given back
     slot: int = -1
+    admission: int = 0                   # which admission of the manager's this is
 
 
 class CacheManager:
@@ -81,6 +82,7 @@ class CacheManager:
             self.state_group_of_plane.append(s)
         self._slots = list(range(max_requests - 1, -1, -1))
         self._requests = {}
+        self._admissions = 0
         self.fresh_slots = []     # slots handed out since the storage last cleared them
 
     # ---- requests ----
@@ -96,12 +98,18 @@ class CacheManager:
     def slot(self, request_id):
         return self._requests[request_id].slot
 
+    def admission(self, request_id):
+        """A number that differs between two admissions of the same request id:
+        who remembers a request's pages checks it before trusting them."""
+        return self._requests[request_id].admission
+
     def admit(self, request_id):
         if request_id in self._requests:
             raise KeyError("request %r is already live" % (request_id,))
         if not self._slots:
             raise OutOfPages("all %d request slots are taken" % self.max_requests)
-        held = _Held(tables=[[] for _ in self.groups], slot=self._slots.pop())
+        self._admissions += 1
+        held = _Held(tables=[[] for _ in self.groups], slot=self._slots.pop(), admission=self._admissions)
         self._requests[request_id] = held
         self.fresh_slots.append(held.slot)
         return held.slot

@@ -25,28 +25,60 @@ class _DecodeGraph:
         self.graph = None
         self.logits = None
         self.copied = torch.cuda.Event()
+        self.last_ids = self.last_lengths = self.last_slots = self.last_table_lens = None
 
     def run(self, runner, entries, lengths, slots, tables):
         self.copied.synchronize()          # the last step's copy has left the host buffer
-        batch, block_tables = pack_step(entries, lengths, slots, tables, runner.device,
-                                        fixed_widths=self.widths, buffers=(self.host, self.dev), all_rows=True)
+        ids = [(e.request_id, runner.manager.admission(e.request_id)) for e in entries]
+        if (self.graph is not None and ids == self.last_ids and slots == self.last_slots
+                and all(n == m + 1 for n, m in zip(lengths, self.last_lengths))):
+            self._advance(runner, entries, tables)
+        else:
+            batch, block_tables = pack_step(entries, lengths, slots, tables, runner.device,
+                                            fixed_widths=self.widths, buffers=(self.host, self.dev), all_rows=True)
+            batch.max_kv_len = self.max_kv_len
+            if self.graph is None:
+                self._capture(runner, batch, block_tables)
         self.copied.record()
-        batch.max_kv_len = self.max_kv_len
-        runner.storage.bind(block_tables)
-        if self.graph is None:
-            # once eagerly on a side stream (libraries build and tune at first use), then capture
-            side = torch.cuda.Stream(device=runner.device)
-            side.wait_stream(torch.cuda.current_stream(runner.device))
-            with torch.cuda.stream(side):
-                runner.model.forward(batch, runner.storage)
-            torch.cuda.current_stream(runner.device).wait_stream(side)
-            torch.cuda.synchronize(runner.device)
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                self.logits = runner.model.forward(batch, runner.storage)
-            self.graph = graph
+        self.last_ids, self.last_lengths, self.last_slots = ids, list(lengths), list(slots)
+        self.last_table_lens = [[len(t) for t in group] for group in tables]
         self.graph.replay()
         return self.logits
+
+    def _advance(self, runner, entries, tables):
+        """The same requests (and admissions of them) as in the last step, each one token further: the
+        packed description changes in its tokens, by one in positions and
+        lengths, and in the block tables' new entries (all entries where a
+        window gives pages back)."""
+        B, host = self.B, self.host.numpy()
+        host[0:B] = [e.tokens[0] for e in entries]
+        host[B:2 * B] += 1                        # positions
+        host[4 * B + 1:5 * B + 1] += 1            # keys visible after the step
+        base = 7 * B + 1
+        for g, (group_tables, w) in enumerate(zip(tables, self.widths)):
+            windowed = runner.manager.groups[g].window > 0
+            for i, t in enumerate(group_tables):
+                had = 0 if windowed else self.last_table_lens[g][i]
+                if len(t) > w:
+                    raise ValueError("a block table is wider than the fixed width %d" % w)
+                if len(t) > had:
+                    host[base + i * w + had: base + i * w + len(t)] = t[had:]
+            base += B * w
+        self.dev.copy_(self.host, non_blocking=True)
+
+    def _capture(self, runner, batch, block_tables):
+        runner.storage.bind(block_tables)
+        # once eagerly on a side stream (libraries build and tune at first use), then capture
+        side = torch.cuda.Stream(device=runner.device)
+        side.wait_stream(torch.cuda.current_stream(runner.device))
+        with torch.cuda.stream(side):
+            runner.model.forward(batch, runner.storage)
+        torch.cuda.current_stream(runner.device).wait_stream(side)
+        torch.cuda.synchronize(runner.device)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            self.logits = runner.model.forward(batch, runner.storage)
+        self.graph = graph
 
 
 class ModelRunner:

@@ -461,7 +461,7 @@ def linear_residual_norm(x, weight, tiled, residual, norm_weight):
     return values, sums
 
 
-def sample(logits, temperature, top_k, seed, counter, out=None):
+def sample(logits, temperature, top_k, seed, counter, out=None, any_top_k=True):
     """One token per row of float32 logits (R, V).
 
     Row r: temperature[r] <= 0 takes the arg-max (lowest index among equals).
@@ -469,7 +469,8 @@ def sample(logits, temperature, top_k, seed, counter, out=None):
     top_k[r] > 0, to logits not below the k-th largest; the draw is the
     arg-max of logits / temperature + Gumbel noise from a counter-based
     generator keyed by (seed[r], counter[r], column), so a request's tokens do
-    not depend on what else is in the batch.
+    not depend on what else is in the batch. `any_top_k=False` promises that no row has a
+    top_k in effect, which saves the selection pass.
     """
     _dev(logits, temperature, top_k, seed, counter, out)
     _need(logits.dim() == 2 and logits.dtype == torch.float32, "logits must be float32 (R, V)")
@@ -482,7 +483,10 @@ def sample(logits, temperature, top_k, seed, counter, out=None):
         out = torch.empty((R,), dtype=torch.int32, device=logits.device)
     _need(out.shape == (R,) and out.dtype == torch.int32, "out int32 (R,)")
     if R:
-        _check(library("sampling").q3_sample(
+        lib = library("sampling")
+        lib.q3_sample_workspace.restype = ctypes.c_long
+        workspace = torch.empty((lib.q3_sample_workspace(R, V) + 7) // 8, dtype=torch.int64, device=logits.device)
+        _check(lib.q3_sample(
             _ptr(logits), _ptr(temperature), _ptr(top_k), _ptr(seed), _ptr(counter), _ptr(out),
-            R, V, _stream()), "sample")
+            R, V, 1 if any_top_k else 0, _ptr(workspace), _stream()), "sample")
     return out

@@ -2,6 +2,7 @@
 
 from dataclasses import dataclass
 
+import numpy as np
 import torch
 
 from .. import ops
@@ -31,6 +32,21 @@ class Sampler:
 
     def __init__(self, device):
         self.device = torch.device(device)
+        self._buffers = {}
+
+    def _buffer(self, R):
+        """Five int32 words per row, pinned on the host and on the device: seed (two words),
+        temperature, top_k, counter; one copy brings a step's parameters."""
+        pair = self._buffers.get(R)
+        if pair is None:
+            host = torch.empty(5 * R, dtype=torch.int32)
+            if self.device.type == "cuda":
+                host = host.pin_memory()
+            pair = (host, torch.empty(5 * R, dtype=torch.int32, device=self.device))
+            if len(self._buffers) > 64:
+                self._buffers.clear()
+            self._buffers[R] = pair
+        return pair
 
     def sample(self, logits, params, counters):
         """`params[r]` and `counters[r]` (number of tokens the request has
@@ -38,14 +54,15 @@ class Sampler:
         R = logits.shape[0]
         if R == 0:
             return []
-        host = torch.empty((R, 4), dtype=torch.int64)
-        temps = torch.empty(R, dtype=torch.float32)
-        for r, (p, c) in enumerate(zip(params, counters)):
-            temps[r] = p.temperature
-            host[r, 0] = p.top_k
-            host[r, 1] = p.seed
-            host[r, 2] = c
-        dev = host.to(self.device)
-        out = ops.sample(logits, temps.to(self.device), dev[:, 0].to(torch.int32).contiguous(),
-                         dev[:, 1].contiguous(), dev[:, 2].to(torch.int32).contiguous())
+        host, dev = self._buffer(R)
+        words = host.numpy()
+        words[0:2 * R].view(np.int64)[:] = [p.seed for p in params]
+        words[2 * R:3 * R].view(np.float32)[:] = [p.temperature for p in params]
+        words[3 * R:4 * R] = [p.top_k for p in params]
+        words[4 * R:5 * R] = counters
+        # queued behind the step's kernels without waiting for them; the list below is the only wait
+        dev.copy_(host, non_blocking=True)
+        any_top_k = any(p.top_k > 0 and p.temperature > 0 for p in params)
+        out = ops.sample(logits, dev[2 * R:3 * R].view(torch.float32), dev[3 * R:4 * R], dev[0:2 * R].view(torch.int64),
+                         dev[4 * R:5 * R], any_top_k=any_top_k)
         return out.tolist()

@@ -151,7 +151,7 @@ def _uniform(seed, counter, n, device):
     return torch.rand(n, generator=g).to(device)
 
 
-def sample(logits, temperature, top_k, seed, counter, out=None):
+def sample(logits, temperature, top_k, seed, counter, out=None, any_top_k=True):
     R, V = logits.shape
     res = torch.empty(R, dtype=torch.int32, device=logits.device)
     for r in range(R):

@@ -67,6 +67,8 @@ class EngineConfig:
     num_blocks: int = 0
     seed: int = 0
     use_graphs: bool = True
+    # launch a decode step before the previous step's tokens have reached the host
+    lookahead: bool = True
 
     def __post_init__(self):
         self.dtype = parse_dtype(self.dtype)

@@ -27,7 +27,7 @@ class _DecodeGraph:
         self.copied = torch.cuda.Event()
         self.last_ids = self.last_lengths = self.last_slots = self.last_table_lens = None
 
-    def run(self, runner, entries, lengths, slots, tables):
+    def run(self, runner, entries, lengths, slots, tables, device_tokens=None):
         self.copied.synchronize()          # the last step's copy has left the host buffer
         ids = [(e.request_id, runner.manager.admission(e.request_id)) for e in entries]
         if (self.graph is not None and ids == self.last_ids and slots == self.last_slots
@@ -40,6 +40,8 @@ class _DecodeGraph:
             if self.graph is None:
                 self._capture(runner, batch, block_tables)
         self.copied.record()
+        if device_tokens is not None:      # the tokens are still on the device: they replace the placeholders
+            self.dev[0:self.B].copy_(device_tokens)
         self.last_ids, self.last_lengths, self.last_slots = ids, list(lengths), list(slots)
         self.last_table_lens = [[len(t) for t in group] for group in tables]
         self.graph.replay()
@@ -110,12 +112,19 @@ class ModelRunner:
         self._graphs = {}
         self.max_graphs = 32
 
-    def step(self, entries):
+    def step(self, entries, device_tokens=None):
         """entries: list of StepEntry. Returns logits (R, V) float32 on the
         device, rows in the order of the entries and of their `want`. The
-        tensor may be overwritten by the next call of step()."""
+        tensor may be overwritten by the next call of step().
+        `device_tokens`: an int32 device tensor with one token per entry, for a
+        step of single tokens that are not on the host yet (the last step's
+        sampled ones); the entries' own tokens are then placeholders."""
         if not entries:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
+        single = all(len(e.tokens) == 1 for e in entries)
+        if device_tokens is not None and not (single and device_tokens.shape == (len(entries),)
+                                              and device_tokens.dtype == torch.int32):
+            raise ValueError("device tokens come one per entry (int32), for entries of one token each")
         seen = set()
         for e in entries:
             if e.request_id in seen:
@@ -146,17 +155,19 @@ class ModelRunner:
         slots = [m.slot(e.request_id) for e in entries]
         tables = [[m.block_table(e.request_id, g) for e in entries] for g in range(len(m.groups))]
         self.storage.clear_fresh_slots()
-        if self.use_graphs and all(len(e.tokens) == 1 for e in entries):
-            logits = self._step_graph(entries, lengths, slots, tables)
+        if self.use_graphs and single:
+            logits = self._step_graph(entries, lengths, slots, tables, device_tokens)
         else:
             batch, block_tables = pack_step(entries, lengths, slots, tables, self.device)
+            if device_tokens is not None:
+                batch.token_ids.copy_(device_tokens)
             self.storage.bind(block_tables)
             logits = self.model.forward(batch, self.storage)
         for e in entries:
             m.commit(e.request_id, len(e.tokens))
         return logits
 
-    def _step_graph(self, entries, lengths, slots, tables):
+    def _step_graph(self, entries, lengths, slots, tables, device_tokens=None):
         B = len(entries)
         longest = max(lengths) + 1
         bucket = 256
@@ -169,7 +180,7 @@ class ModelRunner:
                 self._graphs.pop(next(iter(self._graphs)))
             graph = _DecodeGraph(self, B, bucket)
         self._graphs[(B, bucket)] = graph                   # most recently used last
-        logits = graph.run(self, entries, lengths, slots, tables)
+        logits = graph.run(self, entries, lengths, slots, tables, device_tokens)
         wanted = [i for i, e in enumerate(entries) for _ in e.want]
         if wanted == list(range(B)):
             return logits

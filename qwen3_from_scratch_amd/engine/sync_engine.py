@@ -22,7 +22,7 @@ from ..sampling import Sampler, SamplingParams
 from .batch import StepEntry
 from .loading import load_model
 from .runner import ModelRunner
-from .scheduler import Request, RequestStatus, Scheduler
+from .scheduler import Request, RequestStatus, Scheduled, Scheduler
 
 
 @dataclass
@@ -59,6 +59,14 @@ def _load_tokenizer(path):
     return AutoTokenizer.from_pretrained(path)
 
 
+@dataclass
+class _InFlight:
+    """A step that is on the GPU: its plan, and its tokens on their way."""
+
+    plan: list
+    sampled: object
+
+
 class SyncEngine:
     def __init__(self, config_path=None, model_name=None, log_interval=0, *, config=None, model=None,
                  **overrides):
@@ -88,6 +96,10 @@ class SyncEngine:
         self.eos_ids = self._eos_ids()
         self._ids = itertools.count()
         self.steps = 0
+        # one step ahead of the tokens only where a step is a graph replay: otherwise the host
+        # is busy launching kernels anyway
+        self.lookahead = bool(config.lookahead) and self.runner.use_graphs
+        self._ahead = None
 
     # ---- set-up ----
     def _blocks_from_memory(self):
@@ -163,10 +175,38 @@ class SyncEngine:
     def step(self):
         """Schedule, run the step function, sample, book-keep. Returns the plan
         (a list of Scheduled); requests that got a token have it in
-        `last_token_id`, finished ones have status FINISHED."""
-        plan = self.scheduler.schedule()
-        if not plan:
-            return plan
+        `last_token_id`, finished ones have status FINISHED.
+
+        While the same requests decode on, the next step is put on the GPU
+        before this one's tokens are read back (`_launch_ahead`), so that the
+        GPU does not wait for the host between steps; the plan returned is
+        always that of the step whose tokens have arrived."""
+        current, self._ahead = self._ahead, None
+        if current is not None and not any(s.request.status == RequestStatus.RUNNING for s in current.plan):
+            current = None               # its requests ended or were taken out meanwhile: nothing to report
+        if current is None:
+            plan = self.scheduler.schedule()
+            if not plan:
+                return plan
+            current = self._launch(plan)
+        if self.lookahead:
+            self._ahead = self._launch_ahead(current)
+        tokens = self.sampler.collect(current.sampled) if current.sampled is not None else []
+        it = iter(tokens)
+        plan, sampled = [], []
+        for s in current.plan:
+            token = next(it) if s.samples else None
+            if s.request.status != RequestStatus.RUNNING:
+                continue                 # ended (or was taken out) while this step was on its way
+            plan.append(s)
+            if s.samples:
+                sampled.append(token)
+        self.scheduler.after_step(plan, sampled)
+        self.steps += 1
+        return plan
+
+    def _launch(self, plan):
+        """Put a scheduled plan on the GPU: the step function, then sampling."""
         entries = []
         for s in plan:
             req = s.request
@@ -174,11 +214,35 @@ class SyncEngine:
             entries.append(StepEntry(req.request_id, tokens, [s.num_tokens - 1] if s.samples else []))
         logits = self.runner.step(entries)
         sampling = [s.request for s in plan if s.samples]
-        sampled = self.sampler.sample(logits, [r.params for r in sampling],
-                                      [len(r.generated) for r in sampling])
-        self.scheduler.after_step(plan, sampled)
-        self.steps += 1
-        return plan
+        sampled = None
+        if sampling:
+            sampled = self.sampler.launch(logits, [r.params for r in sampling], [len(r.generated) for r in sampling])
+        return _InFlight(plan, sampled)
+
+    def _launch_ahead(self, current):
+        """The step after `current`, if it is certain enough what it will be:
+        every running request decodes in `current`, none of them ends with
+        `current`'s token by its count, nobody waits, and pages are there.
+        Its input tokens are `current`'s sampled ones, read on the device. A
+        request that ends with `current`'s token after all (an end-of-sequence
+        token) has then made one step too many, whose token is dropped and
+        whose pages went back with the others'."""
+        sched = self.scheduler
+        plan = current.plan
+        if sched.waiting or len(plan) != len(sched.running) or current.sampled is None:
+            return None
+        spare = [0] * len(self.runner.manager.groups)
+        for s in plan:
+            req = s.request
+            if (s.num_tokens != 1 or not s.samples or req.status != RequestStatus.RUNNING or req.is_prefill
+                    or len(req.generated) + 2 > req.params.max_new_tokens
+                    or not self.runner.manager.can_grow(req.request_id, 1, spare)):
+                return None
+        entries = [StepEntry(s.request.request_id, [0], [0]) for s in plan]
+        logits = self.runner.step(entries, device_tokens=current.sampled.tokens)
+        sampled = self.sampler.launch(logits, [s.request.params for s in plan],
+                                      [len(s.request.generated) + 1 for s in plan])
+        return _InFlight([Scheduled(s.request, 1, True) for s in plan], sampled)
 
     # ---- the reference's interface ----
     def warmup(self, prompt=None, num_tokens=3):

@@ -23,46 +23,89 @@ class SamplingParams:
     ignore_eos: bool = False
 
 
+class Sampled:
+    """A step's tokens on their way: `tokens` on the device (the next step may
+    read them there), a pinned copy on the host, and the event after which the
+    copy has arrived."""
+
+    def __init__(self, tokens, host, event):
+        self.tokens = tokens
+        self.host = host
+        self.event = event
+
+
 class Sampler:
     """Greedy: arg-max (inference/sampler.py:17-21). Temperature:
     a draw from softmax(logits / temperature) (:24-33). Top-k: the same among
-    the k largest logits (:36-56). All three are one kernel launch over the
-    float32 logits; draws use Gumbel noise keyed by (seed, index of the token
-    being generated)."""
+    the k largest logits (:36-56). All three go through the same kernels over
+    the float32 logits; draws use Gumbel noise keyed by (seed, index of the token
+    being generated).
+
+    `launch` queues a step's sampling behind its kernels and returns at once;
+    `collect` waits for the tokens. Up to `RING` launches may be uncollected at
+    a time: each has staging buffers of its own."""
+
+    RING = 4
 
     def __init__(self, device):
         self.device = torch.device(device)
-        self._buffers = {}
+        self._rings = {}
 
-    def _buffer(self, R):
-        """Five int32 words per row, pinned on the host and on the device: seed (two words),
-        temperature, top_k, counter; one copy brings a step's parameters."""
-        pair = self._buffers.get(R)
-        if pair is None:
-            host = torch.empty(5 * R, dtype=torch.int32)
+    def _staging(self, R):
+        """Pinned host memory and its device twin for a step's parameters (five
+        int32 words per row: seed in two, temperature, top_k, counter) and
+        tokens (one int32 per row); RING sets per batch size, used in turn."""
+        ring = self._rings.get(R)
+        if ring is None:
+            if len(self._rings) > 64:
+                self._rings.clear()
+            ring = self._rings[R] = {"next": 0, "sets": []}
+        if len(ring["sets"]) < self.RING:
+            host = torch.empty(6 * R, dtype=torch.int32)
             if self.device.type == "cuda":
                 host = host.pin_memory()
-            pair = (host, torch.empty(5 * R, dtype=torch.int32, device=self.device))
-            if len(self._buffers) > 64:
-                self._buffers.clear()
-            self._buffers[R] = pair
-        return pair
+            entry = {"host": host, "dev": torch.empty(6 * R, dtype=torch.int32, device=self.device), "event": None}
+            ring["sets"].append(entry)
+            return entry
+        entry = ring["sets"][ring["next"]]
+        ring["next"] = (ring["next"] + 1) % self.RING
+        if entry["event"] is not None:
+            entry["event"].synchronize()           # its last user's copies are done
+        return entry
 
-    def sample(self, logits, params, counters):
+    def launch(self, logits, params, counters):
         """`params[r]` and `counters[r]` (number of tokens the request has
-        generated so far) belong to row r. Returns a list of token ids."""
+        generated before this one) belong to row r. Returns a `Sampled`."""
         R = logits.shape[0]
-        if R == 0:
-            return []
-        host, dev = self._buffer(R)
+        entry = self._staging(R)
+        host, dev = entry["host"], entry["dev"]
         words = host.numpy()
         words[0:2 * R].view(np.int64)[:] = [p.seed for p in params]
         words[2 * R:3 * R].view(np.float32)[:] = [p.temperature for p in params]
         words[3 * R:4 * R] = [p.top_k for p in params]
         words[4 * R:5 * R] = counters
-        # queued behind the step's kernels without waiting for them; the list below is the only wait
-        dev.copy_(host, non_blocking=True)
+        # queued behind the step's kernels without waiting for them
+        dev[:5 * R].copy_(host[:5 * R], non_blocking=True)
         any_top_k = any(p.top_k > 0 and p.temperature > 0 for p in params)
-        out = ops.sample(logits, dev[2 * R:3 * R].view(torch.float32), dev[3 * R:4 * R], dev[0:2 * R].view(torch.int64),
-                         dev[4 * R:5 * R], any_top_k=any_top_k)
-        return out.tolist()
+        tokens = dev[5 * R:6 * R]
+        ops.sample(logits, dev[2 * R:3 * R].view(torch.float32), dev[3 * R:4 * R], dev[0:2 * R].view(torch.int64),
+                   dev[4 * R:5 * R], out=tokens, any_top_k=any_top_k)
+        host[5 * R:6 * R].copy_(tokens, non_blocking=True)
+        event = None
+        if self.device.type == "cuda":
+            event = torch.cuda.Event()
+            event.record()
+        entry["event"] = event
+        return Sampled(tokens, host[5 * R:6 * R], event)
+
+    def collect(self, sampled):
+        """The tokens of a `launch`, as a list."""
+        if sampled.event is not None:
+            sampled.event.synchronize()
+        return sampled.host.tolist()
+
+    def sample(self, logits, params, counters):
+        """`launch` and `collect` in one call."""
+        if logits.shape[0] == 0:
+            return []
+        return self.collect(self.launch(logits, params, counters))

@@ -163,3 +163,42 @@ def max_live_tokens(steps, page=64):
         for rid in ends:
             held.pop(rid, None)
     return worst
+
+
+def arrivals_scenario(folder, lookahead, num_blocks, name="B", device="cpu", dtype="float32", block_size=8):
+    """Requests that arrive over time, end by count or by an end-of-sequence token, sample with
+    seeds or greedily, and (with few pages) preempt one another. Returns what was generated
+    and how many steps were put on the GPU ahead of their tokens."""
+    from qwen3_from_scratch_amd.engine import SyncEngine
+
+    vocab = TINY[name]["config"]["vocab_size"]
+    engine = SyncEngine(path=folder, dtype=dtype, device=device, block_size=block_size, num_blocks=num_blocks,
+                        max_num_seqs=4, chunked_prefill_size=16)
+    engine.lookahead = lookahead
+    engine.eos_ids = tuple(range(0, vocab, 9))            # every ninth token ends a request that honours it
+    ahead = [0]
+    launch_ahead = engine._launch_ahead
+
+    def counting(current):
+        got = launch_ahead(current)
+        ahead[0] += got is not None
+        return got
+
+    engine._launch_ahead = counting
+    arrivals = {0: [(21, dict(temperature=0.9, seed=3), 40, True), (9, dict(temperature=0.0), 25, True)],
+                7: [(33, dict(temperature=0.7, top_k=5, seed=11), 30, False)],
+                30: [(5, dict(temperature=0.0), 12, False)]}
+    requests = []
+    step = 0
+    while step < 400 and (engine.scheduler.has_work() or step <= max(arrivals)):
+        for n, sampling, new, ignore in arrivals.get(step, []):
+            params = engine.default_params(new, ignore_eos=ignore, **sampling)
+            requests.append(engine.add_request(random_tokens(n, vocab, 90 + n), params))
+        plan = engine.step()
+        for s in plan:
+            assert s.request.status.name in ("RUNNING", "FINISHED")
+        engine.runner.manager.audit()
+        step += 1
+    assert not engine.scheduler.has_work()
+    assert engine.runner.manager.num_free() == num_blocks
+    return [list(r.generated) for r in requests], [r.preemptions for r in requests], ahead[0]

@@ -11,7 +11,7 @@ import pytest
 import torch
 
 import plain_qwen3
-from helpers import TINY, max_live_tokens, random_tokens, trace_mixed, trace_portions
+from helpers import TINY, arrivals_scenario, max_live_tokens, random_tokens, trace_mixed, trace_portions
 from qwen3_from_scratch_amd.engine import SyncEngine
 
 pytestmark = pytest.mark.gpu
@@ -58,6 +58,21 @@ def test_bfloat16_generation_and_seeded_sampling(model_folders):
     b = SyncEngine(max_num_seqs=1, **kw).generate_ids(prompts[2:3], 6, temperature=0.8, top_k=20, seed=3,
                                                       ignore_eos=True)
     assert a[2] == b[0]                       # a request's draws do not depend on its batch
+
+
+@pytest.mark.parametrize("name,dtype,block_size,num_blocks", [("E", "bfloat16", 16, 40), ("E", "bfloat16", 16, 5),
+                                                              ("B", "float32", 8, 10), ("D", "bfloat16", 16, 6)])
+def test_a_step_ahead_changes_no_token(model_folders, name, dtype, block_size, num_blocks):
+    """Decode steps launched before the last step's tokens are on the host (graph replays fed
+    from the device) give the tokens of the step-by-step engine, through arrivals, ends by
+    count and by token, seeded sampling, and preemption."""
+    kw = dict(name=name, device="cuda", dtype=dtype, block_size=block_size)
+    plain, preempted, none_ahead = arrivals_scenario(model_folders[name], False, num_blocks, **kw)
+    ahead, preempted_ahead, steps_ahead = arrivals_scenario(model_folders[name], True, num_blocks, **kw)
+    assert none_ahead == 0 and steps_ahead > (10 if num_blocks >= 20 else 0)
+    assert ahead == plain and preempted_ahead == preempted
+    if num_blocks < 20:
+        assert sum(preempted) > 0
 
 
 def _replay(folder, dtype, steps, out, max_tokens):

@@ -6,7 +6,7 @@ import pytest
 import torch
 
 import plain_qwen3
-from helpers import TINY, random_tokens
+from helpers import TINY, arrivals_scenario, random_tokens
 from qwen3_from_scratch_amd.engine import SyncEngine
 
 
@@ -80,3 +80,34 @@ def test_sampling_is_reproducible_per_request(cpu_ops, model_folders):
     other = SyncEngine(max_num_seqs=1, **kw).generate_ids([prompts[0]], 8, temperature=0.8, seed=6,
                                                           ignore_eos=True)[0]
     assert other != alone
+
+
+@pytest.mark.parametrize("num_blocks", [40, 10])
+def test_a_step_ahead_changes_no_token(cpu_ops, model_folders, num_blocks):
+    plain, preempted, none_ahead = arrivals_scenario(model_folders["B"], False, num_blocks)
+    ahead, preempted_ahead, steps_ahead = arrivals_scenario(model_folders["B"], True, num_blocks)
+    assert none_ahead == 0 and steps_ahead > 10
+    assert ahead == plain
+    assert [len(g) for g in plain][:2] == [40, 25] and len(plain[2]) < 30         # the third ends early, by a token
+    if num_blocks == 10:
+        assert sum(preempted) > 0 and sum(preempted_ahead) > 0
+
+
+def test_abort_while_a_step_is_ahead(cpu_ops, model_folders):
+    vocab = TINY["A"]["config"]["vocab_size"]
+    engine = SyncEngine(path=model_folders["A"], dtype="float32", device="cpu", num_blocks=16, max_num_seqs=2)
+    engine.lookahead = True
+    a = engine.add_request(random_tokens(6, vocab, 1), engine.default_params(30, temperature=0.0, ignore_eos=True))
+    b = engine.add_request(random_tokens(9, vocab, 2), engine.default_params(30, temperature=0.0, ignore_eos=True))
+    for _ in range(5):
+        engine.step()
+    assert engine._ahead is not None
+    engine.abort(a)                                   # its row of the step ahead is dropped
+    before = len(b.generated)
+    plan = engine.step()
+    assert [s.request for s in plan] == [b] and len(b.generated) == before + 1 and len(a.generated) < 30
+    while engine.scheduler.has_work():
+        engine.step()
+    assert len(b.generated) == 30 and engine.runner.manager.num_free() == 16
+    solo = SyncEngine(path=model_folders["A"], dtype="float32", device="cpu", num_blocks=16, max_num_seqs=2)
+    assert solo.generate_ids([b.prompt], 30, temperature=0.0, ignore_eos=True)[0] == b.generated

@@ -674,15 +674,19 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
 // (A kernel of its own rather than the work of the decode kernel's last-arriving
 // block: the device-scope fences that needs write back and invalidate each XCD's
 // L2, which measured three times slower than this second launch.)
-// The weights of the splits are formed once per row in shared memory, then
-// every thread sums a few output elements over the splits with loads that are
-// contiguous across the block.
+// The kernel is a chain of latencies, so it asks for as much as it can at once: a thread
+// owns four neighbouring output elements and every `groups`-th split (groups = as many as
+// 256 threads allow), loads its first eight partial accumulators before anything else,
+// then the maxima and sums, from which a wavefront forms a row's weights (a split per lane)
+// and leaves them in shared memory; the groups' sums meet there too.
 #define MAX_SPLITS 64
+#define REDUCE_BATCH 8
 template <int D>
 __global__ __launch_bounds__(256) void attn_decode_reduce_kernel(
     bf16_t* __restrict__ out, const int* __restrict__ cu_q, int Hq, int Hkv, int splits,
     const float* __restrict__ ws_acc, const float* __restrict__ ws_ml) {
-  __shared__ float sh_w[16][MAX_SPLITS], sh_l[16][MAX_SPLITS];
+  __shared__ float sh_w[16][MAX_SPLITS];
+  __shared__ float4 sh_part[256];
   const int b = blockIdx.y, g_kv = blockIdx.x;
   const int G = Hq / Hkv;
   const int q0 = cu_q[b];
@@ -690,54 +694,80 @@ __global__ __launch_bounds__(256) void attn_decode_reduce_kernel(
   if (q_len <= 0 || q_len * G > 16) return;
   const int rows = q_len * G;
   const size_t base = ((size_t)b * Hkv + g_kv) * splits;
-  // every load of the kernel is issued before anything waits: maxima and sums here, and
-  // this thread's first accumulator elements
-  const int n_elems = rows * D;
-  float first[4] = {0.f, 0.f, 0.f, 0.f};
-  const int e0 = threadIdx.x;
-  if (splits <= 4 && e0 < n_elems) {
-    const int r = e0 / D, d = e0 - r * D;
-    for (int s = 0; s < splits; ++s) first[s] = ws_acc[((base + s) * 16 + r) * D + d];
-  }
-  for (int idx = threadIdx.x; idx < rows * splits; idx += blockDim.x) {
-    const int r = idx / splits, s = idx - r * splits;
-    const float2 ml = *reinterpret_cast<const float2*>(ws_ml + ((base + s) * 16 + r) * 2);
-    sh_w[r][s] = ml.x;
-    sh_l[r][s] = ml.y;
-  }
-  __syncthreads();
-  if ((int)threadIdx.x < rows) {
-    const int r = threadIdx.x;
-    float m_all = -INFINITY;
-    for (int s = 0; s < splits; ++s) m_all = fmaxf(m_all, sh_w[r][s]);
-    float l_all = 0.f;
-    for (int s = 0; s < splits; ++s) {
-      const float ms = sh_w[r][s];
-      const float e = ms > -INFINITY ? exp2f(ms - m_all) : 0.f;
-      l_all += sh_l[r][s] * e;
-      sh_w[r][s] = e;
+  const int cols = rows * (D / 4);                       // float4 columns of the output
+  const int groups = cols <= 256 ? 256 / cols : 1;       // threads per column, each with its share of the splits
+  const int t = threadIdx.x;
+  const int grp = cols <= 256 ? t / cols : 0;
+  const int c0 = cols <= 256 ? t - grp * cols : t;
+  const bool active = grp < groups;
+
+  // this thread's first column: its first batch of partial accumulators is asked for now
+  float4 first[REDUCE_BATCH];
+#pragma unroll
+  for (int k = 0; k < REDUCE_BATCH; ++k) {
+    const int s = grp + k * groups;
+    first[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (active && c0 < cols && s < splits) {
+      const int r = c0 / (D / 4), d = 4 * (c0 - r * (D / 4));
+      first[k] = *reinterpret_cast<const float4*>(ws_acc + ((base + s) * 16 + r) * D + d);
     }
-    const float inv = 1.f / l_all;
-    for (int s = 0; s < splits; ++s) sh_w[r][s] *= inv;
+  }
+  // the splits' weights, a row per wavefront at a time: lane s holds split s
+  {
+    const int lane = t & 63, wave = t >> 6;
+    for (int r = wave; r < rows; r += 4) {
+      float2 ml = make_float2(-INFINITY, 0.f);
+      if (lane < splits) ml = *reinterpret_cast<const float2*>(ws_ml + ((base + lane) * 16 + r) * 2);
+      const float m_all = wave_max(ml.x);
+      const float e = ml.x > -INFINITY ? exp2f(ml.x - m_all) : 0.f;
+      const float l_all = wave_sum(ml.y * e);
+      if (lane < splits) sh_w[r][lane] = e / l_all;
+    }
   }
   __syncthreads();
-  for (int idx = threadIdx.x; idx < n_elems; idx += blockDim.x) {
-    const int r = idx / D, d = idx - r * D;
-    float o = 0.f;
-    if (splits <= 4 && idx == e0) {
-      for (int s = 0; s < splits; ++s) o += first[s] * sh_w[r][s];
-    } else {
-      const float* src = ws_acc + (base * 16 + r) * D + d;
-      int s = 0;
-      for (; s + 4 <= splits; s += 4) {  // four loads in flight at a time; an empty split's partial is zero
-        const float a0 = src[(size_t)(s + 0) * 16 * D], a1 = src[(size_t)(s + 1) * 16 * D];
-        const float a2 = src[(size_t)(s + 2) * 16 * D], a3 = src[(size_t)(s + 3) * 16 * D];
-        o += a0 * sh_w[r][s] + a1 * sh_w[r][s + 1] + a2 * sh_w[r][s + 2] + a3 * sh_w[r][s + 3];
+  for (int c = c0; c < cols; c += 256) {   // one pass unless there are more columns than threads
+    const int r = c / (D / 4), d = 4 * (c - r * (D / 4));
+    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (active) {
+      for (int k0 = 0; grp + k0 * groups < splits; k0 += REDUCE_BATCH) {
+        float4 a[REDUCE_BATCH];
+#pragma unroll
+        for (int k = 0; k < REDUCE_BATCH; ++k) {
+          const int s = grp + (k0 + k) * groups;
+          if (c == c0 && k0 == 0)
+            a[k] = first[k];
+          else
+            a[k] = s < splits ? *reinterpret_cast<const float4*>(ws_acc + ((base + s) * 16 + r) * D + d)
+                              : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int k = 0; k < REDUCE_BATCH; ++k) {  // an empty split's partial is zero and so is its weight
+          const int s = grp + (k0 + k) * groups;
+          const float w = s < splits ? sh_w[r][s] : 0.f;
+          o.x += a[k].x * w; o.y += a[k].y * w; o.z += a[k].z * w; o.w += a[k].w * w;
+        }
       }
-      for (; s < splits; ++s) o += src[(size_t)s * 16 * D] * sh_w[r][s];
     }
-    const int token = q0 + r / G, head = g_kv * G + r % G;
-    out[(size_t)token * Hq * D + (size_t)head * D + d] = float_to_bf16(o);
+    if (groups > 1) {
+      if (active && grp > 0) sh_part[t] = o;
+      __syncthreads();
+      if (grp == 0) {
+        for (int g2 = 1; g2 < groups; ++g2) {
+          const float4 p = sh_part[g2 * cols + c];
+          o.x += p.x; o.y += p.y; o.z += p.z; o.w += p.w;
+        }
+      }
+    }
+    if (grp == 0) {
+      const int token = q0 + r / G, head = g_kv * G + r % G;
+      union {
+        uint2 u;
+        bf16_t e[4];
+      } pk;
+      pk.e[0] = float_to_bf16(o.x); pk.e[1] = float_to_bf16(o.y);
+      pk.e[2] = float_to_bf16(o.z); pk.e[3] = float_to_bf16(o.w);
+      *reinterpret_cast<uint2*>(out + (size_t)token * Hq * D + (size_t)head * D + d) = pk.u;
+    }
   }
 }
 

@@ -22,8 +22,9 @@ from qwen3_from_scratch_amd.models import DecoderModel, LayerSpec, ModelSpec, Ru
 from qwen3_from_scratch_amd.parts import CacheNeed, Part, PartSpec, Precision
 from qwen3_from_scratch_amd.weights import RandomWeights
 
-H, V, HQ, HKV, D, I = 48, 97, 4, 2, 16, 80
+V, HQ, HKV, I = 97, 4, 2, 80
 EPS, THETA, WINDOW, MAXPOS = 1e-5, 10000.0, 19, 512
+H, D = 48, 16                 # the default sizes; `sizes()` swaps in others for one test
 
 
 @register_part("mixer", "toy_running_mean")
@@ -87,7 +88,7 @@ class LearnedPosition(Part):
         return None
 
 
-def toy_spec(position):
+def toy_spec(position, with_state=True):
     norm = PartSpec.of("norm", "rms", size=H, eps=EPS)
     attn = dict(hidden_size=H, num_heads=HQ, num_kv_heads=HKV, head_dim=D, qk_norm=True, qk_norm_eps=EPS)
     ff = PartSpec.of("feed_forward", "swiglu", hidden_size=H, intermediate_size=I)
@@ -98,7 +99,8 @@ def toy_spec(position):
 
     layers = (
         layer(0, PartSpec.of("mixer", "attention", window=0, **attn)),
-        layer(1, PartSpec.of("mixer", "toy_running_mean", hidden_size=H)),
+        layer(1, PartSpec.of("mixer", "toy_running_mean", hidden_size=H) if with_state
+              else PartSpec.of("mixer", "attention", window=0, **dict(attn, qk_norm=False))),
         layer(2, PartSpec.of("mixer", "attention", window=WINDOW, **attn)),
         layer(3, PartSpec.of("mixer", "attention", window=0, **dict(attn, qk_norm=False))),
     )
@@ -154,8 +156,8 @@ def plain_toy_logits(w, spec, position, tokens):
     return plain.rms_norm(x, w["toy.norm.weight"], EPS) @ w["toy.head.weight"].T
 
 
-def build(position, dtype, device):
-    spec = toy_spec(position)
+def build(position, dtype, device, with_state=True):
+    spec = toy_spec(position, with_state)
     model = DecoderModel(spec, Precision.named(dtype), device)
     source = RandomWeights(model.tensors(), seed=3, std=0.08, norm_jitter=0.2)
     model.load(source)
@@ -163,17 +165,20 @@ def build(position, dtype, device):
     return spec, model, weights
 
 
-def check(position, dtype, device, tol):
-    spec, model, weights = build(position, dtype, device)
-    assert not model.graph_safe()                       # the toy mixer says it is not: it runs without graphs
+def check(position, dtype, device, tol, with_state=True, page=8):
+    spec, model, weights = build(position, dtype, device, with_state)
     needs = model.plane_needs
-    assert [n.window for n in needs if n.paged] == [0, WINDOW, 0] and needs[1].has_state
+    if with_state:
+        assert not model.graph_safe()                   # the toy mixer says it is not: it runs without graphs
+        assert [n.window for n in needs if n.paged] == [0, WINDOW, 0] and needs[1].has_state
+    else:
+        assert model.graph_safe() and [n.window for n in needs if n.paged] == [0, 0, WINDOW, 0]
     requests = {"t%d" % i: random_tokens(n, V, 30 + i) for i, n in enumerate([70, 9, 41, 130, 25])}
     want = {rid: plain_toy_logits(weights, spec, position, toks) for rid, toks in requests.items()}
     for make in (trace_whole, trace_tail_decoded, trace_portions, trace_mixed):
         steps = make(requests)
-        runner = ModelRunner(model, page_size=8, num_pages=max_live_tokens(steps, page=8) // 8, max_requests=4)
-        assert len(runner.manager.groups) == 2 and len(runner.manager.state_groups) == 1
+        runner = ModelRunner(model, page_size=page, num_pages=max_live_tokens(steps, page=page) // page, max_requests=4)
+        assert len(runner.manager.groups) == 2 and len(runner.manager.state_groups) == (1 if with_state else 0)
         got = run_trace(runner, steps)
         worst = max(float((got[(rid, p)] - logits[p]).abs().max())
                     for rid, logits in want.items() for p in range(logits.shape[0]))
@@ -191,6 +196,23 @@ def test_toy_model_on_the_host(cpu_ops, position):
 @pytest.mark.parametrize("dtype,tol", [("float32", 5e-4), ("bfloat16", 0.25)])
 def test_toy_model_on_the_gpu(position, dtype, tol):
     check(position, dtype, "cuda", tol)
+
+
+@pytest.fixture
+def graph_sizes(monkeypatch):
+    """Sizes the matrix-core and few-row kernels take (head 64, width 64), so that a model of
+    built-in parts alone goes through graph replays, the fused decoding kernel and the norm
+    fusion, with a window and a layer that reads another's cache in play."""
+    import sys
+    module = sys.modules[__name__]
+    monkeypatch.setattr(module, "H", 64)
+    monkeypatch.setattr(module, "D", 64)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,tol", [("float32", 5e-4), ("bfloat16", 0.25)])
+def test_windows_and_shared_caches_through_graph_replays(graph_sizes, dtype, tol):
+    check("rotary", dtype, "cuda", tol, with_state=False, page=16)
 
 
 def test_a_window_frees_pages_while_the_request_lives(cpu_ops):

@@ -131,14 +131,13 @@ __global__ void qk_norm_rope_store_kernel(T* __restrict__ qkv, const W* __restri
 // STORE_V the value heads are handled here too, element by element into the transposed
 // cache (for steps of few tokens, where a second launch would cost more than it saves).
 template <typename W, int LPH, bool STORE_V>
-__global__ __launch_bounds__(256) void qk_norm_rope_store_vec_kernel(
-    bf16_t* __restrict__ qkv, const W* __restrict__ q_weight, const W* __restrict__ k_weight, float eps,
-    const float* __restrict__ table, int max_pos, const int* __restrict__ positions,
+__device__ __forceinline__ void qk_vec_body(
+    int t, int head_block, bf16_t* __restrict__ qkv, const W* __restrict__ q_weight, const W* __restrict__ k_weight,
+    float eps, const float* __restrict__ table, int max_pos, const int* __restrict__ positions,
     const int* __restrict__ seq_index, const int* __restrict__ block_table, int bt_stride, int bt_rows,
     bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache, int page_size, int num_pages, int Hq, int Hkv) {
   constexpr int D = LPH * 16, HALF = D / 2;
-  const int t = blockIdx.x;
-  const int head = blockIdx.y * (256 / LPH) + threadIdx.x / LPH;
+  const int head = head_block * (256 / LPH) + threadIdx.x / LPH;
   const int c = threadIdx.x % LPH;  // which eight of the half
   if (head >= Hq + (STORE_V ? 2 : 1) * Hkv) return;
   bf16_t* src = qkv + ((size_t)t * (Hq + 2 * Hkv) + head) * D;
@@ -206,23 +205,32 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_vec_kernel(
   *reinterpret_cast<uint4*>(dst + HALF + 8 * c) = x2.u;
 }
 
-// Values of this step into the transposed value cache, one block per (logical
+template <typename W, int LPH, bool STORE_V>
+__global__ __launch_bounds__(256) void qk_norm_rope_store_vec_kernel(
+    bf16_t* __restrict__ qkv, const W* __restrict__ q_weight, const W* __restrict__ k_weight, float eps,
+    const float* __restrict__ table, int max_pos, const int* __restrict__ positions,
+    const int* __restrict__ seq_index, const int* __restrict__ block_table, int bt_stride, int bt_rows,
+    bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache, int page_size, int num_pages, int Hq, int Hkv) {
+  qk_vec_body<W, LPH, STORE_V>(blockIdx.x, blockIdx.y, qkv, q_weight, k_weight, eps, table, max_pos, positions,
+                               seq_index, block_table, bt_stride, bt_rows, k_cache, v_cache, page_size, num_pages,
+                               Hq, Hkv);
+}
+
+// Values of this step into the transposed value cache, the work of one block for (logical
 // page j of the step's span, key head, sequence): the rows of the up to
 // `page_size` (<= 64) tokens that fall in the page are staged in shared memory and
 // written as rows of the page, 16 bytes at a time where eight neighbouring slots
 // are all written in this step, element by element otherwise.
 template <int D>
-__global__ __launch_bounds__(256) void store_values_kernel(
-    const bf16_t* __restrict__ qkv, const int* __restrict__ cu_q, const int* __restrict__ kv_lens,
-    const int* __restrict__ block_table, int bt_stride, bf16_t* __restrict__ v_cache, int page_size,
-    int num_pages, int Hq, int Hkv) {
-  __shared__ bf16_t tile[64][D + 8];
-  const int b = blockIdx.z, g = blockIdx.y;
+__device__ __forceinline__ void store_values_body(
+    int span_page, int g, int b, bf16_t (*tile)[D + 8], const bf16_t* __restrict__ qkv,
+    const int* __restrict__ cu_q, const int* __restrict__ kv_lens, const int* __restrict__ block_table,
+    int bt_stride, bf16_t* __restrict__ v_cache, int page_size, int num_pages, int Hq, int Hkv) {
   const int q0 = cu_q[b];
   const int q_len = cu_q[b + 1] - q0;
   if (q_len <= 0) return;
   const int first_pos = kv_lens[b] - q_len;
-  const int blk = first_pos / page_size + blockIdx.x;       // logical page
+  const int blk = first_pos / page_size + span_page;        // logical page
   const int lo = max(first_pos, blk * page_size);           // positions written in it: [lo, hi)
   const int hi = min(first_pos + q_len, (blk + 1) * page_size);
   if (lo >= hi) return;
@@ -255,6 +263,33 @@ __global__ __launch_bounds__(256) void store_values_kernel(
       }
     }
   }
+}
+
+// Both kinds of block in one launch, for steps of many tokens: the first `value_blocks` blocks
+// (span_pages x Hkv x B of them) transpose values, the others prepare queries and keys. The
+// two touch different parts of qkv and different caches, so they need no order, and a launch
+// of its own for the values, which is short on work per block, would only add its latency.
+template <typename W, int LPH>
+__global__ __launch_bounds__(256) void qk_and_values_kernel(
+    bf16_t* __restrict__ qkv, const W* __restrict__ q_weight, const W* __restrict__ k_weight, float eps,
+    const float* __restrict__ table, int max_pos, const int* __restrict__ positions,
+    const int* __restrict__ seq_index, const int* __restrict__ block_table, int bt_stride, int bt_rows,
+    bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache, int page_size, int num_pages, int Hq, int Hkv,
+    const int* __restrict__ cu_q, const int* __restrict__ kv_lens, int span_pages, int value_blocks,
+    int head_blocks) {
+  constexpr int D = LPH * 16;
+  __shared__ bf16_t tile[64][D + 8];
+  int id = blockIdx.x;
+  if (id < value_blocks) {
+    const int span_page = id % span_pages, g = (id / span_pages) % Hkv, b = id / (span_pages * Hkv);
+    store_values_body<D>(span_page, g, b, tile, qkv, cu_q, kv_lens, block_table, bt_stride, v_cache, page_size,
+                         num_pages, Hq, Hkv);
+    return;
+  }
+  id -= value_blocks;
+  qk_vec_body<W, LPH, false>(id / head_blocks, id % head_blocks, qkv, q_weight, k_weight, eps, table, max_pos,
+                             positions, seq_index, block_table, bt_stride, bt_rows, k_cache, v_cache, page_size,
+                             num_pages, Hq, Hkv);
 }
 
 extern "C" int q3_rope_table(const float* inv_freq, float* table, int max_pos, int half,
@@ -300,21 +335,32 @@ static int launch_qk_vec(void* qkv, const void* qw, const void* kw, float eps, c
                          int bt_rows, void* k_cache, void* v_cache, int page_size, int num_pages, int T_, int Hq,
                          int Hkv, int D, const int* cu_q, const int* kv_lens, int B, int max_q_len,
                          hipStream_t stream) {
-  const bool few = max_q_len < 8;  // values element by element in the same launch
+  const bool few = max_q_len < 8;  // values element by element by the lanes that prepare queries and keys
+  const bool values_apart = v_cache != nullptr && !few;
   const int nheads = Hq + (few ? 2 : 1) * Hkv;
-#define Q3_QKV_LAUNCH(LPH)                                                                                   \
-  do {                                                                                                       \
-    const dim3 grid(T_, (nheads + 256 / LPH - 1) / (256 / LPH));                                             \
-    if (few)                                                                                                 \
-      hipLaunchKernelGGL((qk_norm_rope_store_vec_kernel<W, LPH, true>), grid, dim3(256), 0, stream,          \
+  const int span_pages = values_apart ? (max_q_len + page_size - 1) / page_size + 1 : 0;
+  const long value_blocks = values_apart ? (long)span_pages * Hkv * B : 0;
+#define Q3_QKV_LAUNCH(LPH)                                                                                    \
+  do {                                                                                                        \
+    const int head_blocks = (nheads + 256 / LPH - 1) / (256 / LPH);                                           \
+    if (values_apart) {                                                                                       \
+      const long blocks = value_blocks + (long)T_ * head_blocks;                                              \
+      if (blocks > 0x7fffffffL) return Q3_ERR_UNSUPPORTED;                                                    \
+      hipLaunchKernelGGL((qk_and_values_kernel<W, LPH>), dim3((unsigned)blocks), dim3(256), 0, stream,        \
                          (bf16_t*)qkv, (const W*)qw, (const W*)kw, eps, table, max_pos, positions, seq_index, \
-                         block_table, bt_stride, bt_rows, (bf16_t*)k_cache, (bf16_t*)v_cache, page_size,     \
-                         num_pages, Hq, Hkv);                                                                \
-    else                                                                                                     \
-      hipLaunchKernelGGL((qk_norm_rope_store_vec_kernel<W, LPH, false>), grid, dim3(256), 0, stream,         \
-                         (bf16_t*)qkv, (const W*)qw, (const W*)kw, eps, table, max_pos, positions, seq_index, \
-                         block_table, bt_stride, bt_rows, (bf16_t*)k_cache, (bf16_t*)v_cache, page_size,     \
-                         num_pages, Hq, Hkv);                                                                \
+                         block_table, bt_stride, bt_rows, (bf16_t*)k_cache, (bf16_t*)v_cache, page_size,      \
+                         num_pages, Hq, Hkv, cu_q, kv_lens, span_pages, (int)value_blocks, head_blocks);      \
+    } else if (few) {                                                                                         \
+      hipLaunchKernelGGL((qk_norm_rope_store_vec_kernel<W, LPH, true>), dim3(T_, head_blocks), dim3(256), 0,  \
+                         stream, (bf16_t*)qkv, (const W*)qw, (const W*)kw, eps, table, max_pos, positions,    \
+                         seq_index, block_table, bt_stride, bt_rows, (bf16_t*)k_cache, (bf16_t*)v_cache,      \
+                         page_size, num_pages, Hq, Hkv);                                                      \
+    } else {                                                                                                  \
+      hipLaunchKernelGGL((qk_norm_rope_store_vec_kernel<W, LPH, false>), dim3(T_, head_blocks), dim3(256), 0, \
+                         stream, (bf16_t*)qkv, (const W*)qw, (const W*)kw, eps, table, max_pos, positions,    \
+                         seq_index, block_table, bt_stride, bt_rows, (bf16_t*)k_cache, (bf16_t*)v_cache,      \
+                         page_size, num_pages, Hq, Hkv);                                                      \
+    }                                                                                                         \
   } while (0)
   switch (D) {
     case 16: Q3_QKV_LAUNCH(1); break;
@@ -325,20 +371,6 @@ static int launch_qk_vec(void* qkv, const void* qw, const void* kw, float eps, c
     default: return Q3_ERR_UNSUPPORTED;
   }
 #undef Q3_QKV_LAUNCH
-  if (v_cache != nullptr && !few) {
-    const dim3 grid((max_q_len + page_size - 1) / page_size + 1, Hkv, B);
-#define Q3_V_LAUNCH(DD)                                                                                       \
-  hipLaunchKernelGGL(store_values_kernel<DD>, grid, dim3(256), 0, stream, (const bf16_t*)qkv, cu_q, kv_lens, \
-                     block_table, bt_stride, (bf16_t*)v_cache, page_size, num_pages, Hq, Hkv)
-    switch (D) {
-      case 16: Q3_V_LAUNCH(16); break;
-      case 32: Q3_V_LAUNCH(32); break;
-      case 64: Q3_V_LAUNCH(64); break;
-      case 128: Q3_V_LAUNCH(128); break;
-      case 256: Q3_V_LAUNCH(256); break;
-    }
-#undef Q3_V_LAUNCH
-  }
   return q3_launch_status();
 }
 

@@ -111,3 +111,57 @@ def test_abort_while_a_step_is_ahead(cpu_ops, model_folders):
     assert len(b.generated) == 30 and engine.runner.manager.num_free() == 16
     solo = SyncEngine(path=model_folders["A"], dtype="float32", device="cpu", num_blocks=16, max_num_seqs=2)
     assert solo.generate_ids([b.prompt], 30, temperature=0.0, ignore_eos=True)[0] == b.generated
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_a_step_ahead_under_random_arrivals(cpu_ops, model_folders, seed):
+    """Random prompts, counts, sampling options, arrival steps, end-of-sequence sets, page
+    budgets and aborts: the engine that looks a step ahead produces what the one that does not
+    produces, request by request, and gives every page back."""
+    import random
+
+    rng = random.Random(seed)
+    vocab = TINY["A"]["config"]["vocab_size"]
+    num_blocks = rng.choice([8, 12, 30])
+    eos = tuple(rng.sample(range(vocab), rng.choice([0, 8, 40])))
+    plan = []
+    for i in range(rng.randint(3, 7)):
+        n, new = rng.randint(1, 40), rng.randint(1, 30)
+        if n + new > 16 * num_blocks:
+            continue
+        sampling = rng.choice([dict(temperature=0.0), dict(temperature=0.8, seed=rng.randint(0, 99)),
+                               dict(temperature=1.1, top_k=rng.randint(1, 9), seed=rng.randint(0, 99))])
+        plan.append(dict(at=rng.randint(0, 25), prompt=random_tokens(n, vocab, 1000 * seed + i), new=new,
+                         ignore=rng.random() < 0.5, sampling=sampling,
+                         abort_after=rng.choice([None, None, None, rng.randint(1, 10)])))
+
+    def run(lookahead):
+        engine = SyncEngine(path=model_folders["A"], dtype="float32", device="cpu", block_size=16,
+                            num_blocks=num_blocks, max_num_seqs=3, chunked_prefill_size=rng.choice([8, 64]))
+        engine.lookahead = lookahead
+        engine.eos_ids = eos
+        live, out = {}, {}
+        step = 0
+        while step < 600 and (engine.scheduler.has_work() or step <= 25):
+            for i, item in enumerate(plan):
+                if item["at"] == step:
+                    params = engine.default_params(item["new"], ignore_eos=item["ignore"], **item["sampling"])
+                    live[i] = engine.add_request(item["prompt"], params)
+            for i, request in list(live.items()):
+                limit = plan[i]["abort_after"]
+                if limit is not None and len(request.generated) >= limit and request.status.name != "FINISHED":
+                    engine.abort(request)
+            engine.step()
+            engine.runner.manager.audit()
+            step += 1
+        assert not engine.scheduler.has_work()
+        assert engine.runner.manager.num_free() == num_blocks
+        for i, request in live.items():
+            limit = plan[i]["abort_after"]
+            out[i] = request.generated if limit is None else request.generated[:limit]   # an abort lands a step later when ahead
+        return out
+
+    state = rng.getstate()
+    plain = run(False)
+    rng.setstate(state)
+    assert run(True) == plain

@@ -774,15 +774,12 @@ __global__ __launch_bounds__(256) void attn_decode_reduce_kernel(
 // ---- sequences with many rows: portions of prompts ----------------------------
 // grid (row tiles, Hkv, B), 256 threads; a block owns 128 / G tokens x G heads,
 // each wavefront 32 rows of them (two blocks of 16). The block's threads bring
-// each 64-key tile from the cache into shared memory once, 16 bytes per load,
-// two tiles in flight (the next tile's loads are issued before the current
-// tile's arithmetic and stored after it); the wavefronts read their matrix-core
-// operands from there. K rows are padded by 16 bytes so that the sixteen rows a
-// read touches fall in different banks; V^T rows hold each 32-key half of the
-// tile in the order the P operand has it (for lane group g: keys 4g..4g+3 of the
-// half's first 16-key block, then of its second), so a V^T operand is one
-// 16-byte read. Two stages of a 64-key tile take 72 KB of the CU's 160 KB, so two
-// blocks share a CU. The first half of the key heads takes its row tiles from the
+// each 64-key tile from the cache into shared memory once, with loads that write
+// shared memory directly (no registers in between), the next tile's while the
+// current tile is worked on; the wavefronts read their matrix-core operands from
+// there. The 16-byte pieces of a tile are placed so that the sixteen rows an operand
+// read touches fall in different banks (see PrefillSmem). Two stages of a 64-key
+// tile take 64 KB of the CU's 160 KB, so two blocks share a CU. The first half of the key heads takes its row tiles from the
 // sequence's end, the second half from its start, so that the blocks which come
 // to share a CU add up to about the same work. Block-table entries are copied to
 // shared memory PREFILL_PAGES at a time, so that no cache load waits for a table load.
@@ -790,11 +787,19 @@ __global__ __launch_bounds__(256) void attn_decode_reduce_kernel(
 #define PF_TILE 64
 template <int D>
 struct PrefillSmem {
-  static constexpr int K_ROW = D * 2 + 16;        // bytes
-  static constexpr int V_ROW = PF_TILE * 2 + 16;  // 64 keys * 2 bytes + pad
-  static constexpr int K_BYTES = PF_TILE * K_ROW;
-  static constexpr int V_BYTES = D * V_ROW;
+  // A stage holds a tile's keys (PF_TILE rows of D) and values (D rows of PF_TILE), both as
+  // 16-byte pieces in an order chosen so that the matrix-core operand reads spread over all
+  // banks without padding (the loads that fill a stage write whole kilobytes, see below).
+  // Keys: pieces of 256-byte windows, a window = RPW rows of CPR pieces; piece c of row r sits
+  // at place (r % RPW) * CPR + (c ^ (window % CPR)) of window r / RPW. Values: a window = two
+  // rows of eight pieces (a piece = eight keys of one 16-key block: q = 2 * block + half);
+  // piece q of row d sits at place (d % 2) * 8 + (q ^ (window % 8)) of window d / 2.
+  static constexpr int CPR = D / 8;          // 16-byte pieces per key row
+  static constexpr int RPW = 16 / CPR > 0 ? 16 / CPR : 1;   // key rows per window (D <= 128)
+  static constexpr int K_BYTES = PF_TILE * D * 2;
+  static constexpr int V_BYTES = D * PF_TILE * 2;
   static constexpr int STAGE = K_BYTES + V_BYTES;
+  static constexpr int K_PIECES = K_BYTES / 16, V_PIECES = V_BYTES / 16;
 };
 
 // The softmax update of one block of 16 rows for one 64-key tile: as softmax_step, over
@@ -915,83 +920,107 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
   if (window > 0 && pos_max >= 0) my_lo = max(0, pos_min - window + 1) / PF_TILE;
   const int* bt_row = block_table + (size_t)b * bt_stride;
 
-  constexpr int CHUNKS = D / 32;  // 16-byte chunks of K, and of V, per thread and tile
-  uint4 kreg[CHUNKS], vreg[CHUNKS];
+  // The copy of a tile from the caches into a stage. Place s (a 16-byte piece) of the keys'
+  // or values' part of a stage is filled by thread s % 256 in its turn s / 256: a wavefront's
+  // 64 lanes fill one contiguous kilobyte per turn, which is what a load that writes shared
+  // memory directly asks for (lane L's 16 bytes land at the wavefront's base + 16 L; the
+  // global address is each lane's own). Tiles that lie whole inside the sequence, with no
+  // page given back, are copied that way, without passing through registers; the others go
+  // through registers, where what lies past the sequence's end is zeroed.
+  constexpr int K_TURNS = SM::K_PIECES / 256, V_TURNS = SM::V_PIECES / 256;
   int page_base = 0;  // sh_pages[i] is the table's entry page_base + i
-
-  // per-thread constants of the copy: which 16-key block, which row and chunk of it
   const int page_shift = 31 - __clz(page);  // the page size is a power of two here
-  int c_kb[CHUNKS], c_koff[CHUNKS], c_voff[CHUNKS], c_h[CHUNKS];
+  // which piece of which row a place holds: keys (row of the tile, element offset), values
+  // (16-key block, row d, half of the block)
+  int k_row[K_TURNS], k_off[K_TURNS], v_kb[V_TURNS], v_d[V_TURNS], v_h[V_TURNS];
 #pragma unroll
-  for (int u = 0; u < CHUNKS; ++u) {
-    const int idx = tid + 256 * u;
-    c_kb[u] = idx / (2 * D);
-    c_koff[u] = ((idx / (D / 8)) % 16) * D + 8 * (idx % (D / 8));
-    c_h[u] = idx & 1;
-    c_voff[u] = ((idx >> 1) % D) * page + 8 * c_h[u];
+  for (int j = 0; j < K_TURNS; ++j) {
+    const int place = tid + 256 * j, w = place >> 4, u = place & 15;
+    k_row[j] = w * SM::RPW + u / SM::CPR;
+    k_off[j] = 8 * ((u % SM::CPR) ^ (w % SM::CPR));
+  }
+#pragma unroll
+  for (int j = 0; j < V_TURNS; ++j) {
+    const int place = tid + 256 * j, w = place >> 4, u = place & 15;
+    const int q = (u & 7) ^ (w & 7);
+    v_d[j] = 2 * w + (u >> 3);
+    v_kb[j] = q >> 1;
+    v_h[j] = q & 1;
   }
   const size_t page_elems = (size_t)page * D;  // elements of one (page, head) in either cache
+  typedef __attribute__((address_space(3))) void* lds_ptr;
 
-  auto fetch = [&](int t) {
+  auto plain_tile = [&](int t) { return t * PF_TILE + PF_TILE <= kv_len && window == 0; };
+  auto copy_direct = [&](int t, int stage) {
     const int key0 = t * PF_TILE;
-    if (key0 + PF_TILE <= kv_len && window == 0) {
-      // the whole tile lies inside the sequence and no page has been given back: no checks
+    unsigned char* ks = smem + stage * SM::STAGE + 1024 * wave;  // this wavefront's kilobyte of each turn
+    unsigned char* vs = ks + SM::K_BYTES;
 #pragma unroll
-      for (int u = 0; u < CHUNKS; ++u) {
-        const int kbase = key0 + 16 * c_kb[u];
-        int pg = sh_pages[(kbase >> page_shift) - page_base];
-        pg = min(max(pg, 0), num_pages - 1);
-        const size_t base = (size_t)(pg * Hkv + g_kv) * page_elems;
-        const int slot0 = kbase & (page - 1);
-        kreg[u] = *reinterpret_cast<const uint4*>(k_cache + base + (slot0 * D + c_koff[u]));
-        vreg[u] = *reinterpret_cast<const uint4*>(v_cache + base + (c_voff[u] + slot0));
-      }
-      return;
+    for (int j = 0; j < K_TURNS; ++j) {
+      const int key = key0 + k_row[j];
+      int pg = sh_pages[(key >> page_shift) - page_base];
+      pg = min(max(pg, 0), num_pages - 1);
+      const bf16_t* src = k_cache + (size_t)(pg * Hkv + g_kv) * page_elems + ((key & (page - 1)) * D + k_off[j]);
+      __builtin_amdgcn_global_load_lds(src, (lds_ptr)(ks + 4096 * j), 16, 0, 0);
     }
 #pragma unroll
-    for (int u = 0; u < CHUNKS; ++u) {
-      const int kbase = key0 + 16 * c_kb[u];
-      kreg[u] = make_uint4(0, 0, 0, 0);
-      vreg[u] = make_uint4(0, 0, 0, 0);
-      if (kbase < kv_len) {
-        const int pg = sh_pages[(kbase >> page_shift) - page_base];
-        if (pg >= 0 && pg < num_pages) {
-          const size_t base = (size_t)(pg * Hkv + g_kv) * page_elems;
-          const int slot0 = kbase & (page - 1);
-          // K: chunk c of key row r of the block (rows past the end are zero)
-          if (kbase + (c_koff[u] / D) < kv_len)
-            kreg[u] = *reinterpret_cast<const uint4*>(k_cache + base + (slot0 * D + c_koff[u]));
-          // V^T: half h (8 slots) of row d of the block
-          if (kbase + 8 * c_h[u] < kv_len) {
-            Pack16 v;
-            v.u = *reinterpret_cast<const uint4*>(v_cache + base + (c_voff[u] + slot0));
-            if (kbase + 8 * c_h[u] + 8 > kv_len) {  // slots past the end hold anything: zero them (0 * NaN is NaN)
-#pragma unroll
-              for (int j = 0; j < 8; ++j)
-                if (kbase + 8 * c_h[u] + j >= kv_len) v.e[j] = (__bf16)0.f;
-            }
-            vreg[u] = v.u;
-          }
-        }
-      }
+    for (int j = 0; j < V_TURNS; ++j) {
+      const int key = key0 + 16 * v_kb[j];
+      int pg = sh_pages[(key >> page_shift) - page_base];
+      pg = min(max(pg, 0), num_pages - 1);
+      const bf16_t* src =
+          v_cache + (size_t)(pg * Hkv + g_kv) * page_elems + (v_d[j] * page + (key & (page - 1)) + 8 * v_h[j]);
+      __builtin_amdgcn_global_load_lds(src, (lds_ptr)(vs + 4096 * j), 16, 0, 0);
     }
   };
-  auto stash = [&](int stage) {
+  auto copy_checked = [&](int t, int stage) {
+    const int key0 = t * PF_TILE;
     unsigned char* ks = smem + stage * SM::STAGE;
     unsigned char* vs = ks + SM::K_BYTES;
 #pragma unroll
-    for (int u = 0; u < CHUNKS; ++u) {
-      const int idx = tid + 256 * u;
-      const int r = idx / (D / 8), c = idx % (D / 8);
-      *reinterpret_cast<uint4*>(ks + r * SM::K_ROW + 16 * c) = kreg[u];
-      const int h = idx & 1, d = (idx >> 1) % D, kb4 = idx / (2 * D);
-      // within a 32-key half: keys 8h..8h+3 of a 16-key block belong to lane group 2h, keys
-      // 8h+4..8h+7 to group 2h+1; within a group's 16 bytes the half's first block comes first
-      unsigned char* row = vs + d * SM::V_ROW + 64 * (kb4 >> 1) + 8 * (kb4 & 1);
-      *reinterpret_cast<uint2*>(row + 16 * (2 * h)) = make_uint2(vreg[u].x, vreg[u].y);
-      *reinterpret_cast<uint2*>(row + 16 * (2 * h + 1)) = make_uint2(vreg[u].z, vreg[u].w);
+    for (int j = 0; j < K_TURNS; ++j) {
+      const int key = key0 + k_row[j];
+      uint4 piece = make_uint4(0, 0, 0, 0);  // rows past the end are zero
+      if (key < kv_len) {
+        const int pg = sh_pages[(key >> page_shift) - page_base];
+        if (pg >= 0 && pg < num_pages)
+          piece = *reinterpret_cast<const uint4*>(k_cache + (size_t)(pg * Hkv + g_kv) * page_elems +
+                                                  ((key & (page - 1)) * D + k_off[j]));
+      }
+      *reinterpret_cast<uint4*>(ks + 16 * (tid + 256 * j)) = piece;
+    }
+#pragma unroll
+    for (int j = 0; j < V_TURNS; ++j) {
+      const int key = key0 + 16 * v_kb[j] + 8 * v_h[j];  // the first of the piece's eight keys
+      Pack16 piece;
+      piece.u = make_uint4(0, 0, 0, 0);
+      if (key < kv_len) {
+        const int pg = sh_pages[(key >> page_shift) - page_base];
+        if (pg >= 0 && pg < num_pages) {
+          piece.u = *reinterpret_cast<const uint4*>(v_cache + (size_t)(pg * Hkv + g_kv) * page_elems +
+                                                    (v_d[j] * page + (key & (page - 1))));
+          if (key + 8 > kv_len) {  // slots past the end hold anything: zero them (0 * NaN is NaN)
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+              if (key + i >= kv_len) piece.e[i] = (__bf16)0.f;
+          }
+        }
+      }
+      *reinterpret_cast<uint4*>(vs + 16 * (tid + 256 * j)) = piece.u;
     }
   };
+  auto copy_tile = [&](int t, int stage) {
+    if (plain_tile(t))
+      copy_direct(t, stage);
+    else
+      copy_checked(t, stage);
+  };
+  // the operand reads' addresses: this lane's window and swizzle for the key rows 16 kb4 + col
+  // and for the value rows 16 nb + col
+  const int k_lane = (col / SM::RPW) * 256 + (col % SM::RPW) * SM::CPR * 16;
+  const int k_swz = (col / SM::RPW) % SM::CPR;
+  const int v_lane = (col >> 1) * 256 + (col & 1) * 128 + 8 * (grp & 1);
+  const int v_swz = (col >> 1) & 7;
 
   // tiles are worked through in spans whose table entries fit sh_pages
   const int tiles_per_span = max(1, (PREFILL_PAGES - 4) * (page / 16) / 4);
@@ -1004,13 +1033,14 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
       for (int i = tid; page_base + i <= last_page; i += 256) sh_pages[i] = bt_row[page_base + i];
     }
     __syncthreads();
-    fetch(span_lo);
-    stash(0);
+    copy_tile(span_lo, 0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     for (int t = span_lo; t < span_hi; ++t) {
       const int stage = (t - span_lo) & 1;
       const bool more = t + 1 < span_hi;
-      if (more) fetch(t + 1);
+      // the next tile into the other stage, which every wavefront left at the last barrier
+      if (more) copy_tile(t + 1, stage ^ 1);
       if (t >= my_lo && t < my_hi) {
         const unsigned char* ks = smem + stage * SM::STAGE;
         const unsigned char* vs = ks + SM::K_BYTES;
@@ -1021,7 +1051,8 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
           Pack16 a[D / 32];
 #pragma unroll
           for (int i = 0; i < D / 32; ++i)
-            a[i].u = *reinterpret_cast<const uint4*>(ks + (16 * kb4 + col) * SM::K_ROW + 64 * i + 16 * grp);
+            a[i].u = *reinterpret_cast<const uint4*>(ks + (16 / SM::RPW) * 256 * kb4 + k_lane +
+                                                     16 * ((4 * i + grp) ^ k_swz));
 #pragma unroll
           for (int qb = 0; qb < 2; ++qb) {
             f32x4_t c = {0.f, 0.f, 0.f, 0.f};
@@ -1042,14 +1073,17 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
         for (int nb = 0; nb < D / 16; ++nb)
 #pragma unroll
           for (int half = 0; half < 2; ++half) {
-            Pack16 vt;
-            vt.u = *reinterpret_cast<const uint4*>(vs + (16 * nb + col) * SM::V_ROW + 64 * half + 16 * grp);
+            Pack16 vt;  // keys 4 grp .. 4 grp + 3 of the half's two 16-key blocks
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+              vt.h[kb] = *reinterpret_cast<const uint2*>(vs + 2048 * nb + v_lane +
+                                                        16 * ((2 * (2 * half + kb) + (grp >> 1)) ^ v_swz));
 #pragma unroll
             for (int qb = 0; qb < 2; ++qb)
               acc[qb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt.v, p[qb][half].v, acc[qb][nb], 0, 0, 0);
           }
       }
-      if (more) stash(stage ^ 1);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's share of the next tile has landed
       __syncthreads();
     }
   }

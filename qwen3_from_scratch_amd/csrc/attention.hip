@@ -783,37 +783,44 @@ __global__ __launch_bounds__(256) void attn_decode_reduce_kernel(
 // sequence's end, the second half from its start, so that the blocks which come
 // to share a CU add up to about the same work. Block-table entries are copied to
 // shared memory PREFILL_PAGES at a time, so that no cache load waits for a table load.
-#define PREFILL_PAGES 1024
-#define PF_TILE 64
-template <int D>
+#define PREFILL_PAGES 512
+// (measured for one 2,048-token prompt at head size 128: 64-key tiles in two stages 94 us, 32-key
+// tiles in four stages, which have three tiles on their way, 116 us; three stages of 64 keys
+// leave room for one block a CU only, 184 us)
+#define PF_TILE 64    // keys per tile
+#define PF_STAGES 2  // tiles in shared memory: one being worked on, the others on their way
+template <int D, int TILE>
 struct PrefillSmem {
-  // A stage holds a tile's keys (PF_TILE rows of D) and values (D rows of PF_TILE), both as
+  // A stage holds a tile's keys (TILE rows of D) and values (D rows of TILE), both as
   // 16-byte pieces in an order chosen so that the matrix-core operand reads spread over all
   // banks without padding (the loads that fill a stage write whole kilobytes, see below).
-  // Keys: pieces of 256-byte windows, a window = RPW rows of CPR pieces; piece c of row r sits
-  // at place (r % RPW) * CPR + (c ^ (window % CPR)) of window r / RPW. Values: a window = two
-  // rows of eight pieces (a piece = eight keys of one 16-key block: q = 2 * block + half);
-  // piece q of row d sits at place (d % 2) * 8 + (q ^ (window % 8)) of window d / 2.
+  // A window is 256 bytes. Keys: a window = RPW rows of CPR pieces; piece c of row r sits at
+  // place (r % RPW) * CPR + (c ^ (window % CPR)) of window r / RPW. Values: a window = VRW
+  // rows of VPR pieces (a piece = eight keys of one 16-key block: q = 2 * block + half);
+  // piece q of row d sits at place (d % VRW) * VPR + (q ^ (window % VPR)) of window d / VRW.
   static constexpr int CPR = D / 8;          // 16-byte pieces per key row
   static constexpr int RPW = 16 / CPR > 0 ? 16 / CPR : 1;   // key rows per window (D <= 128)
-  static constexpr int K_BYTES = PF_TILE * D * 2;
-  static constexpr int V_BYTES = D * PF_TILE * 2;
+  static constexpr int VPR = TILE / 8;       // pieces per value row
+  static constexpr int VRW = 16 / VPR;       // value rows per window
+  static constexpr int K_BYTES = TILE * D * 2;
+  static constexpr int V_BYTES = D * TILE * 2;
   static constexpr int STAGE = K_BYTES + V_BYTES;
   static constexpr int K_PIECES = K_BYTES / 16, V_PIECES = V_BYTES / 16;
 };
 
-// The softmax update of one block of 16 rows for one 64-key tile: as softmax_step, over
-// four 16-key blocks; the probabilities come back as the two P operands of the tile's halves.
-template <int NB>
-__device__ __forceinline__ void softmax_step64(const f32x4_t (&s)[4], bool full, int key0, int grp, int row_pos,
-                                               int window, float scale_log2, float& m_run, float& l_run,
-                                               f32x4_t (&acc)[NB], Pack16 (&p)[2]) {
-  float v[16];
+// The softmax update of one block of 16 rows for one tile of KB4 16-key blocks: as
+// softmax_step; the probabilities come back as the P operands of the tile's 32-key halves.
+template <int NB, int KB4>
+__device__ __forceinline__ void softmax_tile(const f32x4_t (&s)[KB4], bool full, int key0, int grp, int row_pos,
+                                             int window, float scale_log2, float& m_run, float& l_run,
+                                             f32x4_t (&acc)[NB], Pack16 (&p)[KB4 / 2]) {
+  constexpr int N = 4 * KB4;
+  float v[N];
 #pragma unroll
-  for (int j = 0; j < 16; ++j) v[j] = s[j >> 2][j & 3];
+  for (int j = 0; j < N; ++j) v[j] = s[j >> 2][j & 3];
   if (!full) {
 #pragma unroll
-    for (int j = 0; j < 16; ++j) {
+    for (int j = 0; j < N; ++j) {
       const int key = key0 + 16 * (j >> 2) + 4 * grp + (j & 3);
       bool seen = key <= row_pos;
       if (window > 0 && row_pos - key >= window) seen = false;
@@ -822,21 +829,21 @@ __device__ __forceinline__ void softmax_step64(const f32x4_t (&s)[4], bool full,
   }
   float mx = v[0];
 #pragma unroll
-  for (int j = 1; j < 16; ++j) mx = fmaxf(mx, v[j]);
+  for (int j = 1; j < N; ++j) mx = fmaxf(mx, v[j]);
   mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
   mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
   const float m_new = fmaxf(m_run, mx * scale_log2);
   float sum = 0.f;
   if (m_new > -INFINITY) {
 #pragma unroll
-    for (int j = 0; j < 16; ++j) {
+    for (int j = 0; j < N; ++j) {
       const float e = fast_exp2(fmaf(v[j], scale_log2, -m_new));
       sum += e;
       p[j >> 3].e[j & 7] = (__bf16)e;
     }
   } else {
-    p[0].u = make_uint4(0, 0, 0, 0);
-    p[1].u = make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int h = 0; h < KB4 / 2; ++h) p[h].u = make_uint4(0, 0, 0, 0);
   }
   const bool moved = m_new != m_run;
   if (__builtin_amdgcn_ballot_w64(moved) != 0) {
@@ -849,14 +856,15 @@ __device__ __forceinline__ void softmax_step64(const f32x4_t (&s)[4], bool full,
   l_run += sum;
 }
 
-template <int D>
+template <int D, int TILE, int STAGES>
 __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, int num_pages, const int* __restrict__ block_table, int bt_stride,
     const int* __restrict__ cu_q, const int* __restrict__ kv_lens, int Hq, int Hkv, int page, float scale_log2,
     int window, int tokens_per_block) {
-  typedef PrefillSmem<D> SM;
-  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * SM::STAGE];
+  typedef PrefillSmem<D, TILE> SM;
+  constexpr int KB4 = TILE / 16;  // 16-key blocks per tile
+  __shared__ __attribute__((aligned(16))) unsigned char smem[STAGES * SM::STAGE];
   __shared__ int sh_pages[PREFILL_PAGES];  // the block-table entries of the tiles in hand
   const int b = blockIdx.z, g_kv = blockIdx.y;
   const int G = Hq / Hkv;
@@ -913,11 +921,11 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
   const int blk_first_tok = tile * tokens_per_block;
   const int blk_last_tok = min(q_len, blk_first_tok + tokens_per_block) - 1;
   int tile_lo = 0;
-  if (window > 0) tile_lo = max(0, first_pos + blk_first_tok - window + 1) / PF_TILE;
-  const int tile_hi = (first_pos + blk_last_tok) / PF_TILE + 1;
+  if (window > 0) tile_lo = max(0, first_pos + blk_first_tok - window + 1) / TILE;
+  const int tile_hi = (first_pos + blk_last_tok) / TILE + 1;
   // and this wavefront's own (a wavefront whose rows do not exist has none)
-  int my_lo = tile_lo, my_hi = pos_max >= 0 ? pos_max / PF_TILE + 1 : 0;
-  if (window > 0 && pos_max >= 0) my_lo = max(0, pos_min - window + 1) / PF_TILE;
+  int my_lo = tile_lo, my_hi = pos_max >= 0 ? pos_max / TILE + 1 : 0;
+  if (window > 0 && pos_max >= 0) my_lo = max(0, pos_min - window + 1) / TILE;
   const int* bt_row = block_table + (size_t)b * bt_stride;
 
   // The copy of a tile from the caches into a stage. Place s (a 16-byte piece) of the keys'
@@ -942,17 +950,17 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
 #pragma unroll
   for (int j = 0; j < V_TURNS; ++j) {
     const int place = tid + 256 * j, w = place >> 4, u = place & 15;
-    const int q = (u & 7) ^ (w & 7);
-    v_d[j] = 2 * w + (u >> 3);
+    const int q = (u % SM::VPR) ^ (w % SM::VPR);
+    v_d[j] = SM::VRW * w + u / SM::VPR;
     v_kb[j] = q >> 1;
     v_h[j] = q & 1;
   }
   const size_t page_elems = (size_t)page * D;  // elements of one (page, head) in either cache
   typedef __attribute__((address_space(3))) void* lds_ptr;
 
-  auto plain_tile = [&](int t) { return t * PF_TILE + PF_TILE <= kv_len && window == 0; };
+  auto plain_tile = [&](int t) { return t * TILE + TILE <= kv_len && window == 0; };
   auto copy_direct = [&](int t, int stage) {
-    const int key0 = t * PF_TILE;
+    const int key0 = t * TILE;
     unsigned char* ks = smem + stage * SM::STAGE + 1024 * wave;  // this wavefront's kilobyte of each turn
     unsigned char* vs = ks + SM::K_BYTES;
 #pragma unroll
@@ -974,7 +982,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
     }
   };
   auto copy_checked = [&](int t, int stage) {
-    const int key0 = t * PF_TILE;
+    const int key0 = t * TILE;
     unsigned char* ks = smem + stage * SM::STAGE;
     unsigned char* vs = ks + SM::K_BYTES;
 #pragma unroll
@@ -1019,35 +1027,49 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
   // and for the value rows 16 nb + col
   const int k_lane = (col / SM::RPW) * 256 + (col % SM::RPW) * SM::CPR * 16;
   const int k_swz = (col / SM::RPW) % SM::CPR;
-  const int v_lane = (col >> 1) * 256 + (col & 1) * 128 + 8 * (grp & 1);
-  const int v_swz = (col >> 1) & 7;
+  const int v_lane = (col / SM::VRW) * 256 + (col % SM::VRW) * SM::VPR * 16 + 8 * (grp & 1);
+  const int v_swz = (col / SM::VRW) % SM::VPR;
+  constexpr int LOADS_PER_TILE = K_TURNS + V_TURNS;  // this thread's loads in flight per tile on its way
 
   // tiles are worked through in spans whose table entries fit sh_pages
-  const int tiles_per_span = max(1, (PREFILL_PAGES - 4) * (page / 16) / 4);
+  const int tiles_per_span = max(1, (PREFILL_PAGES - 4) * page / TILE);
   for (int span_lo = tile_lo; span_lo < tile_hi; span_lo += tiles_per_span) {
     const int span_hi = min(tile_hi, span_lo + tiles_per_span);
     __syncthreads();
-    page_base = (span_lo * PF_TILE) >> page_shift;
+    page_base = (span_lo * TILE) >> page_shift;
     {
-      const int last_page = min((kv_len - 1) >> page_shift, (span_hi * PF_TILE - 1) >> page_shift);
+      const int last_page = min((kv_len - 1) >> page_shift, (span_hi * TILE - 1) >> page_shift);
       for (int i = tid; page_base + i <= last_page; i += 256) sh_pages[i] = bt_row[page_base + i];
     }
     __syncthreads();
-    copy_tile(span_lo, 0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // STAGES - 1 tiles are on their way at any time: the first ones here, then tile
+    // t + STAGES - 1 at the top of tile t's turn, into the stage tile t - 1 has left. Loads
+    // complete in the order they were issued, so waiting until no more than the later tiles'
+    // loads are outstanding means the next tile has landed.
+    auto wait_for_tile = [&](int tiles_after) {
+      if (tiles_after <= 0)
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      else if (tiles_after == 1)
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LOADS_PER_TILE) : "memory");
+      else
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * LOADS_PER_TILE) : "memory");
+    };
+    static_assert(STAGES >= 2 && STAGES <= 4 && 2 * LOADS_PER_TILE < 64, "the wait counts above");
+#pragma unroll
+    for (int ahead = 0; ahead < STAGES - 1; ++ahead)
+      if (span_lo + ahead < span_hi) copy_tile(span_lo + ahead, ahead);
+    wait_for_tile(min(span_hi - span_lo, STAGES - 1) - 1);
     __syncthreads();
     for (int t = span_lo; t < span_hi; ++t) {
-      const int stage = (t - span_lo) & 1;
-      const bool more = t + 1 < span_hi;
-      // the next tile into the other stage, which every wavefront left at the last barrier
-      if (more) copy_tile(t + 1, stage ^ 1);
+      const int stage = (t - span_lo) % STAGES;
+      if (t + STAGES - 1 < span_hi) copy_tile(t + STAGES - 1, (t + STAGES - 1 - span_lo) % STAGES);
       if (t >= my_lo && t < my_hi) {
         const unsigned char* ks = smem + stage * SM::STAGE;
         const unsigned char* vs = ks + SM::K_BYTES;
-        const int key0 = t * PF_TILE;
-        f32x4_t sc[2][4];
+        const int key0 = t * TILE;
+        f32x4_t sc[2][KB4];
 #pragma unroll
-        for (int kb4 = 0; kb4 < 4; ++kb4) {
+        for (int kb4 = 0; kb4 < KB4; ++kb4) {
           Pack16 a[D / 32];
 #pragma unroll
           for (int i = 0; i < D / 32; ++i)
@@ -1063,27 +1085,28 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
           }
         }
         // no key of the tile is hidden from any row of this wavefront?
-        const bool full = key0 + PF_TILE - 1 <= pos_min && (window == 0 || pos_max - key0 < window);
-        Pack16 p[2][2];
+        const bool full = key0 + TILE - 1 <= pos_min && (window == 0 || pos_max - key0 < window);
+        Pack16 p[2][KB4 / 2];
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb)
-          softmax_step64<D / 16>(sc[qb], full, key0, grp, row_pos[qb], window, scale_log2, m_run[qb], l_run[qb],
-                                 acc[qb], p[qb]);
+          softmax_tile<D / 16, KB4>(sc[qb], full, key0, grp, row_pos[qb], window, scale_log2, m_run[qb], l_run[qb],
+                                    acc[qb], p[qb]);
 #pragma unroll
         for (int nb = 0; nb < D / 16; ++nb)
 #pragma unroll
-          for (int half = 0; half < 2; ++half) {
+          for (int half = 0; half < KB4 / 2; ++half) {
             Pack16 vt;  // keys 4 grp .. 4 grp + 3 of the half's two 16-key blocks
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
-              vt.h[kb] = *reinterpret_cast<const uint2*>(vs + 2048 * nb + v_lane +
+              vt.h[kb] = *reinterpret_cast<const uint2*>(vs + (16 / SM::VRW) * 256 * nb + v_lane +
                                                         16 * ((2 * (2 * half + kb) + (grp >> 1)) ^ v_swz));
 #pragma unroll
             for (int qb = 0; qb < 2; ++qb)
               acc[qb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt.v, p[qb][half].v, acc[qb][nb], 0, 0, 0);
           }
       }
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's share of the next tile has landed
+      // this wavefront's share of the next tile has landed; the tiles after it may still travel
+      wait_for_tile(min(t + STAGES - 1, span_hi - 1) - (t + 1));
       __syncthreads();
     }
   }
@@ -1127,7 +1150,8 @@ static int launch_fast(const void* q, int q_stride, void* out, const void* k_cac
   if (max_q_len * G > 16) {
     const int tokens_per_block = 128 / G;
     const int tiles = (max_q_len + tokens_per_block - 1) / tokens_per_block;
-    hipLaunchKernelGGL(attn_prefill_kernel<D>, dim3(tiles, Hkv, B), dim3(256), 0, stream, (const bf16_t*)q, q_stride,
+    hipLaunchKernelGGL((attn_prefill_kernel<D, PF_TILE, PF_STAGES>), dim3(tiles, Hkv, B), dim3(256), 0, stream,
+                       (const bf16_t*)q, q_stride,
                        (bf16_t*)out, (const bf16_t*)k_cache, (const bf16_t*)v_cache, num_pages, block_table,
                        bt_stride, cu_q, kv_lens, Hq, Hkv, page, scale_log2, window, tokens_per_block);
   }

@@ -959,25 +959,38 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
   typedef __attribute__((address_space(3))) void* lds_ptr;
 
   auto plain_tile = [&](int t) { return t * TILE + TILE <= kv_len && window == 0; };
+  // the pages of a tile's 16-key blocks, looked up once per tile (every lane reads the same few
+  // table entries, all in one go) rather than once per load
+  constexpr int KB4_ = TILE / 16;
+  auto tile_pages = [&](int t, int (&pg)[KB4_]) {
+#pragma unroll
+    for (int kb = 0; kb < KB4_; ++kb) pg[kb] = sh_pages[((t * TILE + 16 * kb) >> page_shift) - page_base];
+#pragma unroll
+    for (int kb = 0; kb < KB4_; ++kb) pg[kb] = min(max(pg[kb], 0), num_pages - 1);
+  };
   auto copy_direct = [&](int t, int stage) {
     const int key0 = t * TILE;
     unsigned char* ks = smem + stage * SM::STAGE + 1024 * wave;  // this wavefront's kilobyte of each turn
     unsigned char* vs = ks + SM::K_BYTES;
+    int pg[KB4_];
+    tile_pages(t, pg);
 #pragma unroll
     for (int j = 0; j < K_TURNS; ++j) {
       const int key = key0 + k_row[j];
-      int pg = sh_pages[(key >> page_shift) - page_base];
-      pg = min(max(pg, 0), num_pages - 1);
-      const bf16_t* src = k_cache + (size_t)(pg * Hkv + g_kv) * page_elems + ((key & (page - 1)) * D + k_off[j]);
+      int mine = pg[0];
+#pragma unroll
+      for (int kb = 1; kb < KB4_; ++kb) mine = (k_row[j] >> 4) == kb ? pg[kb] : mine;
+      const bf16_t* src = k_cache + (size_t)(mine * Hkv + g_kv) * page_elems + ((key & (page - 1)) * D + k_off[j]);
       __builtin_amdgcn_global_load_lds(src, (lds_ptr)(ks + 4096 * j), 16, 0, 0);
     }
 #pragma unroll
     for (int j = 0; j < V_TURNS; ++j) {
       const int key = key0 + 16 * v_kb[j];
-      int pg = sh_pages[(key >> page_shift) - page_base];
-      pg = min(max(pg, 0), num_pages - 1);
+      int mine = pg[0];
+#pragma unroll
+      for (int kb = 1; kb < KB4_; ++kb) mine = v_kb[j] == kb ? pg[kb] : mine;
       const bf16_t* src =
-          v_cache + (size_t)(pg * Hkv + g_kv) * page_elems + (v_d[j] * page + (key & (page - 1)) + 8 * v_h[j]);
+          v_cache + (size_t)(mine * Hkv + g_kv) * page_elems + (v_d[j] * page + (key & (page - 1)) + 8 * v_h[j]);
       __builtin_amdgcn_global_load_lds(src, (lds_ptr)(vs + 4096 * j), 16, 0, 0);
     }
   };

@@ -1,13 +1,17 @@
 """Decode and prefill throughput of the Qwen3-8B-shaped model on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L]
+                    [--shape 8b|14b|32b] [--prompt P] [--context C]
 
 Random bfloat16 weights, uniform-random prompts of 2,048 tokens, greedy decoding
 through the engine's own step loop (scheduler, step function, sampling). A
 "step" is one decode step of the whole batch. One JSON line is printed:
 `value` is decoded tokens per second at the default batch; `prefill` is one
 2,048-token prompt in one step; `roofline` prices the decode step against HBM
-bandwidth; `points` holds decoding at batch 1 and 64.
+bandwidth; `points` holds decoding at batch 1 and 64. The default run is the
+8B shape with prompts of 2,048 in a context of 8,192; `--shape`, `--prompt` and
+`--context` move the decode measurement to the larger shapes and to longer
+contexts (the prefill measurement stays at 2,048 tokens).
 """
 
 import argparse
@@ -22,8 +26,10 @@ QWEN3_8B = dict(architectures=["Qwen3ForCausalLM"], vocab_size=151936, hidden_si
                 num_hidden_layers=36, max_position_embeddings=40960, num_attention_heads=32,
                 num_key_value_heads=8, head_dim=128, intermediate_size=12288, rms_norm_eps=1e-6,
                 rope_theta=1000000.0, tie_word_embeddings=False)
-CONTEXT = 8192
-PROMPT = 2048
+QWEN3_14B = dict(QWEN3_8B, hidden_size=5120, num_hidden_layers=40, num_attention_heads=40, intermediate_size=17408)
+QWEN3_32B = dict(QWEN3_8B, hidden_size=5120, num_hidden_layers=64, num_attention_heads=64, intermediate_size=25600)
+SHAPES = {"8b": ("Qwen3-8B", QWEN3_8B), "14b": ("Qwen3-14B", QWEN3_14B), "32b": ("Qwen3-32B", QWEN3_32B)}
+PREFILL = 2048
 BLOCK = 16
 
 
@@ -56,6 +62,9 @@ def main():
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration (0 = all)")
     ap.add_argument("--dtype", default="bfloat16")
+    ap.add_argument("--shape", default="8b", choices=sorted(SHAPES))
+    ap.add_argument("--prompt", type=int, default=2048, help="tokens every request holds when decoding starts")
+    ap.add_argument("--context", type=int, default=8192, help="tokens of cache per request")
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 points")
     ap.add_argument("--skip-prefill", action="store_true",
                     help="skip the prefill measurement (for profiles of decoding alone; the line then has no value for it)")
@@ -69,7 +78,12 @@ def main():
     from qwen3_from_scratch_amd.config import ModelConfig
     from qwen3_from_scratch_amd.engine import SyncEngine, random_model
 
-    raw = dict(QWEN3_8B)
+    shape_name, raw = SHAPES[args.shape]
+    raw = dict(raw)
+    prompt_len, context = args.prompt, args.context
+    if not 0 < prompt_len + args.warmup + args.steps < context <= raw["max_position_embeddings"]:
+        print("bench.py: --prompt, --warmup and --steps must fit in --context, and that in the model's positions")
+        return 2
     full_layers = raw["num_hidden_layers"]
     if args.layers:
         raw["num_hidden_layers"] = args.layers
@@ -79,14 +93,14 @@ def main():
     model = random_model(config, dtype=args.dtype, device="cuda:0", seed=0, std=0.02)
     gen = torch.Generator().manual_seed(1)
 
-    def prompts(n):
-        return [torch.randint(0, config.vocab_size, (PROMPT,), generator=gen).tolist() for _ in range(n)]
+    def prompts(n, length):
+        return [torch.randint(0, config.vocab_size, (length,), generator=gen).tolist() for _ in range(n)]
 
     def engine_for(batch):
-        pages = batch * (CONTEXT // BLOCK)
-        return SyncEngine(model=model, path="", dtype=args.dtype, device="cuda:0", max_len=CONTEXT,
+        pages = batch * (context // BLOCK)
+        return SyncEngine(model=model, path="", dtype=args.dtype, device="cuda:0", max_len=context,
                           block_size=BLOCK, num_blocks=pages, max_num_seqs=batch,
-                          max_num_tokens=max(PROMPT, batch), chunked_prefill_size=PROMPT)
+                          max_num_tokens=max(PREFILL, batch), chunked_prefill_size=PREFILL)
 
     def sync():
         torch.cuda.synchronize()
@@ -95,26 +109,26 @@ def main():
     engine = engine_for(1)
     prefill_s = None
     for _ in range(0 if args.skip_prefill else 2):   # warm-up, then the timed one
-        req = engine.add_request(prompts(1)[0], engine.default_params(1, temperature=0.0, ignore_eos=True))
+        engine.add_request(prompts(1, PREFILL)[0], engine.default_params(1, temperature=0.0, ignore_eos=True))
         sync()
         t0 = time.perf_counter()
         plan = engine.step()
         sync()
         prefill_s = time.perf_counter() - t0
-        assert len(plan) == 1 and plan[0].num_tokens == PROMPT
+        assert len(plan) == 1 and plan[0].num_tokens == PREFILL
         while engine.scheduler.has_work():
             engine.step()
     prefill = None
     if prefill_s is not None:
-        prefill = {"value": round(PROMPT / prefill_s, 1), "tokens": PROMPT, "ms": round(prefill_s * 1e3, 3),
-                   "frac": round(prefill_flops(config, PROMPT) / prefill_s / PEAK_FLOPS[args.dtype], 4)}
+        prefill = {"value": round(PREFILL / prefill_s, 1), "tokens": PREFILL, "ms": round(prefill_s * 1e3, 3),
+                   "frac": round(prefill_flops(config, PREFILL) / prefill_s / PEAK_FLOPS[args.dtype], 4)}
     del engine
 
     # ---- decode ----
     def decode(batch, steps, warmup):
         engine = engine_for(batch)
-        params = engine.default_params(CONTEXT - PROMPT - 1, temperature=0.0, ignore_eos=True)
-        requests = [engine.add_request(p, params) for p in prompts(batch)]
+        params = engine.default_params(context - prompt_len - 1, temperature=0.0, ignore_eos=True)
+        requests = [engine.add_request(p, params) for p in prompts(batch, prompt_len)]
         while any(r.is_prefill for r in requests) or len(engine.scheduler.waiting):
             engine.step()
         for _ in range(warmup):
@@ -144,13 +158,13 @@ def main():
             points["decode_b%d" % b] = round(p_tps, 1)
 
     line = {
-        "metric": "decode tok/s at batch 1/8/64 + prefill tok/s at 2048 tokens, Qwen3-8B bf16",
+        "metric": "decode tok/s at batch 1/8/64 + prefill tok/s at 2048 tokens, %s bf16" % shape_name,
         "value": round(tps, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
         "config": {
-            "model": "Qwen3-8B-shaped, random weights N(0, 0.02)", "global_batch": args.batch,
-            "seq_len": PROMPT, "parallelism": "single-gpu", "context_len": CONTEXT,
+            "model": "%s-shaped, random weights N(0, 0.02)" % shape_name, "global_batch": args.batch,
+            "seq_len": prompt_len, "parallelism": "single-gpu", "context_len": context,
             "layers": config.num_hidden_layers, "layers_full": full_layers, "hidden_size": config.hidden_size,
             "num_attention_heads": config.num_attention_heads, "num_key_value_heads": config.num_key_value_heads,
             "head_dim": config.head_dim, "intermediate_size": config.intermediate_size,

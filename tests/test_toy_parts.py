@@ -1,8 +1,8 @@
 """Parts defined here, outside the framework, are registered, built into a model
 with the framework's own parts, and stepped: a mixer with a state of fixed size
-per request, a position encoding added to the embeddings, an attention layer
-with a window, a layer that runs twice, and a layer that reads another layer's
-cache. Nothing under qwen3_from_scratch_amd changes for them. They never
+per request, a feed-forward whose router gives most experts no weight, a
+position encoding added to the embeddings, an attention layer with a window, a
+layer that runs twice, and a layer that reads another layer's cache. Nothing under qwen3_from_scratch_amd changes for them. They never
 become a model of anyone's: they exist to show what the interfaces carry.
 
 The same test runs on the CPU (plain twins in place of the kernels) and, marked
@@ -23,6 +23,7 @@ from qwen3_from_scratch_amd.parts import CacheNeed, Part, PartSpec, Precision
 from qwen3_from_scratch_amd.weights import RandomWeights
 
 V, HQ, HKV, I = 97, 4, 2, 80
+EXPERTS, EXPERT_I = 4, 24
 EPS, THETA, WINDOW, MAXPOS = 1e-5, 10000.0, 19, 512
 H, D = 48, 16                 # the default sizes; `sizes()` swaps in others for one test
 
@@ -88,14 +89,59 @@ class LearnedPosition(Part):
         return None
 
 
+def routing_weights(probabilities):
+    """An expert counts by how far its probability lies above the uniform one,
+    and not at all below it; the weights sum to one. Unlike a top-k choice this
+    is continuous in the router's logits, so that rounding moves the result a
+    little and never to another expert's."""
+    above = torch.relu(probabilities - 1.0 / probabilities.shape[-1])
+    return above / above.sum(dim=-1, keepdim=True).clamp_min(1e-6)
+
+
+@register_part("feed_forward", "toy_routed")
+class RoutedFeedForward(Part):
+    """sum_e g_e(x) . down_e(relu(up_e(x))), the router in float32. All experts
+    are computed for all rows and weighted (g_e is zero for most), which keeps
+    the part free of host decisions and so fit for graph replays."""
+
+    graph_safe = True
+
+    def __init__(self, prefix, precision, device, hidden_size, intermediate_size, num_experts):
+        super().__init__(prefix, precision, device)
+        self.hidden_size, self.intermediate_size, self.num_experts = hidden_size, intermediate_size, num_experts
+        self.router = self.up = self.down = None
+
+    def tensors(self):
+        names = {self._name("router.weight"): (self.num_experts, self.hidden_size)}
+        for e in range(self.num_experts):
+            names[self._name("experts.%d.up.weight" % e)] = (self.intermediate_size, self.hidden_size)
+            names[self._name("experts.%d.down.weight" % e)] = (self.hidden_size, self.intermediate_size)
+        return names
+
+    def load(self, fetch):
+        act = self.precision.act
+        self.router = fetch(self._name("router.weight"), torch.float32)
+        self.up = [fetch(self._name("experts.%d.up.weight" % e), act) for e in range(self.num_experts)]
+        self.down = [fetch(self._name("experts.%d.down.weight" % e), act) for e in range(self.num_experts)]
+
+    def forward(self, x, batch=None):
+        g = routing_weights(torch.softmax(x.float() @ self.router.T, dim=-1))
+        out = torch.zeros(x.shape, dtype=torch.float32, device=x.device)
+        for e in range(self.num_experts):
+            out += g[:, e:e + 1] * (torch.relu(x @ self.up[e].T) @ self.down[e].T).float()
+        return out.to(x.dtype)
+
+
 def toy_spec(position, with_state=True):
     norm = PartSpec.of("norm", "rms", size=H, eps=EPS)
     attn = dict(hidden_size=H, num_heads=HQ, num_kv_heads=HKV, head_dim=D, qk_norm=True, qk_norm_eps=EPS)
     ff = PartSpec.of("feed_forward", "swiglu", hidden_size=H, intermediate_size=I)
 
+    routed = PartSpec.of("feed_forward", "toy_routed", hidden_size=H, intermediate_size=EXPERT_I, num_experts=EXPERTS)
+
     def layer(i, mixer):
-        return LayerSpec(prefix="toy.layers.%d" % i, mixer=mixer, feed_forward=ff, mixer_norm=norm,
-                         feed_forward_norm=norm)
+        return LayerSpec(prefix="toy.layers.%d" % i, mixer=mixer, feed_forward=routed if i == 2 else ff,
+                         mixer_norm=norm, feed_forward_norm=norm)
 
     layers = (
         layer(0, PartSpec.of("mixer", "attention", window=0, **attn)),
@@ -152,7 +198,13 @@ def plain_toy_logits(w, spec, position, tokens):
             d = o.reshape(T, HQ * D) @ w[a + ".o_proj.weight"].T
         x = x + d
         h = plain.rms_norm(x, w[p + ".post_attention_layernorm.weight"], EPS)
-        x = x + plain.swiglu_mlp(h, w, p + ".mlp")
+        if spec.layers[i].feed_forward.name == "toy_routed":
+            g = routing_weights(torch.softmax(h @ w[p + ".mlp.router.weight"].T, dim=-1))
+            for e in range(EXPERTS):
+                up, down = w[p + ".mlp.experts.%d.up.weight" % e], w[p + ".mlp.experts.%d.down.weight" % e]
+                x = x + g[:, e:e + 1] * (torch.relu(h @ up.T) @ down.T)
+        else:
+            x = x + plain.swiglu_mlp(h, w, p + ".mlp")
     return plain.rms_norm(x, w["toy.norm.weight"], EPS) @ w["toy.head.weight"].T
 
 

@@ -1,0 +1,238 @@
+// Matrix products with many rows, out[M, N] = x[M, K] . w[N, K]^T in bfloat16
+// with float32 accumulation, through the vendor library (hipBLASLt), as the
+// reference's engine uses its vendor library for them
+// (src/qwen3_from_scratch/models/linear.py:24-31 calls F.linear).
+//
+// The library's heuristic returns a ranked list of kernels for a problem; its
+// first choice is often not its fastest (for 576 x 5120 x 17408 the first took
+// 108 us and the fourth 92; for 2048 x 4096 x 4096, 101 against 55). The first
+// time a problem size is seen outside a graph capture, the leading candidates
+// are timed on the caller's own operands and the fastest is kept for the life
+// of the process. A size first seen during a capture runs the first candidate
+// and is tuned at its next eager call. In the model every weight is read once
+// a step, with gigabytes of other traffic in between, so a candidate is timed
+// with cold caches: a kernel that reads a buffer larger than the last-level
+// cache runs before each timed run. Timed warm, products of few rows pick
+// kernels that are the fastest only while the weight sits in that cache.
+//
+// One workspace and one such buffer per device, allocated at first need and kept. Calls on one
+// device share it and the plans: they are serialised by a lock and are meant
+// to come from one stream at a time.
+
+#include "common.h"
+
+#include <hipblaslt/hipblaslt.h>
+
+#include <map>
+#include <mutex>
+#include <tuple>
+#include <vector>
+
+#define Q3_ERR_LIBRARY 20000   // + the library's status
+
+namespace {
+
+constexpr size_t WORKSPACE_BYTES = 128u << 20;
+constexpr size_t EVICT_BYTES = 512u << 20;     // twice the 256 MB last-level cache
+constexpr int EVICT_BLOCKS = 2048, EVICT_THREADS = 256;
+constexpr int MAX_CANDIDATES = 64;
+
+// Reads the whole buffer; the store never happens (the buffer holds zeros) but keeps the loads alive.
+__global__ void evict_kernel(float4* buffer, size_t count) {
+  float sum = 0.f;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x) {
+    const float4 v = buffer[i];
+    sum += v.x + v.y + v.z + v.w;
+  }
+  if (sum == 12345.f) buffer[0].x = sum;
+}
+
+struct Plan {
+  hipblasLtMatmulDesc_t desc = nullptr;
+  hipblasLtMatrixLayout_t w = nullptr, x = nullptr, out = nullptr;
+  hipblasLtMatmulAlgo_t algo;
+  bool tuned = false;
+  int candidates = 0, chosen = 0;
+  float first_us = 0.f, best_us = 0.f;
+};
+
+struct Device {
+  hipblasLtHandle_t handle = nullptr;
+  void* workspace = nullptr;
+  void* evict = nullptr;
+  hipEvent_t begin = nullptr, end = nullptr;
+  std::map<std::tuple<int, int, int, int>, Plan> plans;
+};
+
+std::mutex g_lock;
+std::map<int, Device> g_devices;
+int g_candidates = 16;
+
+#define HIP_TRY(call)                    \
+  do {                                   \
+    hipError_t e_ = (call);              \
+    if (e_ != hipSuccess) return (int)e_; \
+  } while (0)
+#define LT_TRY(call)                                              \
+  do {                                                            \
+    hipblasStatus_t s_ = (call);                                  \
+    if (s_ != HIPBLAS_STATUS_SUCCESS) return Q3_ERR_LIBRARY + (int)s_; \
+  } while (0)
+
+int describe(Plan& p, int M, int N, int K, int out_dtype) {
+  // Row-major x (M, K), w (N, K), out (M, N) are column-major (K, M), (K, N), (N, M):
+  // out_cm = w_cm^T . x_cm.
+  const hipDataType out_type = out_dtype == Q3_F32 ? HIP_R_32F : HIP_R_16BF;
+  LT_TRY(hipblasLtMatmulDescCreate(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F));
+  hipblasOperation_t transposed = HIPBLAS_OP_T, plain = HIPBLAS_OP_N;
+  LT_TRY(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &transposed, sizeof(transposed)));
+  LT_TRY(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &plain, sizeof(plain)));
+  LT_TRY(hipblasLtMatrixLayoutCreate(&p.w, HIP_R_16BF, K, N, K));
+  LT_TRY(hipblasLtMatrixLayoutCreate(&p.x, HIP_R_16BF, K, M, K));
+  LT_TRY(hipblasLtMatrixLayoutCreate(&p.out, out_type, N, M, N));
+  return 0;
+}
+
+void forget(Plan& p) {
+  if (p.w) (void)hipblasLtMatrixLayoutDestroy(p.w);
+  if (p.x) (void)hipblasLtMatrixLayoutDestroy(p.x);
+  if (p.out) (void)hipblasLtMatrixLayoutDestroy(p.out);
+  if (p.desc) (void)hipblasLtMatmulDescDestroy(p.desc);
+  p = Plan();
+}
+
+hipblasStatus_t run(Device& d, const Plan& p, const hipblasLtMatmulAlgo_t& algo, const void* x, const void* w,
+                    void* out, hipStream_t stream) {
+  const float one = 1.f, zero = 0.f;
+  return hipblasLtMatmul(d.handle, p.desc, &one, w, p.w, x, p.x, &zero, out, p.out, out, p.out, &algo, d.workspace,
+                         WORKSPACE_BYTES, stream);
+}
+
+// The shortest of `reps` runs, each with cold caches, in microseconds; negative if the candidate fails.
+float time_candidate(Device& d, const Plan& p, const hipblasLtMatmulAlgo_t& algo, const void* x, const void* w,
+                     void* out, hipStream_t stream, int reps) {
+  float best = -1.f;
+  for (int r = 0; r < reps; ++r) {
+    evict_kernel<<<EVICT_BLOCKS, EVICT_THREADS, 0, stream>>>((float4*)d.evict, EVICT_BYTES / sizeof(float4));
+    if (hipEventRecord(d.begin, stream) != hipSuccess) return -1.f;
+    if (run(d, p, algo, x, w, out, stream) != HIPBLAS_STATUS_SUCCESS) return -1.f;
+    if (hipEventRecord(d.end, stream) != hipSuccess || hipEventSynchronize(d.end) != hipSuccess) return -1.f;
+    float ms = 0.f;
+    if (hipEventElapsedTime(&ms, d.begin, d.end) != hipSuccess) return -1.f;
+    if (best < 0.f || ms * 1000.f < best) best = ms * 1000.f;
+  }
+  return best;
+}
+
+int choose(Device& d, Plan& p, int M, int N, int K, const void* x, const void* w, void* out, hipStream_t stream,
+           bool capturing) {
+  hipblasLtMatmulPreference_t pref = nullptr;
+  LT_TRY(hipblasLtMatmulPreferenceCreate(&pref));
+  size_t bytes = WORKSPACE_BYTES;
+  hipblasStatus_t s = hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &bytes,
+                                                            sizeof(bytes));
+  const int want = capturing ? 1 : g_candidates;
+  std::vector<hipblasLtMatmulHeuristicResult_t> found(want);
+  int got = 0;
+  if (s == HIPBLAS_STATUS_SUCCESS)
+    s = hipblasLtMatmulAlgoGetHeuristic(d.handle, p.desc, p.w, p.x, p.out, p.out, pref, want, found.data(), &got);
+  (void)hipblasLtMatmulPreferenceDestroy(pref);
+  if (s != HIPBLAS_STATUS_SUCCESS) return Q3_ERR_LIBRARY + (int)s;
+  if (got == 0) return Q3_ERR_UNSUPPORTED;
+  p.candidates = got;
+  p.chosen = 0;
+  p.algo = found[0].algo;
+  p.tuned = !capturing;
+  if (capturing || got == 1) return 0;
+  if (!d.evict) {
+    HIP_TRY(hipMalloc(&d.evict, EVICT_BYTES));
+    HIP_TRY(hipMemsetAsync(d.evict, 0, EVICT_BYTES, stream));
+  }
+  // two passes: all candidates briefly (the first run of each also loads its code), then those
+  // near the front again and longer
+  std::vector<float> us(got, -1.f);
+  float best = -1.f;
+  for (int i = 0; i < got; ++i) {
+    if (run(d, p, found[i].algo, x, w, out, stream) != HIPBLAS_STATUS_SUCCESS) continue;
+    us[i] = time_candidate(d, p, found[i].algo, x, w, out, stream, 2);
+    if (us[i] > 0.f && (best < 0.f || us[i] < best)) best = us[i];
+  }
+  if (best < 0.f) return Q3_ERR_UNSUPPORTED;
+  for (int i = 0; i < got; ++i) {
+    if (us[i] < 0.f || us[i] > 1.2f * best) continue;
+    const float again = time_candidate(d, p, found[i].algo, x, w, out, stream, 5);
+    if (again > 0.f && again < us[i]) us[i] = again;
+  }
+  int chosen = -1;
+  for (int i = 0; i < got; ++i)
+    if (us[i] > 0.f && (chosen < 0 || us[i] < us[chosen])) chosen = i;
+  p.chosen = chosen;
+  p.algo = found[chosen].algo;
+  p.first_us = us[0];
+  p.best_us = us[chosen];
+  return 0;
+}
+
+}  // namespace
+
+// How many of the library's candidates are timed for a new problem size (1: take its first choice).
+extern "C" int q3_matmul_set_candidates(int n) {
+  if (n < 1 || n > MAX_CANDIDATES) return Q3_ERR_BAD_ARGUMENT;
+  std::lock_guard<std::mutex> hold(g_lock);
+  g_candidates = n;
+  return 0;
+}
+
+// What was chosen for a size on the current device: info[0] candidates timed, info[1] index chosen,
+// info[2] microseconds of the first candidate, info[3] of the chosen one. Returns 1 if the size is known.
+extern "C" int q3_matmul_plan(int M, int N, int K, int out_dtype, float* info) {
+  std::lock_guard<std::mutex> hold(g_lock);
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) return 0;
+  auto d = g_devices.find(device);
+  if (d == g_devices.end()) return 0;
+  auto p = d->second.plans.find(std::make_tuple(M, N, K, out_dtype));
+  if (p == d->second.plans.end()) return 0;
+  info[0] = (float)p->second.candidates;
+  info[1] = (float)p->second.chosen;
+  info[2] = p->second.first_us;
+  info[3] = p->second.best_us;
+  return 1;
+}
+
+extern "C" int q3_matmul(const void* x, const void* w, void* out, int M, int N, int K, int out_dtype, void* stream_) {
+  if (M <= 0 || N <= 0 || K <= 0 || !x || !w || !out) return Q3_ERR_BAD_ARGUMENT;
+  if (out_dtype != Q3_F32 && out_dtype != Q3_BF16) return Q3_ERR_BAD_ARGUMENT;
+  hipStream_t stream = (hipStream_t)stream_;
+  std::lock_guard<std::mutex> hold(g_lock);
+  int device = 0;
+  HIP_TRY(hipGetDevice(&device));
+  Device& d = g_devices[device];
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  HIP_TRY(hipStreamIsCapturing(stream, &capture));
+  const bool capturing = capture != hipStreamCaptureStatusNone;
+  if (!d.handle) {
+    if (capturing) return (int)hipErrorStreamCaptureUnsupported;   // the first call on a device allocates
+    HIP_TRY(hipMalloc(&d.workspace, WORKSPACE_BYTES));
+    HIP_TRY(hipEventCreate(&d.begin));
+    HIP_TRY(hipEventCreate(&d.end));
+    LT_TRY(hipblasLtCreate(&d.handle));
+  }
+  Plan& p = d.plans[std::make_tuple(M, N, K, out_dtype)];
+  if (!p.desc) {
+    const int status = describe(p, M, N, K, out_dtype);
+    if (status) {
+      forget(p);
+      return status;
+    }
+  }
+  if (!p.candidates || (!p.tuned && !capturing)) {
+    const int status = choose(d, p, M, N, K, x, w, out, stream, capturing);
+    if (status) {
+      forget(p);
+      return status;
+    }
+  }
+  LT_TRY(run(d, p, p.algo, x, w, out, stream));
+  return 0;
+}

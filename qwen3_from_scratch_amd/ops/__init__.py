@@ -31,11 +31,14 @@ __all__ = [
     "linear",
     "linear_swiglu",
     "linear_residual_norm",
+    "matmul_candidates",
+    "matmul_plan",
     "tile_weight",
     "sample",
 ]
 
 _DT = {torch.float32: 0, torch.bfloat16: 1}
+_UNSUPPORTED = 10002          # a launcher's refusal of a size it has no kernel for
 
 
 class OperandError(ValueError):
@@ -64,8 +67,25 @@ def _dev(*tensors):
 
 
 def _check(status, what):
+    if status >= 20000:
+        raise RuntimeError("%s failed: hipBLASLt status %d" % (what, status - 20000))
     if status != 0:
         raise RuntimeError("%s failed: HIP error %d" % (what, status))
+
+
+def matmul_candidates(n):
+    """How many of the vendor library's candidate kernels are timed when a product with many rows
+    meets a new size (1: its first choice is taken untimed)."""
+    _check(library("matmul").q3_matmul_set_candidates(int(n)), "matmul_candidates")
+
+
+def matmul_plan(M, N, K, out_dtype=torch.bfloat16):
+    """What was chosen for a size on the current device, or None if it has not been met:
+    (candidates timed, index chosen, microseconds of the first candidate, of the chosen one)."""
+    info = (ctypes.c_float * 4)()
+    if not library("matmul").q3_matmul_plan(int(M), int(N), int(K), _DT[out_dtype], info):
+        return None
+    return int(info[0]), int(info[1]), float(info[2]), float(info[3])
 
 
 def embed_rows(ids, table, out=None):
@@ -393,13 +413,21 @@ def linear(x, weight, out_dtype=None, out=None, tiled=None, unscaled=None):
         return out
     _need(unscaled is None, "unscaled rows need the few-row kernel: bfloat16, at most 16 rows, a tiled weight")
     if M and x.dtype == torch.bfloat16 and not library("gemm").q3_linear_is_skinny(M, N, K, 1):
-        # bfloat16 products with many rows go to the vendor library (hipBLASLt through
-        # torch), as the reference's engine uses its vendor library for them; accumulation
-        # is float32. Few rows take the weight-streaming kernel below.
-        if out_dtype == torch.bfloat16:
-            torch.mm(x, weight.t(), out=out)
+        # bfloat16 products with many rows go to the vendor library (hipBLASLt), as the
+        # reference's engine uses its vendor library for them; accumulation is float32.
+        # The module picks the library's kernel for each size by timing its candidates
+        # once. Few rows take the weight-streaming kernel below.
+        _need(x.is_contiguous() and weight.is_contiguous() and out.is_contiguous(), "operands must be contiguous")
+        status = library("matmul").q3_matmul(_ptr(x), _ptr(weight), _ptr(out), M, N, K, _DT[out_dtype], _stream())
+        if status == _UNSUPPORTED:
+            # a size hipBLASLt offers no kernel for (an odd inner size, say): the vendor's other
+            # library, through torch
+            if out_dtype == torch.bfloat16:
+                torch.mm(x, weight.t(), out=out)
+            else:
+                torch.mm(x, weight.t(), out_dtype=torch.float32, out=out)
         else:
-            torch.mm(x, weight.t(), out_dtype=torch.float32, out=out)
+            _check(status, "matmul")
     elif M:
         _check(library("gemm").q3_linear(
             _ptr(x), _ptr(weight), _ptr(out), M, N, K, _DT[x.dtype], _DT[out_dtype], _stream()), "linear")

@@ -29,7 +29,9 @@ FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
 ]
-MODULES = ("elementwise", "norm", "rotary", "attention", "gemm", "sampling")
+MODULES = ("elementwise", "norm", "rotary", "attention", "gemm", "matmul", "sampling")
+# what a module links besides the HIP runtime
+LINKS = {"matmul": ["-lhipblaslt"]}
 
 _loaded = {}
 _lock = threading.Lock()
@@ -52,7 +54,7 @@ def _hipcc():
 
 def _digest(module):
     h = hashlib.sha256()
-    h.update(" ".join(FLAGS).encode())
+    h.update(" ".join(FLAGS + LINKS.get(module, [])).encode())
     for name in sorted(os.listdir(CSRC)):
         if name.endswith(".h") or name == module + ".hip":
             with open(os.path.join(CSRC, name), "rb") as fh:
@@ -100,6 +102,9 @@ def compile_module(module, force=False):
         so = os.path.join(lib_dir, module + ".so")
         tmp = so + ".tmp%d" % os.getpid()
         cmd = [hipcc] + FLAGS + ["-I", CSRC, source, "-o", tmp]
+        if module in LINKS:
+            rocm_lib = os.path.join(os.path.dirname(os.path.dirname(os.path.realpath(hipcc))), "lib")
+            cmd += ["-L" + rocm_lib] + LINKS[module]
         _say("compiling %s.hip for %s ..." % (module, ARCH))
         started = time.time()
         env = dict(os.environ)

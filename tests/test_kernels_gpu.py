@@ -355,6 +355,61 @@ def test_linear_few_rows_streams_weights(M, N, K):
         assert torch.equal(alone[0], got[0])
 
 
+@pytest.mark.parametrize("M,N,K", [(17, 4096, 4096), (64, 6144, 4096), (200, 1000, 2056), (576, 5120, 1024),
+                                   (2048, 768, 512), (33, 331, 72), (40, 129, 515)])
+def test_linear_many_rows_is_the_library_kernel_that_was_fastest(M, N, K):
+    """More than 16 bfloat16 rows go to the vendor library, which times its candidates once
+    for a size; the choice holds from then on, also inside a graph, and a size it has no
+    kernel for takes the other route."""
+    ops = _ops()
+    x = _rand((M, K), torch.bfloat16, 41)
+    w = _rand((N, K), torch.bfloat16, 42, scale=0.05)
+    want = x.double() @ w.double().T
+    got = ops.linear(x, w, out_dtype=torch.float32)
+    torch.testing.assert_close(got.double(), want, rtol=2e-3, atol=2e-3)
+    got16 = ops.linear(x, w)
+    torch.testing.assert_close(got16.double(), want, rtol=1.6e-2, atol=1e-2)
+    plan = ops.matmul_plan(M, N, K)
+    if K % 8 == 0:
+        assert plan is not None and plan[0] >= 1 and 0 <= plan[1] < plan[0]
+        assert plan[3] <= plan[2] or plan[0] == 1          # the chosen one was no slower than the first
+    assert torch.equal(ops.linear(x, w), got16)            # and stays chosen
+    # rows do not mix: a row's result is the same whatever its neighbours hold
+    other = x.clone()
+    other[1:] = _rand((M - 1, K), torch.bfloat16, 43)
+    assert torch.equal(ops.linear(other, w)[0], got16[0])
+
+
+def test_linear_many_rows_first_met_in_a_graph():
+    """A size first met while a graph is captured runs untimed there, is timed at its next
+    eager call, and the graph's replays keep giving the right product."""
+    ops = _ops()
+    M, N, K = 48, 1184, 608
+    x = _rand((M, K), torch.bfloat16, 44)
+    w = _rand((N, K), torch.bfloat16, 45, scale=0.05)
+    ops.linear(_rand((20, 64), torch.bfloat16, 1), _rand((64, 64), torch.bfloat16, 2))   # the device's set-up is eager
+    out = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    assert ops.matmul_plan(M, N, K) is None
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            ops.linear(x, w, out=out)
+    torch.cuda.current_stream().wait_stream(side)
+    assert ops.matmul_plan(M, N, K)[0] == 1
+    want = x.double() @ w.double().T
+    for seed in (46, 47, 48):
+        out.zero_()
+        graph.replay()
+        torch.testing.assert_close(out.double(), want, rtol=1.6e-2, atol=1e-2)
+        eager = ops.linear(x, w)                               # timed at the first of these
+        torch.testing.assert_close(eager.double(), want, rtol=1.6e-2, atol=1e-2)
+        x.copy_(_rand((M, K), torch.bfloat16, seed))
+        want = x.double() @ w.double().T
+    assert ops.matmul_plan(M, N, K)[0] > 1
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 6144, 4096), (8, 4096, 12288), (16, 1000, 96), (3, 331, 64), (9, 24, 2048),
                                    (5, 151936, 256)])
 def test_linear_from_the_tiled_copy(M, N, K):

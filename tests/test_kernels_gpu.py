@@ -272,6 +272,32 @@ def test_paged_attention_portions_over_long_prefixes():
     torch.testing.assert_close(got.float(), want, rtol=2e-2, atol=2e-2)
 
 
+def test_paged_attention_contexts_of_tens_of_thousands():
+    """Contexts whose block tables are longer than what the prompt kernel keeps in shared memory
+    at a time (508 pages: 8,128 keys of page 16), and that the decoding kernel cuts into its
+    largest number of splits. A key on either side of such an edge is made to dominate the last
+    row of a portion and a single token."""
+    ops = _ops()
+    Hq, Hkv, D, page = 8, 2, 128, 16
+    G = Hq // Hkv
+    q_lens, kv_lens = [300, 1, 40], [20000, 40000, 8200]
+    scale = D ** -0.5
+    for far in (8127, 8128, 16255, 16256, 19999 - 300):
+        q, kc, vc, bt, cu, kvl = _paged_case(torch.bfloat16, 3, Hq, Hkv, D, page, q_lens, kv_lens, 50 + far % 7,
+                                             spread=False)
+        last_rows = (q_lens[0] - 1, q_lens[0])           # the portion's last row, the single token
+        for b, row in enumerate(last_rows):
+            pg = int(bt[b, far // page])
+            kc[pg, :, far % page] = (q[row].view(Hkv, G, D)[:, 0] * 4).to(torch.bfloat16)
+        got = ops.paged_attention(q, Hq, kc, vc, bt, cu, kvl, max(q_lens), max(kv_lens), scale, min_q_len=1)
+        want = torch_ops.paged_attention(q.float(), Hq, kc.float(), vc.float(), bt, cu, kvl, max(q_lens),
+                                         max(kv_lens), scale)
+        torch.testing.assert_close(got.float(), want, rtol=2e-2, atol=2e-2)
+        for b, row in enumerate(last_rows):
+            v_far = vc[int(bt[b, far // page]), :, :, far % page].float()
+            assert (got[row].float().view(Hq, D)[::G] - v_far).abs().max() < 0.2, (far, b)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_paged_attention_far_key_stands_out(dtype):
     """One key far back is made to dominate: a kernel that drops, repeats or

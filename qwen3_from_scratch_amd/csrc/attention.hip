@@ -211,8 +211,7 @@ __device__ __forceinline__ Pack16 softmax_step(const f32x4_t (&s)[2], bool full,
     }
   }
   float mx = fmaxf(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])), fmaxf(fmaxf(v[4], v[5]), fmaxf(v[6], v[7])));
-  mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-  mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+  mx = quad_rows_max(mx);
   const float m_new = fmaxf(m_run, mx * scale_log2);
   Pack16 p;
   float sum = 0.f;
@@ -833,8 +832,7 @@ __device__ __forceinline__ void softmax_tile(const f32x4_t (&s)[KB4], bool full,
   float mx = v[0];
 #pragma unroll
   for (int j = 1; j < N; ++j) mx = fmaxf(mx, v[j]);
-  mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-  mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+  mx = quad_rows_max(mx);
   const float m_new = fmaxf(m_run, mx * scale_log2);
   float sum = 0.f;
   if (m_new > -INFINITY) {
@@ -869,6 +867,9 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
   constexpr int KB4 = TILE / 16;  // 16-key blocks per tile
   __shared__ __attribute__((aligned(16))) unsigned char smem[STAGES * SM::STAGE];
   __shared__ int sh_pages[PREFILL_PAGES];  // the block-table entries of the tiles in hand
+  // and where each entry's (page, this key head) begins in either cache, in elements: worked out
+  // once per entry, so that a tile's loads find their addresses with a few additions
+  __shared__ long long sh_base[PREFILL_PAGES];
   const int b = blockIdx.z, g_kv = blockIdx.x;
   const int G = Hq / Hkv;
   const int q0 = cu_q[b];
@@ -964,42 +965,45 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
     v_h[j] = q & 1;
   }
   const size_t page_elems = (size_t)page * D;  // elements of one (page, head) in either cache
-  typedef __attribute__((address_space(3))) void* lds_ptr;
+  int v_in[V_TURNS];                           // a value piece's place in its page, but for the key's
+#pragma unroll
+  for (int j = 0; j < V_TURNS; ++j) v_in[j] = v_d[j] * page + 8 * v_h[j];
+  // A load of 16 bytes per lane that writes shared memory directly: lane L's bytes land at
+  // `lds` + 16 L (`lds` the same in all lanes). It is written as assembly on purpose: for the
+  // compiler's own form of this instruction the compiler makes every later read of shared
+  // memory wait until no load at all is outstanding, since it cannot tell the stage being
+  // filled from the stage being read, and the next tile's copy would not overlap with this
+  // tile's work in the same wavefront. What orders these loads against the reads is
+  // `wait_for_tile` and the barrier after it.
+  typedef __attribute__((address_space(3))) unsigned char* lds_ptr;
+  const unsigned smem_lds = (unsigned)(unsigned long)(lds_ptr)smem;
+  auto load_to_lds = [&](const void* src, unsigned lds) {
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds) : "memory", "m0");
+  };
 
   auto plain_tile = [&](int t) { return t * TILE + TILE <= kv_len && window == 0; };
-  // the pages of a tile's 16-key blocks, looked up once per tile (every lane reads the same few
-  // table entries, all in one go) rather than once per load
-  constexpr int KB4_ = TILE / 16;
-  auto tile_pages = [&](int t, int (&pg)[KB4_]) {
-#pragma unroll
-    for (int kb = 0; kb < KB4_; ++kb) pg[kb] = sh_pages[((t * TILE + 16 * kb) >> page_shift) - page_base];
-#pragma unroll
-    for (int kb = 0; kb < KB4_; ++kb) pg[kb] = min(max(pg[kb], 0), num_pages - 1);
-  };
   auto copy_direct = [&](int t, int stage) {
     const int key0 = t * TILE;
-    unsigned char* ks = smem + stage * SM::STAGE + 1024 * wave;  // this wavefront's kilobyte of each turn
-    unsigned char* vs = ks + SM::K_BYTES;
-    int pg[KB4_];
-    tile_pages(t, pg);
+    // this wavefront's kilobyte of each turn
+    const unsigned ks = __builtin_amdgcn_readfirstlane(smem_lds + stage * SM::STAGE + 1024 * wave);
+    const unsigned vs = ks + SM::K_BYTES;
+    long long base[K_TURNS + V_TURNS];
+    int key[K_TURNS + V_TURNS];
+#pragma unroll
+    for (int j = 0; j < K_TURNS; ++j) key[j] = key0 + k_row[j];
+#pragma unroll
+    for (int j = 0; j < V_TURNS; ++j) key[K_TURNS + j] = key0 + 16 * v_kb[j];
+#pragma unroll
+    for (int j = 0; j < K_TURNS + V_TURNS; ++j) base[j] = sh_base[(key[j] >> page_shift) - page_base];
 #pragma unroll
     for (int j = 0; j < K_TURNS; ++j) {
-      const int key = key0 + k_row[j];
-      int mine = pg[0];
-#pragma unroll
-      for (int kb = 1; kb < KB4_; ++kb) mine = (k_row[j] >> 4) == kb ? pg[kb] : mine;
-      const bf16_t* src = k_cache + (size_t)(mine * Hkv + g_kv) * page_elems + ((key & (page - 1)) * D + k_off[j]);
-      __builtin_amdgcn_global_load_lds(src, (lds_ptr)(ks + 4096 * j), 16, 0, 0);
+      const int in = (key[j] & (page - 1)) * D + k_off[j];
+      load_to_lds(k_cache + (base[j] + in), ks + 4096 * j);
     }
 #pragma unroll
     for (int j = 0; j < V_TURNS; ++j) {
-      const int key = key0 + 16 * v_kb[j];
-      int mine = pg[0];
-#pragma unroll
-      for (int kb = 1; kb < KB4_; ++kb) mine = v_kb[j] == kb ? pg[kb] : mine;
-      const bf16_t* src =
-          v_cache + (size_t)(mine * Hkv + g_kv) * page_elems + (v_d[j] * page + (key & (page - 1)) + 8 * v_h[j]);
-      __builtin_amdgcn_global_load_lds(src, (lds_ptr)(vs + 4096 * j), 16, 0, 0);
+      const int in = v_in[j] + (key[K_TURNS + j] & (page - 1));
+      load_to_lds(v_cache + (base[K_TURNS + j] + in), vs + 4096 * j);
     }
   };
   auto copy_checked = [&](int t, int stage) {
@@ -1052,6 +1056,15 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
   const int v_swz = (col / SM::VRW) % SM::VPR;
   constexpr int LOADS_PER_TILE = K_TURNS + V_TURNS;  // this thread's loads in flight per tile on its way
 
+  // The query rows are used here, before the tile loop, so that the compiler waits for their
+  // loads here: a wait it would otherwise place at their first use inside the loop, where it
+  // would also wait, every time round, for the next tile's copy (the compiler counts loads,
+  // and does not know of those it did not issue).
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+    for (int i = 0; i < D / 32; ++i) asm volatile("" : "+v"(qreg[qb][i].v));
+
   // tiles are worked through in spans whose table entries fit sh_pages
   const int tiles_per_span = max(1, (PREFILL_PAGES - 4) * page / TILE);
   for (int span_lo = tile_lo; span_lo < tile_hi; span_lo += tiles_per_span) {
@@ -1060,7 +1073,11 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
     page_base = (span_lo * TILE) >> page_shift;
     {
       const int last_page = min((kv_len - 1) >> page_shift, (span_hi * TILE - 1) >> page_shift);
-      for (int i = tid; page_base + i <= last_page; i += 256) sh_pages[i] = bt_row[page_base + i];
+      for (int i = tid; page_base + i <= last_page; i += 256) {
+        const int pg = bt_row[page_base + i];
+        sh_pages[i] = pg;
+        sh_base[i] = (long long)(min(max(pg, 0), num_pages - 1) * Hkv + g_kv) * (long long)page_elems;
+      }
     }
     __syncthreads();
     // STAGES - 1 tiles are on their way at any time: the first ones here, then tile

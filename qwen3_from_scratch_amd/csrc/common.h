@@ -71,6 +71,27 @@ __device__ inline float wave_max(float v) {
   return v;
 }
 
+// The maximum (sum) over the four lanes l, l ^ 16, l ^ 32, l ^ 48, in all of them: two lane
+// swaps in the vector unit (rows of 16 lanes, then halves of 32) instead of two round trips
+// through shared memory, which is what a shuffle by 16 or 32 lanes compiles to.
+__device__ inline float quad_rows_max(float v) {
+  unsigned u = __float_as_uint(v);
+  auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  u = __float_as_uint(v);
+  auto b = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+
+__device__ inline float quad_rows_sum(float v) {
+  unsigned u = __float_as_uint(v);
+  auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  u = __float_as_uint(v);
+  auto b = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
 // Sum over a block of up to 1024 threads; every thread gets the result.
 // `scratch` holds at least 17 floats of shared memory.
 __device__ inline float block_sum(float v, float* scratch) {

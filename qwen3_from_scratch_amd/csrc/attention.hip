@@ -797,12 +797,16 @@ struct PrefillSmem {
   // 16-byte pieces in an order chosen so that the matrix-core operand reads spread over all
   // banks without padding (the loads that fill a stage write whole kilobytes, see below).
   // A window is 256 bytes. Keys: a window = RPW rows of CPR pieces; piece c of row r sits at
-  // place (r % RPW) * CPR + (c ^ (window % CPR)) of window r / RPW. Values: a window = VRW
-  // rows of VPR pieces (a piece = eight keys of one 16-key block: q = 2 * block + half);
-  // piece q of row d sits at place (d % VRW) * VPR + (q ^ (window % VPR)) of window d / VRW.
+  // place (r % RPW) * CPR + (c ^ (window % CPR)) of window r / RPW. Values (a piece = eight
+  // keys of one 16-key block): sixteen rows' pieces of the tile's first half of blocks are
+  // followed by the same rows' pieces of its second half (two planes), so that the two 8-byte
+  // reads that make one operand of the second product (four keys of block h, four of block
+  // h + blocks / 2) are a fixed, short distance apart and one instruction fetches both. A
+  // plane's sixteen rows are VPR windows of VRW rows of VPR pieces (q = 2 * (block in the
+  // plane) + half); piece q of row d sits at place (d % VRW) * VPR + (q ^ window) of its window.
   static constexpr int CPR = D / 8;          // 16-byte pieces per key row
   static constexpr int RPW = 16 / CPR > 0 ? 16 / CPR : 1;   // key rows per window (D <= 128)
-  static constexpr int VPR = TILE / 8;       // pieces per value row
+  static constexpr int VPR = TILE / 16;      // pieces per value row in a plane
   static constexpr int VRW = 16 / VPR;       // value rows per window
   static constexpr int K_BYTES = TILE * D * 2;
   static constexpr int V_BYTES = D * TILE * 2;
@@ -840,7 +844,7 @@ __device__ __forceinline__ void softmax_tile(const f32x4_t (&s)[KB4], bool full,
     for (int j = 0; j < N; ++j) {
       const float e = fast_exp2(fmaf(v[j], scale_log2, -m_new));
       sum += e;
-      p[j >> 3].e[j & 7] = (__bf16)e;
+      p[(j >> 2) % (KB4 / 2)].e[4 * ((j >> 2) / (KB4 / 2)) + (j & 3)] = (__bf16)e;  // block kb goes with kb + KB4 / 2
     }
   } else {
 #pragma unroll
@@ -858,7 +862,7 @@ __device__ __forceinline__ void softmax_tile(const f32x4_t (&s)[KB4], bool full,
 }
 
 template <int D, int TILE, int STAGES>
-__global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_prefill_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, int num_pages, const int* __restrict__ block_table, int bt_stride,
     const int* __restrict__ cu_q, const int* __restrict__ kv_lens, int Hq, int Hkv, int page, float scale_log2,
@@ -958,10 +962,11 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
   }
 #pragma unroll
   for (int j = 0; j < V_TURNS; ++j) {
-    const int place = tid + 256 * j, w = place >> 4, u = place & 15;
-    const int q = (u % SM::VPR) ^ (w % SM::VPR);
-    v_d[j] = SM::VRW * w + u / SM::VPR;
-    v_kb[j] = q >> 1;
+    const int place = tid + 256 * j, rows16 = place / (SM::VPR * 32), plane = (place / (SM::VPR * 16)) & 1;
+    const int w = (place >> 4) % SM::VPR, u = place & 15;
+    const int q = (u % SM::VPR) ^ w;
+    v_d[j] = 16 * rows16 + SM::VRW * w + u / SM::VPR;
+    v_kb[j] = plane * (TILE / 32) + (q >> 1);
     v_h[j] = q & 1;
   }
   const size_t page_elems = (size_t)page * D;  // elements of one (page, head) in either cache
@@ -1054,6 +1059,11 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
   const int k_swz = (col / SM::RPW) % SM::CPR;
   const int v_lane = (col / SM::VRW) * 256 + (col % SM::VRW) * SM::VPR * 16 + 8 * (grp & 1);
   const int v_swz = (col / SM::VRW) % SM::VPR;
+  int k_read[D / 32], v_read[TILE / 32];
+#pragma unroll
+  for (int i = 0; i < D / 32; ++i) k_read[i] = k_lane + 16 * ((4 * i + grp) ^ k_swz);
+#pragma unroll
+  for (int h = 0; h < TILE / 32; ++h) v_read[h] = v_lane + 16 * ((2 * h + (grp >> 1)) ^ v_swz);
   constexpr int LOADS_PER_TILE = K_TURNS + V_TURNS;  // this thread's loads in flight per tile on its way
 
   // The query rows are used here, before the tile loop, so that the compiler waits for their
@@ -1111,8 +1121,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
           Pack16 a[D / 32];
 #pragma unroll
           for (int i = 0; i < D / 32; ++i)
-            a[i].u = *reinterpret_cast<const uint4*>(ks + (16 / SM::RPW) * 256 * kb4 + k_lane +
-                                                     16 * ((4 * i + grp) ^ k_swz));
+            a[i].u = *reinterpret_cast<const uint4*>(ks + (16 / SM::RPW) * 256 * kb4 + k_read[i]);
 #pragma unroll
           for (int qb = 0; qb < 2; ++qb) {
             f32x4_t c = {0.f, 0.f, 0.f, 0.f};
@@ -1129,19 +1138,37 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
         for (int qb = 0; qb < 2; ++qb)
           softmax_tile<D / 16, KB4>(sc[qb], full, key0, grp, row_pos[qb], window, scale_log2, m_run[qb], l_run[qb],
                                     acc[qb], p[qb]);
+        // the values' operands (keys 4 grp .. 4 grp + 3 of blocks half and half + KB4 / 2) are
+        // read one group of output columns ahead of the matrix instructions that use them
+        Pack16 vt[4][KB4 / 2];
+        auto read_values = [&](int nb, Pack16 (&to)[KB4 / 2]) {
 #pragma unroll
-        for (int nb = 0; nb < D / 16; ++nb)
-#pragma unroll
-          for (int half = 0; half < KB4 / 2; ++half) {
-            Pack16 vt;  // keys 4 grp .. 4 grp + 3 of the half's two 16-key blocks
+          for (int half = 0; half < KB4 / 2; ++half)
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
-              vt.h[kb] = *reinterpret_cast<const uint2*>(vs + (16 / SM::VRW) * 256 * nb + v_lane +
-                                                        16 * ((2 * (2 * half + kb) + (grp >> 1)) ^ v_swz));
+              to[half].h[kb] = *reinterpret_cast<const uint2*>(vs + (2 * nb + kb) * SM::VPR * 256 + v_read[half]);
+        };
+        read_values(0, vt[0]);
+        read_values(1, vt[1]);
+#pragma unroll
+        for (int nb = 0; nb < D / 16; ++nb) {
+          if (nb + 2 < D / 16) read_values(nb + 2, vt[(nb + 2) & 3]);
+#pragma unroll
+          for (int half = 0; half < KB4 / 2; ++half)
 #pragma unroll
             for (int qb = 0; qb < 2; ++qb)
-              acc[qb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt.v, p[qb][half].v, acc[qb][nb], 0, 0, 0);
-          }
+              acc[qb][nb] =
+                  __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt[nb & 3][half].v, p[qb][half].v, acc[qb][nb], 0, 0, 0);
+        }
+        // the order the compiler is to keep (left to itself it reads each operand right before
+        // its use, into the same registers, and waits for it every time): four reads ahead
+        __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+        for (int i = 0; i < (D / 16) * (KB4 / 2) - 4; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
       }
       // this wavefront's share of the next tile has landed; the tiles after it may still travel
       wait_for_tile(min(t + STAGES - 1, span_hi - 1) - (t + 1));

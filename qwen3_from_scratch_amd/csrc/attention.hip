@@ -821,34 +821,41 @@ __device__ __forceinline__ void softmax_tile(const f32x4_t (&s)[KB4], bool full,
                                              int window, float scale_log2, float& m_run, float& l_run,
                                              f32x4_t (&acc)[NB], Pack16 (&p)[KB4 / 2]) {
   constexpr int N = 4 * KB4;
+  static_assert(N % 2 == 0, "maxima are taken three at a time");
   float v[N];
 #pragma unroll
   for (int j = 0; j < N; ++j) v[j] = s[j >> 2][j & 3];
   if (!full) {
+    // (the row's position goes through an empty piece of assembly so that the comparisons'
+    // operands are worked out here, where they are needed, and not before the branch for
+    // every tile)
+    int pos = row_pos;
+    asm volatile("" : "+v"(pos));
 #pragma unroll
     for (int j = 0; j < N; ++j) {
       const int key = key0 + 16 * (j >> 2) + 4 * grp + (j & 3);
-      bool seen = key <= row_pos;
-      if (window > 0 && row_pos - key >= window) seen = false;
+      bool seen = key <= pos;
+      if (window > 0 && pos - key >= window) seen = false;
       if (!seen) v[j] = -INFINITY;
     }
   }
-  float mx = v[0];
+  // the scores are matrix results or minus infinity, never NaN: the three-operand maximum as
+  // it is (the compiler's own first makes every operand a quiet NaN, one instruction each)
+  float mx;
+  asm("v_max_f32 %0, %1, %2" : "=v"(mx) : "v"(v[0]), "v"(v[1]));
 #pragma unroll
-  for (int j = 1; j < N; ++j) mx = fmaxf(mx, v[j]);
+  for (int j = 2; j < N; j += 2) asm("v_max3_f32 %0, %1, %2, %3" : "=v"(mx) : "v"(mx), "v"(v[j]), "v"(v[j + 1]));
   mx = quad_rows_max(mx);
   const float m_new = fmaxf(m_run, mx * scale_log2);
+  // a row that has seen no key yet has minus infinity here and in all its scores: its terms are
+  // exp2(-inf - 0) = 0
+  const float m_use = m_new > -INFINITY ? m_new : 0.f;
   float sum = 0.f;
-  if (m_new > -INFINITY) {
 #pragma unroll
-    for (int j = 0; j < N; ++j) {
-      const float e = fast_exp2(fmaf(v[j], scale_log2, -m_new));
-      sum += e;
-      p[(j >> 2) % (KB4 / 2)].e[4 * ((j >> 2) / (KB4 / 2)) + (j & 3)] = (__bf16)e;  // block kb goes with kb + KB4 / 2
-    }
-  } else {
-#pragma unroll
-    for (int h = 0; h < KB4 / 2; ++h) p[h].u = make_uint4(0, 0, 0, 0);
+  for (int j = 0; j < N; ++j) {
+    const float e = fast_exp2(fmaf(v[j], scale_log2, -m_use));
+    sum += e;
+    p[(j >> 2) % (KB4 / 2)].e[4 * ((j >> 2) / (KB4 / 2)) + (j & 3)] = (__bf16)e;  // block kb goes with kb + KB4 / 2
   }
   const bool moved = m_new != m_run;
   if (__builtin_amdgcn_ballot_w64(moved) != 0) {

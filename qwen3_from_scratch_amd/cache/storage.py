@@ -25,23 +25,32 @@ class CacheStorage:
     the page, so that the keys a matrix-core lane multiplies together lie side
     by side in memory and need no transposition on the way to the registers.
     Per state group one tensor (planes, slots, *shape), zeroed per slot at
-    admission."""
+    admission. Every group has one page, and every state group one slot, more
+    than the manager hands out (`spare_page`, `spare_slot`): rows that only
+    fill a batch up to a size a captured graph exists for write there."""
 
     def __init__(self, manager, act_dtype, device):
         self.manager = manager
         self.device = torch.device(device)
         self.keys, self.values = [], []
         for grp in manager.groups:
-            shape = (len(grp.planes), grp.pool.num_pages, grp.kv_heads, manager.page_size, grp.head_dim)
+            shape = (len(grp.planes), grp.pool.num_pages + 1, grp.kv_heads, manager.page_size, grp.head_dim)
             self.keys.append(torch.zeros(shape, dtype=act_dtype, device=self.device))
             self.values.append(torch.zeros(shape[:3] + (grp.head_dim, manager.page_size),
                                            dtype=act_dtype, device=self.device))
         self.states = []
         for grp in manager.state_groups:
             self.states.append(torch.zeros(
-                (len(grp.planes), manager.max_requests) + tuple(grp.shape),
+                (len(grp.planes), manager.max_requests + 1) + tuple(grp.shape),
                 dtype=grp.dtype, device=self.device))
         self._block_tables = None
+
+    def spare_page(self, group):
+        return self.manager.groups[group].pool.num_pages
+
+    @property
+    def spare_slot(self):
+        return self.manager.max_requests
 
     def bytes(self):
         return sum(t.numel() * t.element_size() for t in self.keys + self.values + self.states)

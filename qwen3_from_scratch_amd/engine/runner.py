@@ -6,9 +6,25 @@ from ..cache import CacheManager, CacheStorage
 from .batch import StepEntry, pack_step, packed_size
 
 
+def padded_batch(n):
+    """The batch size a graph is captured for when `n` requests decode: the
+    next of 1, 2, 3, 4, 6, 8, 12, 16, 24, ... so that batches whose size moves up
+    and down as requests come and go share a few graphs. The rows that fill a
+    batch up stand for nobody: token 0 at position 0, written to the cache's
+    spare page and slot, their logits dropped."""
+    size = 1
+    while size < n:
+        if size < 4:
+            size += 1
+        else:                       # a power of two is followed by its one-and-a-half, that by the next power
+            size = size * 3 // 2 if size & (size - 1) == 0 else size * 4 // 3
+    return size
+
+
 class _DecodeGraph:
-    """A captured HIP graph of the model's forward pass for `B` requests with
-    one token each, none longer than `max_kv_len`. The batch description lives
+    """A captured HIP graph of the model's forward pass for `B` rows of one
+    token each, none longer than `max_kv_len`; the first rows are the step's
+    requests, the rest fill up (see `padded_batch`). The batch description lives
     in fixed device memory that is refilled before every replay; what the
     kernels' launches depend on (the longest sequence, hence how keys are
     split over workgroups) is fixed at `max_kv_len`, a power of two, so a
@@ -34,14 +50,19 @@ class _DecodeGraph:
                 and all(n == m + 1 for n, m in zip(lengths, self.last_lengths))):
             self._advance(runner, entries, tables)
         else:
-            batch, block_tables = pack_step(entries, lengths, slots, tables, runner.device,
-                                            fixed_widths=self.widths, buffers=(self.host, self.dev), all_rows=True)
+            fill = self.B - len(entries)
+            storage = runner.storage
+            batch, block_tables = pack_step(
+                list(entries) + [StepEntry(None, [0])] * fill, list(lengths) + [0] * fill,
+                list(slots) + [storage.spare_slot] * fill,
+                [list(group) + [[storage.spare_page(g)]] * fill for g, group in enumerate(tables)],
+                runner.device, fixed_widths=self.widths, buffers=(self.host, self.dev), all_rows=True)
             batch.max_kv_len = self.max_kv_len
             if self.graph is None:
                 self._capture(runner, batch, block_tables)
         self.copied.record()
         if device_tokens is not None:      # the tokens are still on the device: they replace the placeholders
-            self.dev[0:self.B].copy_(device_tokens)
+            self.dev[0:len(entries)].copy_(device_tokens)
         self.last_ids, self.last_lengths, self.last_slots = ids, list(lengths), list(slots)
         self.last_table_lens = [[len(t) for t in group] for group in tables]
         self.graph.replay()
@@ -52,10 +73,10 @@ class _DecodeGraph:
         packed description changes in its tokens, by one in positions and
         lengths, and in the block tables' new entries (all entries where a
         window gives pages back)."""
-        B, host = self.B, self.host.numpy()
-        host[0:B] = [e.tokens[0] for e in entries]
-        host[B:2 * B] += 1                        # positions
-        host[4 * B + 1:5 * B + 1] += 1            # keys visible after the step
+        B, n, host = self.B, len(entries), self.host.numpy()
+        host[0:n] = [e.tokens[0] for e in entries]
+        host[B:B + n] += 1                        # positions (the rows that fill up stay where they are)
+        host[4 * B + 1:4 * B + 1 + n] += 1        # keys visible after the step
         base = 7 * B + 1
         for g, (group_tables, w) in enumerate(zip(tables, self.widths)):
             windowed = runner.manager.groups[g].window > 0
@@ -169,21 +190,22 @@ class ModelRunner:
 
     def _step_graph(self, entries, lengths, slots, tables, device_tokens=None):
         B = len(entries)
+        rows = padded_batch(B)
         longest = max(lengths) + 1
         bucket = 256
         while bucket < longest:
             bucket *= 2
         bucket = min(bucket, self.max_request_tokens)
-        graph = self._graphs.pop((B, bucket), None)
+        graph = self._graphs.pop((rows, bucket), None)
         if graph is None:
             if len(self._graphs) >= self.max_graphs:       # drop the one used longest ago
                 self._graphs.pop(next(iter(self._graphs)))
-            graph = _DecodeGraph(self, B, bucket)
-        self._graphs[(B, bucket)] = graph                   # most recently used last
+            graph = _DecodeGraph(self, rows, bucket)
+        self._graphs[(rows, bucket)] = graph                # most recently used last
         logits = graph.run(self, entries, lengths, slots, tables, device_tokens)
         wanted = [i for i, e in enumerate(entries) for _ in e.want]
         if wanted == list(range(B)):
-            return logits
+            return logits if rows == B else logits.narrow(0, 0, B)
         index = torch.tensor(wanted, dtype=torch.long, device=self.device)
         return logits.index_select(0, index)
 

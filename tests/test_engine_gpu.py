@@ -3,6 +3,8 @@ bfloat16: every request alone and whole; most of it in one step and the last 32
 tokens one by one; portions of changing size; mixed batches with so few pages
 that they are used again; long decoding; the first tokens of a sequence."""
 
+import random
+
 import pytest
 import torch
 
@@ -111,3 +113,34 @@ def test_graph_replay_equals_eager_steps(model_folders):
     assert a.keys() == b.keys()
     worst = max(float((a[k] - b[k]).abs().max()) for k in a)
     assert worst < 2e-2, worst
+
+
+def test_batches_of_nearby_sizes_share_a_graph(model_folders):
+    """Decoding batches of 11, 9, 10, 5, 7 and 6 requests replay graphs captured for 12, 6 and 8
+    rows; the rows that fill a batch up change no request's logits and leave no trace in the
+    cache, and steps in between that leave requests out go on correctly."""
+    name = "D"
+    vocab = TINY[name]["config"]["vocab_size"]
+    requests = {"r%d" % i: random_tokens(20 + 3 * i, vocab, 60 + i) for i in range(11)}
+    steps = [([(rid, toks[:-8], [])], []) for rid, toks in requests.items()]       # prompts, one a step
+    fed = {rid: len(toks) - 8 for rid, toks in requests.items()}
+    for size, seed in [(11, 0), (9, 1), (10, 2), (5, 3), (7, 4), (6, 5), (11, 6), (6, 7)]:
+        chosen = random.Random(seed).sample(sorted(requests), size)
+        entries = []
+        for rid in chosen:
+            entries.append((rid, [requests[rid][fed[rid]]], [0]))
+            fed[rid] += 1
+        steps.append((entries, []))
+    steps.append(([], list(requests)))
+    kw = dict(dtype="bfloat16", device="cuda", page_size=16, max_tokens=max_live_tokens(steps, page=16),
+              max_requests=12)
+    with_graphs = load_runner(model_folders[name], use_graphs=True, **kw)
+    a = run_trace(with_graphs, steps)
+    b = run_trace(load_runner(model_folders[name], use_graphs=False, **kw), steps)
+    assert a.keys() == b.keys() and len(a) == 11 + 9 + 10 + 5 + 7 + 6 + 11 + 6
+    worst = max(float((a[k] - b[k]).abs().max()) for k in a)
+    assert worst < 2e-2, worst
+    assert sorted(rows for rows, _ in with_graphs._graphs) == [6, 8, 12]
+    with_graphs.manager.audit()
+    assert all(g.pool.num_free == g.pool.num_pages for g in with_graphs.manager.groups)
+

@@ -1,7 +1,7 @@
 """Decode and prefill throughput of the Qwen3-8B-shaped model on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L]
-                    [--shape 8b|14b|32b] [--prompt P] [--context C]
+                    [--shape 8b|14b|32b] [--prompt P] [--context C] [--workload decode|continuous]
 
 Random bfloat16 weights, uniform-random prompts of 2,048 tokens, greedy decoding
 through the engine's own step loop (scheduler, step function, sampling). A
@@ -54,6 +54,49 @@ def prefill_flops(c, tokens):
     return gemm + attn
 
 
+def continuous(args, config, model, shape_name, gen, sync):
+    """64 requests admitted at once and served by continuous batching: prompt lengths uniform in
+    [128, 4096], generated tokens uniform in [64, 512], prompts cut into portions of 512 beside
+    the decoding requests, a budget of 576 tokens a step. Run twice; the second run (graphs
+    captured, library kernels chosen) is the one reported."""
+    import random
+
+    import torch
+
+    from qwen3_from_scratch_amd.engine import SyncEngine
+
+    requests, portion, context = 64, 512, 8192
+    rng = random.Random(0)
+    sizes = [(rng.randint(128, 4096), rng.randint(64, 512)) for _ in range(requests)]
+    engine = SyncEngine(model=model, path="", dtype=args.dtype, device="cuda:0", max_len=context, block_size=BLOCK,
+                        num_blocks=requests * context // BLOCK // 2, max_num_seqs=requests,
+                        max_num_tokens=portion + requests, chunked_prefill_size=portion)
+    for _ in range(2):
+        for prompt, generated in sizes:
+            engine.add_request(torch.randint(0, config.vocab_size, (prompt,), generator=gen).tolist(),
+                               engine.default_params(generated, temperature=0.0, ignore_eos=True))
+        sync()
+        t0 = time.perf_counter()
+        steps = 0
+        while engine.scheduler.has_work():
+            engine.step()
+            steps += 1
+        sync()
+        seconds = time.perf_counter() - t0
+    tokens_in, tokens_out = sum(p for p, _ in sizes), sum(g for _, g in sizes)
+    print(json.dumps({
+        "metric": "continuous batching, tokens/s in and out, %s bf16" % shape_name,
+        "value": round((tokens_in + tokens_out) / seconds, 1), "unit": "tokens/s", "n_gpus": 1,
+        "higher_is_better": True, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
+        "seconds": round(seconds, 3), "steps": steps, "generated_tokens_per_s": round(tokens_out / seconds, 1),
+        "config": {"model": "%s-shaped, random weights N(0, 0.02)" % shape_name, "requests": requests,
+                   "prompt_tokens": tokens_in, "generated_tokens": tokens_out, "prefill_portion": portion,
+                   "step_token_budget": portion + requests, "context_len": context, "kv_block_size": BLOCK,
+                   "layers": config.num_hidden_layers, "sampling": "greedy"},
+    }))
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -65,6 +108,9 @@ def main():
     ap.add_argument("--shape", default="8b", choices=sorted(SHAPES))
     ap.add_argument("--prompt", type=int, default=2048, help="tokens every request holds when decoding starts")
     ap.add_argument("--context", type=int, default=8192, help="tokens of cache per request")
+    ap.add_argument("--workload", default="decode", choices=["decode", "continuous"],
+                    help="continuous: 64 requests at once, prompts of 128 to 4,096 tokens, 64 to 512 generated "
+                         "tokens each, prompts in portions of 512 (its own JSON line; --steps and --warmup unused)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 points")
     ap.add_argument("--skip-prefill", action="store_true",
                     help="skip the prefill measurement (for profiles of decoding alone; the line then has no value for it)")
@@ -104,6 +150,9 @@ def main():
 
     def sync():
         torch.cuda.synchronize()
+
+    if args.workload == "continuous":
+        return continuous(args, config, model, shape_name, gen, sync)
 
     # ---- prefill: one prompt of 2,048 tokens in one step ----
     engine = engine_for(1)

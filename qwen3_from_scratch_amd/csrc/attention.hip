@@ -1206,8 +1206,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 template <int D>
 static int launch_fast(const void* q, int q_stride, void* out, const void* k_cache, const void* v_cache,
                        int num_pages, const int* block_table, int bt_stride, const int* cu_q, const int* kv_lens,
-                       int B, int Hq, int Hkv, int page, float scale, int window, int max_q_len, int min_q_len,
-                       int splits, float* ws_acc, float* ws_ml, hipStream_t stream) {
+                       int B, int total_tokens, int Hq, int Hkv, int page, float scale, int window, int max_q_len,
+                       int min_q_len, int splits, float* ws_acc, float* ws_ml, hipStream_t stream) {
   const int G = Hq / Hkv;
   const float scale_log2 = scale * 1.4426950408889634f;
   if (min_q_len * G <= 16) {
@@ -1220,7 +1220,12 @@ static int launch_fast(const void* q, int q_stride, void* out, const void* k_cac
                          Hkv, splits, ws_acc, ws_ml);
   }
   if (max_q_len * G > 16) {
-    const int tokens_per_block = 128 / G;
+    // A block owns 128 rows; with so few rows that not every CU gets a block (a portion of 512
+    // tokens of one prompt: 128 blocks), a block's rows are halved until they do, down to one
+    // wavefront's 32 (its other wavefronts then only help to copy the tiles).
+    int tokens_per_block = 128 / G;
+    while (Hkv * ((total_tokens + tokens_per_block - 1) / tokens_per_block) < 256 && (tokens_per_block / 2) * G >= 32)
+      tokens_per_block /= 2;
     const int tiles = (max_q_len + tokens_per_block - 1) / tokens_per_block;
     if (tiles > 65535) return Q3_ERR_UNSUPPORTED;
     hipLaunchKernelGGL((attn_prefill_kernel<D, PF_TILE, PF_STAGES>), dim3(Hkv, tiles, B), dim3(256), 0, stream,
@@ -1279,9 +1284,10 @@ extern "C" int q3_paged_attention(const void* q, int q_stride, void* out, const 
     float* ws_ml = workspace ? workspace + (size_t)B * Hkv * splits * 16 * D : nullptr;
     if (D == 64)
       return launch_fast<64>(q, q_stride, out, k_cache, v_cache, num_pages, block_table, bt_stride, cu_q, kv_lens,
-                             B, Hq, Hkv, page, scale, window, max_q_len, min_q_len, splits, ws_acc, ws_ml, stream);
+                             B, T_, Hq, Hkv, page, scale, window, max_q_len, min_q_len, splits, ws_acc, ws_ml,
+                             stream);
     return launch_fast<128>(q, q_stride, out, k_cache, v_cache, num_pages, block_table, bt_stride, cu_q, kv_lens, B,
-                            Hq, Hkv, page, scale, window, max_q_len, min_q_len, splits, ws_acc, ws_ml, stream);
+                            T_, Hq, Hkv, page, scale, window, max_q_len, min_q_len, splits, ws_acc, ws_ml, stream);
   }
   Q3_DISPATCH_DTYPE(dtype, TT, return launch_general<TT>(q, q_stride, out, k_cache, v_cache, num_pages,
                                                         block_table, bt_stride, cu_q, kv_lens, B, Hq, Hkv,

@@ -335,6 +335,7 @@ static int launch_skinny(const void* x, const void* w, void* out, int M, int N, 
 
 // Whether the weight-streaming kernel takes this product.
 extern "C" int q3_linear_is_skinny(int M, int N, int K, int in_dtype) {
+  (void)N;  // any number of weight rows
   return in_dtype == Q3_BF16 && M >= 1 && M <= 16 && K % 8 == 0 && K >= 8;
 }
 

@@ -62,7 +62,13 @@ struct Device {
   void* evict = nullptr;
   hipEvent_t begin = nullptr, end = nullptr;
   std::map<std::tuple<int, int, int, int>, Plan> plans;
+  // what was chosen for a size, by its rows rounded up to a multiple of 32: sizes beyond 64
+  // rows that differ only within such a step take the choice of the first one that was timed
+  // (a serving loop meets dozens of them, a prompt's portion plus however many requests decode)
+  std::map<std::tuple<int, int, int, int>, Plan> chosen_near;
 };
+
+int rows_class(int M) { return M <= 64 ? M : (M + 31) / 32 * 32; }
 
 std::mutex g_lock;
 std::map<int, Device> g_devices;
@@ -124,8 +130,7 @@ float time_candidate(Device& d, const Plan& p, const hipblasLtMatmulAlgo_t& algo
   return best;
 }
 
-int choose(Device& d, Plan& p, int M, int N, int K, const void* x, const void* w, void* out, hipStream_t stream,
-           bool capturing) {
+int choose(Device& d, Plan& p, const void* x, const void* w, void* out, hipStream_t stream, bool capturing) {
   hipblasLtMatmulPreference_t pref = nullptr;
   LT_TRY(hipblasLtMatmulPreferenceCreate(&pref));
   size_t bytes = WORKSPACE_BYTES;
@@ -226,11 +231,34 @@ extern "C" int q3_matmul(const void* x, const void* w, void* out, int M, int N, 
       return status;
     }
   }
+  const auto near_key = std::make_tuple(rows_class(M), N, K, out_dtype);
+  if (!p.tuned) {
+    auto near = d.chosen_near.find(near_key);
+    if (near != d.chosen_near.end()) {   // a neighbour's choice, if the library takes it for this size
+      if (run(d, p, near->second.algo, x, w, out, stream) == HIPBLAS_STATUS_SUCCESS) {
+        p.algo = near->second.algo;
+        p.candidates = near->second.candidates;
+        p.chosen = near->second.chosen;
+        p.first_us = near->second.first_us;
+        p.best_us = near->second.best_us;
+        p.tuned = true;
+        return 0;
+      }
+    }
+  }
   if (!p.candidates || (!p.tuned && !capturing)) {
-    const int status = choose(d, p, M, N, K, x, w, out, stream, capturing);
+    const int status = choose(d, p, x, w, out, stream, capturing);
     if (status) {
       forget(p);
       return status;
+    }
+    if (p.tuned) {
+      Plan& kept = d.chosen_near[near_key];   // the choice only: the descriptors stay with their size
+      kept.algo = p.algo;
+      kept.candidates = p.candidates;
+      kept.chosen = p.chosen;
+      kept.first_us = p.first_us;
+      kept.best_us = p.best_us;
     }
   }
   LT_TRY(run(d, p, p.algo, x, w, out, stream));

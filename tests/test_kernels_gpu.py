@@ -404,6 +404,11 @@ def test_linear_many_rows_is_the_library_kernel_that_was_fastest(M, N, K):
     other = x.clone()
     other[1:] = _rand((M - 1, K), torch.bfloat16, 43)
     assert torch.equal(ops.linear(other, w)[0], got16[0])
+    if M > 64 and K % 8 == 0:
+        # a few rows fewer (the same multiple of 32 rounded up): the same kernel, not timed again
+        fewer = ops.linear(x[:M - 7].contiguous(), w, out_dtype=torch.float32)
+        torch.testing.assert_close(fewer.double(), want[:M - 7], rtol=2e-3, atol=2e-3)
+        assert ops.matmul_plan(M - 7, N, K, torch.float32)[:2] == ops.matmul_plan(M, N, K, torch.float32)[:2]
 
 
 def test_linear_many_rows_first_met_in_a_graph():

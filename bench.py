@@ -85,7 +85,8 @@ def continuous(args, config, model, shape_name, gen, sync):
         seconds = time.perf_counter() - t0
     tokens_in, tokens_out = sum(p for p, _ in sizes), sum(g for _, g in sizes)
     print(json.dumps({
-        "metric": "continuous batching, tokens/s in and out, %s bf16" % shape_name,
+        "metric": "continuous batching, tokens/s in and out, %s %s"
+                  % (shape_name, "bf16" if args.dtype == "bfloat16" else "fp32"),
         "value": round((tokens_in + tokens_out) / seconds, 1), "unit": "tokens/s", "n_gpus": 1,
         "higher_is_better": True, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
         "seconds": round(seconds, 3), "steps": steps, "generated_tokens_per_s": round(tokens_out / seconds, 1),
@@ -207,7 +208,8 @@ def main():
             points["decode_b%d" % b] = round(p_tps, 1)
 
     line = {
-        "metric": "decode tok/s at batch 1/8/64 + prefill tok/s at 2048 tokens, %s bf16" % shape_name,
+        "metric": "decode tok/s at batch 1/8/64 + prefill tok/s at 2048 tokens, %s %s"
+                  % (shape_name, "bf16" if args.dtype == "bfloat16" else "fp32"),
         "value": round(tps, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",

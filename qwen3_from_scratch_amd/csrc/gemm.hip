@@ -333,6 +333,60 @@ static int launch_skinny(const void* x, const void* w, void* out, int M, int N, 
   return q3_launch_status();
 }
 
+// ---------------------------------------------------------------------------
+// float32 with few rows (decoding): the tiled kernel above would give a product of 8 x 4096
+// 64 blocks; here the weights are streamed once by as many wavefronts as there are groups of
+// four weight rows. A wavefront's lanes stride over k four elements at a time (a kilobyte of
+// each weight row per turn, and of each row of x, which all wavefronts of a CU read at about
+// the same time), every lane keeps 4 x MB sums, and the lanes' sums meet at the end in a fixed
+// order: an output's value depends on K alone, not on the rows beside it.
+// ---------------------------------------------------------------------------
+#define F32_FEW_ROWS 4  // weight rows per wavefront
+
+template <int MB>
+__global__ __launch_bounds__(256) void gemm_f32_few_rows_kernel(const float* __restrict__ x,
+                                                                const float* __restrict__ w,
+                                                                float* __restrict__ out, int M, int N, int K) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n0 = (blockIdx.x * 4 + wave) * F32_FEW_ROWS;
+  if (n0 >= N) return;
+  float acc[F32_FEW_ROWS][MB];
+#pragma unroll
+  for (int j = 0; j < F32_FEW_ROWS; ++j)
+#pragma unroll
+    for (int m = 0; m < MB; ++m) acc[j][m] = 0.f;
+  const float* rows[F32_FEW_ROWS];
+#pragma unroll
+  for (int j = 0; j < F32_FEW_ROWS; ++j) rows[j] = w + (size_t)min(n0 + j, N - 1) * K;  // a row past the end: read, not written
+  for (int k = 4 * lane; k < K; k += 256) {
+    float4 wv[F32_FEW_ROWS];
+#pragma unroll
+    for (int j = 0; j < F32_FEW_ROWS; ++j) wv[j] = *reinterpret_cast<const float4*>(rows[j] + k);
+#pragma unroll
+    for (int m = 0; m < MB; ++m) {
+      if (m < M) {
+        const float4 xv = *reinterpret_cast<const float4*>(x + (size_t)m * K + k);
+#pragma unroll
+        for (int j = 0; j < F32_FEW_ROWS; ++j) {
+          float a = acc[j][m];
+          a = fmaf(xv.x, wv[j].x, a);
+          a = fmaf(xv.y, wv[j].y, a);
+          a = fmaf(xv.z, wv[j].z, a);
+          a = fmaf(xv.w, wv[j].w, a);
+          acc[j][m] = a;
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < F32_FEW_ROWS; ++j)
+#pragma unroll
+    for (int m = 0; m < MB; ++m) {
+      const float total = wave_sum(acc[j][m]);
+      if (lane == 0 && m < M && n0 + j < N) out[(size_t)m * N + n0 + j] = total;
+    }
+}
+
 // Whether the weight-streaming kernel takes this product.
 extern "C" int q3_linear_is_skinny(int M, int N, int K, int in_dtype) {
   (void)N;  // any number of weight rows
@@ -344,6 +398,19 @@ extern "C" int q3_linear(const void* x, const void* weight, void* out, int M, in
   if (M <= 0 || N <= 0 || K <= 0) return Q3_ERR_BAD_ARGUMENT;
   if (in_dtype == Q3_F32) {
     if (out_dtype != Q3_F32) return Q3_ERR_BAD_ARGUMENT;
+    if (M <= 16 && K % 4 == 0) {
+      const dim3 few((N + 4 * F32_FEW_ROWS - 1) / (4 * F32_FEW_ROWS));
+      if (M <= 4)
+        hipLaunchKernelGGL(gemm_f32_few_rows_kernel<4>, few, dim3(256), 0, stream, (const float*)x,
+                           (const float*)weight, (float*)out, M, N, K);
+      else if (M <= 8)
+        hipLaunchKernelGGL(gemm_f32_few_rows_kernel<8>, few, dim3(256), 0, stream, (const float*)x,
+                           (const float*)weight, (float*)out, M, N, K);
+      else
+        hipLaunchKernelGGL(gemm_f32_few_rows_kernel<16>, few, dim3(256), 0, stream, (const float*)x,
+                           (const float*)weight, (float*)out, M, N, K);
+      return q3_launch_status();
+    }
     const dim3 grid((N + F32_BN - 1) / F32_BN, (M + F32_BM - 1) / F32_BM);
     if (grid.y > 65535) return Q3_ERR_UNSUPPORTED;
     hipLaunchKernelGGL(gemm_f32_kernel, grid, dim3(256), 0, stream, (const float*)x, (const float*)weight,

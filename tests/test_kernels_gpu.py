@@ -363,6 +363,21 @@ def test_linear(dtype, M, N, K):
     torch.testing.assert_close(got32.double(), want, rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (5, 6144, 4096), (8, 331, 200), (16, 1000, 2056), (3, 7, 12),
+                                   (12, 50000, 256), (9, 4096, 12288), (4, 50, 515)])
+def test_linear_float32_few_rows(M, N, K):
+    """The float32 path's products when decoding: weights streamed once, a row's result the
+    same whatever rows stand beside it."""
+    ops = _ops()
+    x = _rand((M, K), torch.float32, 51)
+    w = _rand((N, K), torch.float32, 52, scale=0.05)
+    got = ops.linear(x, w)
+    torch.testing.assert_close(got.double(), x.double() @ w.double().T, rtol=1e-5, atol=1e-5)
+    if K % 4 == 0:
+        alone = ops.linear(x[M - 1:].contiguous(), w)
+        assert torch.equal(alone[0], got[M - 1])
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 6144, 4096), (8, 4096, 4096), (5, 24576, 512), (16, 4096, 12288),
                                    (17, 1000, 2056), (32, 50000, 256), (48, 777, 4104), (64, 4096, 4096)])
 def test_linear_few_rows_streams_weights(M, N, K):

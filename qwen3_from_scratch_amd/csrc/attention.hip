@@ -873,7 +873,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, int num_pages, const int* __restrict__ block_table, int bt_stride,
     const int* __restrict__ cu_q, const int* __restrict__ kv_lens, int Hq, int Hkv, int page, float scale_log2,
-    int window, int tokens_per_block) {
+    int window, int tokens_per_block, int key_splits, float* __restrict__ part_acc, float* __restrict__ part_ml) {
   typedef PrefillSmem<D, TILE> SM;
   constexpr int KB4 = TILE / 16;  // 16-key blocks per tile
   __shared__ __attribute__((aligned(16))) unsigned char smem[STAGES * SM::STAGE];
@@ -887,13 +887,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int q_len = cu_q[b + 1] - q0;
   if (q_len * G <= 16) return;  // the other kernel's sequence
   const int n_tiles = (q_len + tokens_per_block - 1) / tokens_per_block;
-  if ((int)blockIdx.y >= n_tiles) return;
+  // with `key_splits` > 1 a row tile's keys are shared out over that many blocks, whose
+  // unnormalised results attn_prefill_merge_kernel joins
+  const int split = (int)blockIdx.y % key_splits, tile_index = (int)blockIdx.y / key_splits;
+  if (tile_index >= n_tiles) return;
   // the first half of a head's blocks takes the row tiles from the sequence's end downwards (the
   // long ones start first), the second half from its start upwards: block i and block
   // i + n / 2, a long and a short one, come to share a CU (measured against plain ascending and
   // descending orders and the mirrored one: 87 us against 95, 89 and 88)
   const int half_tiles = (n_tiles + 1) / 2;
-  const int tile = (int)blockIdx.y < half_tiles ? n_tiles - 1 - (int)blockIdx.y : (int)blockIdx.y - half_tiles;
+  const int tile = tile_index < half_tiles ? n_tiles - 1 - tile_index : tile_index - half_tiles;
   const int kv_len = kv_lens[b];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -942,10 +945,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int blk_last_tok = min(q_len, blk_first_tok + tokens_per_block) - 1;
   int tile_lo = 0;
   if (window > 0) tile_lo = max(0, first_pos + blk_first_tok - window + 1) / TILE;
-  const int tile_hi = (first_pos + blk_last_tok) / TILE + 1;
+  int tile_hi = (first_pos + blk_last_tok) / TILE + 1;
   // and this wavefront's own (a wavefront whose rows do not exist has none)
   int my_lo = tile_lo, my_hi = pos_max >= 0 ? pos_max / TILE + 1 : 0;
   if (window > 0 && pos_max >= 0) my_lo = max(0, pos_min - window + 1) / TILE;
+  if (key_splits > 1) {  // this block's share of the range (it may be empty)
+    const int share = (tile_hi - tile_lo + key_splits - 1) / key_splits;
+    tile_lo = min(tile_hi, tile_lo + split * share);
+    tile_hi = min(tile_hi, tile_lo + share);
+    my_lo = max(my_lo, tile_lo);
+    my_hi = min(my_hi, tile_hi);
+  }
   const int* bt_row = block_table + (size_t)b * bt_stride;
 
   // The copy of a tile from the caches into a stage. Place s (a 16-byte piece) of the keys'
@@ -1188,6 +1198,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
     if (row_pos[qb] < 0) continue;
+    if (key_splits > 1) {
+      const size_t slot = ((size_t)row_tok[qb] * Hq + row_head[qb]) * key_splits + split;
+      float* o = part_acc + slot * D + 4 * grp;
+#pragma unroll
+      for (int nb = 0; nb < D / 16; ++nb)
+        *reinterpret_cast<float4*>(o + 16 * nb) =
+            make_float4(acc[qb][nb][0], acc[qb][nb][1], acc[qb][nb][2], acc[qb][nb][3]);
+      if (grp == 0) *reinterpret_cast<float2*>(part_ml + slot * 2) = make_float2(m_run[qb], l);
+      continue;
+    }
     const float inv = 1.f / l;
     bf16_t* o = out + (size_t)row_tok[qb] * Hq * D + (size_t)row_head[qb] * D + 4 * grp;
 #pragma unroll
@@ -1203,11 +1223,76 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   }
 }
 
+// Joins the key splits of attn_prefill_kernel: grid (max_q_len, B), 256 threads; a block takes
+// one token of a sequence, a thread four neighbouring output elements of one (token, head)
+// row at a time. Sequences of few rows are the decoding kernel's.
+template <int D>
+__global__ __launch_bounds__(256) void attn_prefill_merge_kernel(bf16_t* __restrict__ out,
+                                                                 const int* __restrict__ cu_q, int Hq, int Hkv,
+                                                                 int key_splits, const float* __restrict__ part_acc,
+                                                                 const float* __restrict__ part_ml) {
+  const int b = blockIdx.y;
+  const int q0 = cu_q[b], q_len = cu_q[b + 1] - q0;
+  if (q_len * (Hq / Hkv) <= 16) return;
+  constexpr int PER_ROW = D / 4;  // threads a row takes
+  const int first = blockIdx.x;
+  if (first >= q_len) return;
+  const int rows = Hq;
+  for (int i = threadIdx.x; i < rows * PER_ROW; i += 256) {
+    const int row = i / PER_ROW, d = 4 * (i % PER_ROW);
+    const size_t slot = ((size_t)(q0 + first) * Hq + row) * key_splits;
+    float m_all = -INFINITY;
+    for (int s = 0; s < key_splits; ++s) m_all = fmaxf(m_all, part_ml[(slot + s) * 2]);
+    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+    float l_all = 0.f;
+    for (int s = 0; s < key_splits; ++s) {   // in the splits' order: a fixed order of additions
+      const float2 ml = *reinterpret_cast<const float2*>(part_ml + (slot + s) * 2);
+      if (ml.x == -INFINITY) continue;       // a split with no key for this row
+      const float w = fast_exp2(ml.x - m_all);
+      const float4 a = *reinterpret_cast<const float4*>(part_acc + (slot + s) * D + d);
+      o.x += a.x * w; o.y += a.y * w; o.z += a.z * w; o.w += a.w * w;
+      l_all += ml.y * w;
+    }
+    const float inv = 1.f / l_all;
+    union {
+      uint2 u;
+      bf16_t e[4];
+    } pk;
+    pk.e[0] = float_to_bf16(o.x * inv); pk.e[1] = float_to_bf16(o.y * inv);
+    pk.e[2] = float_to_bf16(o.z * inv); pk.e[3] = float_to_bf16(o.w * inv);
+    *reinterpret_cast<uint2*>(out + ((size_t)(q0 + first) * Hq + row) * D + d) = pk.u;
+  }
+}
+
+// How the rows and keys of a step's long sequences go over blocks. A block owns 128 rows
+// (tokens x heads of a group) and all their keys; with so few rows that the blocks do not fill
+// the chip twice (a portion of 512 tokens of one prompt: 128 blocks, each a chain of as many
+// tiles as the prefix is long), first the keys are split over up to four blocks, from 2,048
+// keys on and as long as a split keeps eight tiles (512 tokens over 3,584 keys: 127 us whole,
+// 97 in two, 88 in four; 256 over 7,936: 224, 141, 97; over 512 keys splitting loses), then a
+// block's rows are halved, down to one wavefront's 32 (its other wavefronts then only help
+// to copy the tiles).
+static int prompt_key_splits(int total_tokens, int G, int Hkv, int max_kv_len) {
+  const int tpb = 128 / G;
+  int ks = 1;
+  const int key_tiles = (max_kv_len + PF_TILE - 1) / PF_TILE;
+  while (Hkv * ((total_tokens + tpb - 1) / tpb) * ks < 512 && ks < 4 && key_tiles >= 32 && key_tiles / (2 * ks) >= 8)
+    ks *= 2;
+  return ks;
+}
+
+static int prompt_tokens_per_block(int total_tokens, int G, int Hkv, int key_splits) {
+  int tpb = 128 / G;
+  while (Hkv * ((total_tokens + tpb - 1) / tpb) * key_splits < 256 && (tpb / 2) * G >= 32) tpb /= 2;
+  return tpb;
+}
+
 template <int D>
 static int launch_fast(const void* q, int q_stride, void* out, const void* k_cache, const void* v_cache,
                        int num_pages, const int* block_table, int bt_stride, const int* cu_q, const int* kv_lens,
                        int B, int total_tokens, int Hq, int Hkv, int page, float scale, int window, int max_q_len,
-                       int min_q_len, int splits, float* ws_acc, float* ws_ml, hipStream_t stream) {
+                       int min_q_len, int splits, float* ws_acc, float* ws_ml, int key_splits, float* prompt_ws,
+                       hipStream_t stream) {
   const int G = Hq / Hkv;
   const float scale_log2 = scale * 1.4426950408889634f;
   if (min_q_len * G <= 16) {
@@ -1220,18 +1305,18 @@ static int launch_fast(const void* q, int q_stride, void* out, const void* k_cac
                          Hkv, splits, ws_acc, ws_ml);
   }
   if (max_q_len * G > 16) {
-    // A block owns 128 rows; with so few rows that not every CU gets a block (a portion of 512
-    // tokens of one prompt: 128 blocks), a block's rows are halved until they do, down to one
-    // wavefront's 32 (its other wavefronts then only help to copy the tiles).
-    int tokens_per_block = 128 / G;
-    while (Hkv * ((total_tokens + tokens_per_block - 1) / tokens_per_block) < 256 && (tokens_per_block / 2) * G >= 32)
-      tokens_per_block /= 2;
+    const int tokens_per_block = prompt_tokens_per_block(total_tokens, G, Hkv, key_splits);
     const int tiles = (max_q_len + tokens_per_block - 1) / tokens_per_block;
-    if (tiles > 65535) return Q3_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL((attn_prefill_kernel<D, PF_TILE, PF_STAGES>), dim3(Hkv, tiles, B), dim3(256), 0, stream,
-                       (const bf16_t*)q, q_stride,
-                       (bf16_t*)out, (const bf16_t*)k_cache, (const bf16_t*)v_cache, num_pages, block_table,
-                       bt_stride, cu_q, kv_lens, Hq, Hkv, page, scale_log2, window, tokens_per_block);
+    if (tiles * key_splits > 65535) return Q3_ERR_UNSUPPORTED;
+    float* part_acc = prompt_ws;
+    float* part_ml = prompt_ws ? prompt_ws + (size_t)total_tokens * Hq * key_splits * D : nullptr;
+    hipLaunchKernelGGL((attn_prefill_kernel<D, PF_TILE, PF_STAGES>), dim3(Hkv, tiles * key_splits, B), dim3(256), 0,
+                       stream, (const bf16_t*)q, q_stride, (bf16_t*)out, (const bf16_t*)k_cache,
+                       (const bf16_t*)v_cache, num_pages, block_table, bt_stride, cu_q, kv_lens, Hq, Hkv, page,
+                       scale_log2, window, tokens_per_block, key_splits, part_acc, part_ml);
+    if (key_splits > 1)
+      hipLaunchKernelGGL(attn_prefill_merge_kernel<D>, dim3(max_q_len, B), dim3(256), 0, stream,
+                         (bf16_t*)out, cu_q, Hq, Hkv, key_splits, part_acc, part_ml);
   }
   return q3_launch_status();
 }
@@ -1266,28 +1351,41 @@ extern "C" long q3_paged_attention_workspace(int B, int Hkv, int D, int splits) 
   return splits > 1 ? (long)B * Hkv * splits * 16 * (D + 2) : 0;
 }
 
+// Over how many blocks the keys of a step's long sequences are best split (see above): `T` the
+// step's rows, `max_kv_len` the longest of those sequences. With more than one, the workspace
+// holds T * Hq * splits * (D + 2) floats: unnormalised outputs, then (max, sum) pairs.
+extern "C" int q3_paged_attention_prompt_splits(int T, int Hq, int Hkv, int max_kv_len) {
+  if (T <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv) return 1;
+  return prompt_key_splits(T, Hq / Hkv, Hkv, max_kv_len);
+}
+
+// `splits`, `workspace`: for the sequences of few rows (q3_paged_attention_workspace);
+// `prompt_splits` (1, 2 or 4), `prompt_workspace`: for those of many.
 extern "C" int q3_paged_attention(const void* q, int q_stride, void* out, const void* k_cache,
                                   const void* v_cache, int num_pages, const int* block_table,
                                   int bt_stride, const int* cu_q, const int* kv_lens, int B, int T_, int Hq,
                                   int Hkv, int D, int page, float scale, int window, int max_q_len,
                                   int min_q_len, int max_kv_len, int dtype, int splits, float* workspace,
-                                  hipStream_t stream) {
+                                  int prompt_splits, float* prompt_workspace, hipStream_t stream) {
   if (B <= 0 || T_ <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || page <= 0 || max_q_len <= 0 || min_q_len <= 0 ||
       min_q_len > max_q_len)
     return Q3_ERR_BAD_ARGUMENT;
   if (D % 16 || D < 16 || D > 256) return Q3_ERR_UNSUPPORTED;
   if (B > 65535 || Hq > 65535) return Q3_ERR_UNSUPPORTED;
-  (void)max_kv_len;
   if (q3_paged_attention_fast_path(Hq, Hkv, D, page, dtype) && (q_stride % 8) == 0) {
     if (splits < 1 || splits > MAX_SPLITS || (splits > 1 && workspace == nullptr)) return Q3_ERR_BAD_ARGUMENT;
+    if (prompt_splits < 1 || prompt_splits > 4 || (prompt_splits > 1 && prompt_workspace == nullptr))
+      return Q3_ERR_BAD_ARGUMENT;
+    (void)max_kv_len;
     float* ws_acc = workspace;
     float* ws_ml = workspace ? workspace + (size_t)B * Hkv * splits * 16 * D : nullptr;
     if (D == 64)
       return launch_fast<64>(q, q_stride, out, k_cache, v_cache, num_pages, block_table, bt_stride, cu_q, kv_lens,
                              B, T_, Hq, Hkv, page, scale, window, max_q_len, min_q_len, splits, ws_acc, ws_ml,
-                             stream);
+                             prompt_splits, prompt_workspace, stream);
     return launch_fast<128>(q, q_stride, out, k_cache, v_cache, num_pages, block_table, bt_stride, cu_q, kv_lens, B,
-                            T_, Hq, Hkv, page, scale, window, max_q_len, min_q_len, splits, ws_acc, ws_ml, stream);
+                            T_, Hq, Hkv, page, scale, window, max_q_len, min_q_len, splits, ws_acc, ws_ml,
+                            prompt_splits, prompt_workspace, stream);
   }
   Q3_DISPATCH_DTYPE(dtype, TT, return launch_general<TT>(q, q_stride, out, k_cache, v_cache, num_pages,
                                                         block_table, bt_stride, cu_q, kv_lens, B, Hq, Hkv,

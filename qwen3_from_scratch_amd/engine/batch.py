@@ -37,6 +37,7 @@ class StepBatch:
     max_q_len: int
     min_q_len: int
     max_kv_len: int
+    max_kv_len_portions: int       # the same among the entries that bring more than one token
     q_lens: list                   # host copies
     kv_lens_host: list
 
@@ -125,6 +126,7 @@ def pack_step(entries, lengths, slots, tables_per_group, device, min_table_width
         cu_seqlens_q=dev[s_cu], kv_lens=dev[s_kv], state_slots=dev[s_slot], logits_rows=dev[s_rows],
         max_q_len=max(q_lens) if q_lens else 0, min_q_len=min(q_lens) if q_lens else 0,
         max_kv_len=max(kv) if kv else 0,
+        max_kv_len_portions=max([n for n, q in zip(kv, q_lens) if q > 1] or [0]),
         q_lens=q_lens, kv_lens_host=kv,
     )
     block_tables = [dev[sl].view(B, w) for sl, w in s_tables]

@@ -229,7 +229,7 @@ def qk_norm_rope_store(qkv, num_q_heads, num_kv_heads, head_dim, positions, seq_
 
 
 def paged_attention(q, num_q_heads, k_cache, v_cache, block_table, cu_seqlens_q, kv_lens,
-                    max_q_len, max_kv_len, scale, window=0, out=None, min_q_len=1):
+                    max_q_len, max_kv_len, scale, window=0, out=None, min_q_len=1, max_kv_len_of_many=None):
     """Causal softmax attention of packed query rows over paged keys and values.
 
     q is (T, Hq, D) seen through a row stride (a view of the qkv buffer is
@@ -241,6 +241,9 @@ def paged_attention(q, num_q_heads, k_cache, v_cache, block_table, cu_seqlens_q,
     key head h // (Hq / Hkv). Softmax statistics and accumulation are float32.
     `max_q_len` and `min_q_len` bound the sequences' row counts (they choose
     between the kernels for few and for many rows; loose bounds cost time only).
+    `max_kv_len_of_many`: the most keys of a sequence that brings many rows, if
+    the caller knows it (it decides whether such sequences' keys are shared out
+    over several blocks; `max_kv_len` stands in).
 
     bfloat16 with head size 64 or 128 and a page size that is a power of two from 16
     runs on the matrix cores; everything else (float32, other head sizes in
@@ -270,18 +273,27 @@ def paged_attention(q, num_q_heads, k_cache, v_cache, block_table, cu_seqlens_q,
     _need(out.shape == (T, Hq * D) and out.dtype == q.dtype, "out must be (T, Hq D)")
     if T and B:
         lib = library("attention")
-        splits, workspace = 1, None
-        if lib.q3_paged_attention_fast_path(Hq, Hkv, D, page, _DT[q.dtype]) and min_q_len * (Hq // Hkv) <= 16:
-            splits = _splits(B, Hkv, max_kv_len)       # few rows per sequence: the keys go over several blocks
-            if splits > 1:
-                lib.q3_paged_attention_workspace.restype = ctypes.c_long
-                n = lib.q3_paged_attention_workspace(B, Hkv, D, splits)
-                workspace = torch.empty((n,), dtype=torch.float32, device=q.device)
+        splits, workspace, prompt_splits, prompt_workspace = 1, None, 1, None
+        if lib.q3_paged_attention_fast_path(Hq, Hkv, D, page, _DT[q.dtype]):
+            if min_q_len * (Hq // Hkv) <= 16:
+                splits = _splits(B, Hkv, max_kv_len)   # few rows per sequence: the keys go over several blocks
+                if splits > 1:
+                    lib.q3_paged_attention_workspace.restype = ctypes.c_long
+                    n = lib.q3_paged_attention_workspace(B, Hkv, D, splits)
+                    workspace = torch.empty((n,), dtype=torch.float32, device=q.device)
+            if max_q_len * (Hq // Hkv) > 16:           # few long sequences over many keys: likewise
+                longest = max_kv_len if max_kv_len_of_many is None else max_kv_len_of_many
+                prompt_splits = lib.q3_paged_attention_prompt_splits(T, Hq, Hkv, int(longest))
+                if prompt_splits > 1:
+                    prompt_workspace = torch.empty((T * Hq * prompt_splits * (D + 2),), dtype=torch.float32,
+                                                   device=q.device)
         _check(lib.q3_paged_attention(
             _ptr(q), q.stride(0), _ptr(out), _ptr(k_cache), _ptr(v_cache), k_cache.shape[0],
             _ptr(block_table), block_table.shape[1], _ptr(cu_seqlens_q), _ptr(kv_lens),
             B, T, Hq, Hkv, D, page, ctypes.c_float(scale), int(window), int(max_q_len), int(min_q_len),
-            int(max_kv_len), _DT[q.dtype], splits, _ptr(workspace), _stream()), "paged_attention")
+            int(max_kv_len), _DT[q.dtype], splits, _ptr(workspace), prompt_splits, _ptr(prompt_workspace),
+            _stream()),
+            "paged_attention")
     return out
 
 

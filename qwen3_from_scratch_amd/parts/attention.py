@@ -106,6 +106,6 @@ class PagedAttention(Part):
         o = ops.paged_attention(
             q, Hq, cache.keys, cache.values, cache.block_table, batch.cu_seqlens_q, batch.kv_lens,
             batch.max_q_len, batch.max_kv_len, self.scale, window=self.window,
-            min_q_len=batch.min_q_len,
+            min_q_len=batch.min_q_len, max_kv_len_of_many=getattr(batch, "max_kv_len_portions", None),
         )
         return self.out.forward(o) if sink is None else self.out.forward_into(o, sink)

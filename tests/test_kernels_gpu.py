@@ -258,18 +258,25 @@ def test_decode_attention_is_its_two_halves(Hq, Hkv, D, page, w_dtype, window, r
     torch.testing.assert_close(got.float().view(B, Hq, D), ref.view(B, Hq, D), rtol=2e-2, atol=2e-2)
 
 
-def test_paged_attention_portions_over_long_prefixes():
-    """Portions of prompts with hundreds of cached keys before them, beside single tokens."""
+@pytest.mark.parametrize("q_lens,kv_lens", [([512, 1, 100, 3, 33], [512, 900, 1100, 64, 2000]),
+                                            ([700, 2], [3000, 50]), ([300], [9000]), ([40, 40, 40], [2100, 40, 700])])
+def test_paged_attention_portions_over_long_prefixes(q_lens, kv_lens):
+    """Portions of prompts with hundreds or thousands of cached keys before them, beside single
+    tokens: few blocks of rows, whose keys are shared out over four blocks, over two, or not at all."""
     ops = _ops()
     Hq, Hkv, D, page = 32, 8, 128, 16
-    q_lens = [512, 1, 100, 3, 33]
-    kv_lens = [512, 900, 1100, 64, 2000]
-    q, kc, vc, bt, cu, kvl = _paged_case(torch.bfloat16, 5, Hq, Hkv, D, page, q_lens, kv_lens, 31)
+    q, kc, vc, bt, cu, kvl = _paged_case(torch.bfloat16, len(q_lens), Hq, Hkv, D, page, q_lens, kv_lens, 31)
     scale = D ** -0.5
-    got = ops.paged_attention(q, Hq, kc, vc, bt, cu, kvl, max(q_lens), max(kv_lens), scale, min_q_len=1)
+    got = ops.paged_attention(q, Hq, kc, vc, bt, cu, kvl, max(q_lens), max(kv_lens), scale, min_q_len=min(q_lens))
     want = torch_ops.paged_attention(q.float(), Hq, kc.float(), vc.float(), bt, cu, kvl, max(q_lens),
                                      max(kv_lens), scale)
     torch.testing.assert_close(got.float(), want, rtol=2e-2, atol=2e-2)
+    for window in (0, 700):
+        got = ops.paged_attention(q, Hq, kc, vc, bt, cu, kvl, max(q_lens), max(kv_lens), scale, window=window,
+                                  min_q_len=min(q_lens))
+        want = torch_ops.paged_attention(q.float(), Hq, kc.float(), vc.float(), bt, cu, kvl, max(q_lens),
+                                         max(kv_lens), scale, window=window)
+        torch.testing.assert_close(got.float(), want, rtol=2e-2, atol=2e-2)
 
 
 def test_paged_attention_contexts_of_tens_of_thousands():

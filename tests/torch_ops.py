@@ -90,7 +90,7 @@ def qk_norm_rope_store(qkv, num_q_heads, num_kv_heads, head_dim, positions, seq_
 
 
 def paged_attention(q, num_q_heads, k_cache, v_cache, block_table, cu_seqlens_q, kv_lens,
-                    max_q_len, max_kv_len, scale, window=0, out=None, min_q_len=1):
+                    max_q_len, max_kv_len, scale, window=0, out=None, min_q_len=1, max_kv_len_of_many=None):
     T, Hq, D = q.shape
     Hkv, page = k_cache.shape[1], k_cache.shape[2]
     G = Hq // Hkv

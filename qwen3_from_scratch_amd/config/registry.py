@@ -6,10 +6,17 @@ The reference keeps a single component registry keyed by slot and name
 class; here the model class is looked up by config.json's `architectures[0]`.
 """
 
+import importlib
 import json
 import os
 
 from .model_config import ConfigError
+
+# Modules named here (comma-separated, importable) are imported the first time an
+# architecture or a part is looked up and not found: they register architectures and
+# parts that live outside this package, for the programs that take only a model folder.
+PLUGINS_VARIABLE = "QWEN3_FROM_SCRATCH_AMD_PLUGINS"
+_plugins_imported = False
 
 _ARCHITECTURES = {}
 _PARTS = {}
@@ -27,7 +34,24 @@ def architectures():
     return sorted(_ARCHITECTURES)
 
 
+def import_plugins():
+    """Import the modules that $QWEN3_FROM_SCRATCH_AMD_PLUGINS names, once."""
+    global _plugins_imported
+    if _plugins_imported:
+        return
+    _plugins_imported = True
+    for module in os.environ.get(PLUGINS_VARIABLE, "").split(","):
+        module = module.strip()
+        if module:
+            try:
+                importlib.import_module(module)
+            except ImportError as exc:
+                raise ConfigError("$%s names %r, which cannot be imported: %s" % (PLUGINS_VARIABLE, module, exc)) from exc
+
+
 def lookup_architecture(name):
+    if name not in _ARCHITECTURES:
+        import_plugins()
     if name not in _ARCHITECTURES:
         raise ConfigError(
             "architecture %r is not registered; known: %s" % (name, ", ".join(architectures()))
@@ -65,6 +89,8 @@ def register_part(kind, name):
 
 
 def lookup_part(kind, name):
+    if name not in _PARTS.get(kind, {}):
+        import_plugins()
     try:
         return _PARTS[kind][name]
     except KeyError:

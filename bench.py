@@ -219,7 +219,8 @@ def main():
             "layers": config.num_hidden_layers, "layers_full": full_layers, "hidden_size": config.hidden_size,
             "num_attention_heads": config.num_attention_heads, "num_key_value_heads": config.num_key_value_heads,
             "head_dim": config.head_dim, "intermediate_size": config.intermediate_size,
-            "vocab_size": config.vocab_size, "kv_block_size": BLOCK, "sampling": "greedy",
+            "vocab_size": config.vocab_size, "rope_theta": config.rope_theta, "rms_norm_eps": config.rms_norm_eps,
+            "tie_word_embeddings": config.tie_word_embeddings, "kv_block_size": BLOCK, "sampling": "greedy",
         },
         "prefill": prefill, "roofline": roofline, "points": points,
     }

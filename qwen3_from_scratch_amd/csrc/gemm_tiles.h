@@ -1,0 +1,245 @@
+// A matrix-core product for many rows, out[M, N] = x[M, K] . w[N, K]^T in bfloat16 with
+// float32 accumulation: the counterpart of the reference's own GEMM kernel
+// (src/qwen3_from_scratch/kernels/triton/gemm.py:26-274, 128 x 128 tiles, float32
+// accumulation), written for gfx950.
+//
+// A block of WM x WN wavefronts owns a BM x BN tile of the output and walks K in steps of
+// 64. Both operands have K contiguous, so a step's slices of x and of w are BM and BN rows of
+// 128 bytes. They travel from memory to shared memory by loads that write shared memory
+// directly (16 bytes a lane, a wavefront's 64 lanes fill one contiguous kilobyte, eight rows),
+// the slices of the next STAGES - 1 steps while the current one is multiplied. Within a row the
+// eight 16-byte pieces are placed by an XOR with bits 1..3 of the row number, so that the
+// sixteen lanes that read one piece of sixteen consecutive rows (an operand of
+// v_mfma_f32_16x16x32_bf16) touch every bank once. The loads are issued as assembly with their
+// own wait counts (see attn_prefill_kernel in attention.hip for why).
+//
+// The weight rows are the matrix instruction's first operand and the rows of x its second, so
+// a lane ends with four consecutive outputs of one row of x: pairs (gate, up) for the SwiGLU
+// epilogue, eight bytes of bfloat16 for the plain one.
+//
+// What bounds it (2,048 x 24,576 x 4,096, 256 x 256 tiles, eight wavefronts of 64 x 128): with
+// the copies taken out 233 us (1.77 PFLOP/s), with copies that always hit the cache 303, as it is
+// 323 (1.27), the vendor library's best kernel 279: a step's operand reads (192 KB) and the
+// copies' writes (64 KB) keep shared memory busy for as many cycles as the matrix instructions
+// take. Wavefront tiles of 128 x 128 would read a third less but leave one wavefront a SIMD and
+// no registers to read ahead with (the compiler's schedule of that shape: 364 us).
+//
+// K must be a multiple of 64. Rows of x beyond M and of w beyond N are read from the last
+// valid row and never written. Blocks are numbered so that the eight XCDs each take a
+// contiguous run of tiles, M fastest: the blocks that share a slice of w run on one XCD at
+// about the same time and the slice comes from memory once.
+
+#pragma once
+
+#include "common.h"
+
+namespace tiles {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+
+union Frag {
+  uint4 u;
+  bf16x8_t v;
+};
+
+enum { EPI_PLAIN = 0, EPI_SWIGLU = 1 };
+
+constexpr int BK = 64;          // k per step: two matrix instructions deep
+constexpr int ROW_BYTES = 128;  // a row of a slice
+
+template <int BM, int BN, int WM, int WN, int STAGES>
+struct Shape {
+  static constexpr int THREADS = 64 * WM * WN;
+  static constexpr int STAGE_BYTES = (BM + BN) * ROW_BYTES;
+  static constexpr int SMEM_BYTES = STAGES * STAGE_BYTES;
+  static constexpr int TURN_ROWS = THREADS / 8;               // rows of a slice that one turn of the block fills
+  static constexpr int X_TURNS = BM / TURN_ROWS, W_TURNS = BN / TURN_ROWS;  // loads a thread issues per step
+  static constexpr int LOADS = X_TURNS + W_TURNS;
+  static constexpr int MI = BM / WM / 16, NJ = BN / WN / 16;  // 16 x 16 blocks of a wavefront's tile
+  static_assert(BM % TURN_ROWS == 0 && BN % TURN_ROWS == 0 && (BM / WM) % 16 == 0 && (BN / WN) % 16 == 0, "shape");
+};
+
+// four outputs to bfloat16 (round to nearest even, as float_to_bf16: the hardware's conversion)
+__device__ inline uint2 pack_bf16x4(f32x4_t c) {
+  typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
+  union {
+    bf16x4_t v;
+    uint2 u;
+  } pk;
+  pk.v = __builtin_convertvector(c, bf16x4_t);
+  return pk.u;
+}
+
+template <typename OUT, int EPI, int BM, int BN, int WM, int WN, int STAGES>
+__global__ __launch_bounds__(64 * WM * WN) void gemm_tiles_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                         OUT* __restrict__ out, int M, int N, int K, int tiles_m,
+                                                         int tiles_total, int tiles_per_xcd) {
+  typedef Shape<BM, BN, WM, WN, STAGES> S;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  // block -> tile: XCD x (blocks x, x + 8, ...) takes tiles [x * per, (x + 1) * per)
+  const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+  const int tile = xcd * tiles_per_xcd + local;
+  if (local >= tiles_per_xcd || tile >= tiles_total) return;
+  const int m0 = (tile % tiles_m) * BM, n0 = (tile / tiles_m) * BN;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col = lane & 15, grp = lane >> 4;
+  const int wm = wave % WM, wn = wave / WM;
+
+  // the copies: in turn j this thread fills place THREADS j + tid of a slice (16 bytes each,
+  // row = place / 8), with the piece that the XOR puts there
+  const int piece = (tid & 7) ^ ((tid >> 4) & 7);
+  const bf16_t* x_src[S::X_TURNS];
+  const bf16_t* w_src[S::W_TURNS];
+#pragma unroll
+  for (int j = 0; j < S::X_TURNS; ++j)
+    x_src[j] = x + (size_t)min(m0 + S::TURN_ROWS * j + (tid >> 3), M - 1) * K + 8 * piece;
+#pragma unroll
+  for (int j = 0; j < S::W_TURNS; ++j)
+    w_src[j] = w + (size_t)min(n0 + S::TURN_ROWS * j + (tid >> 3), N - 1) * K + 8 * piece;
+  typedef __attribute__((address_space(3))) unsigned char* lds_ptr;
+  const unsigned smem_lds = (unsigned)(unsigned long)(lds_ptr)smem;
+  auto load_to_lds = [&](const void* src, unsigned lds) {
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds) : "memory", "m0");
+  };
+  auto copy_step = [&](int kt, int stage) {
+    const unsigned base = __builtin_amdgcn_readfirstlane(smem_lds + stage * S::STAGE_BYTES + 1024 * wave);
+#pragma unroll
+    for (int j = 0; j < S::X_TURNS; ++j) load_to_lds(x_src[j] + (size_t)kt * BK, base + 16 * S::THREADS * j);
+#pragma unroll
+    for (int j = 0; j < S::W_TURNS; ++j)
+      load_to_lds(w_src[j] + (size_t)kt * BK, base + BM * ROW_BYTES + 16 * S::THREADS * j);
+  };
+  // loads complete in the order they were issued: with no more than the later steps' loads
+  // outstanding, this thread's share of the next step has landed
+  auto wait_for_step = [&](int steps_after) {
+    if (steps_after <= 0)
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    else if (steps_after == 1)
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(S::LOADS) : "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * S::LOADS) : "memory");
+  };
+  static_assert(STAGES >= 2 && STAGES <= 4 && 2 * S::LOADS < 64, "the wait counts above");
+
+  // operand reads: row 16 i + col of this wavefront's half of a slice, pieces 4 s + grp
+  const int swz = (col >> 1) & 7;
+  int read_off[2];
+#pragma unroll
+  for (int s = 0; s < 2; ++s) read_off[s] = col * ROW_BYTES + 16 * ((4 * s + grp) ^ swz);
+  const int x_half = wm * (BM / WM) * ROW_BYTES, w_half = BM * ROW_BYTES + wn * (BN / WN) * ROW_BYTES;
+
+  f32x4_t acc[S::MI][S::NJ];
+#pragma unroll
+  for (int i = 0; i < S::MI; ++i)
+#pragma unroll
+    for (int j = 0; j < S::NJ; ++j) acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  const int steps = K / BK;
+#pragma unroll
+  for (int ahead = 0; ahead < STAGES - 1; ++ahead)
+    if (ahead < steps) copy_step(ahead, ahead);
+  for (int kt = 0; kt < steps; ++kt) {
+    // step kt has landed in every thread's view, and nobody still reads the stage that the
+    // next copy overwrites (step kt - 1's)
+    wait_for_step(min(kt + STAGES - 2, steps - 1) - kt);
+    __syncthreads();
+    const unsigned char* st = smem + (kt % STAGES) * S::STAGE_BYTES;
+    if (kt + STAGES - 1 < steps) copy_step(kt + STAGES - 1, (kt + STAGES - 1) % STAGES);
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      Frag xf[S::MI], wf[S::NJ];
+#pragma unroll
+      for (int i = 0; i < S::MI; ++i)
+        xf[i].u = *reinterpret_cast<const uint4*>(st + x_half + 16 * i * ROW_BYTES + read_off[s]);
+#pragma unroll
+      for (int j = 0; j < S::NJ; ++j)
+        wf[j].u = *reinterpret_cast<const uint4*>(st + w_half + 16 * j * ROW_BYTES + read_off[s]);
+#pragma unroll
+      for (int i = 0; i < S::MI; ++i)
+#pragma unroll
+        for (int j = 0; j < S::NJ; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j].v, xf[i].v, acc[i][j], 0, 0, 0);
+    }
+  }
+
+  // lane (col, grp) of block (i, j) holds out[m][n .. n + 3]
+#pragma unroll
+  for (int i = 0; i < S::MI; ++i) {
+    const int m = m0 + wm * (BM / WM) + 16 * i + col;
+    if (m >= M) continue;
+#pragma unroll
+    for (int j = 0; j < S::NJ; ++j) {
+      const int n = n0 + wn * (BN / WN) + 16 * j + 4 * grp;
+      if (n >= N) continue;
+      const f32x4_t c = acc[i][j];
+      if constexpr (EPI == EPI_SWIGLU) {
+        // rows of w interleave gate and up (row 2 i gate, row 2 i + 1 up); both are rounded to
+        // the activation type first, as a separate activation kernel would have read them
+        OUT* o = out + (size_t)m * (N / 2) + n / 2;
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+          if (n + 2 * p + 1 < N) {
+            const float g = to_float(from_float<OUT>(c[2 * p])), u = to_float(from_float<OUT>(c[2 * p + 1]));
+            o[p] = from_float<OUT>(g / (1.f + expf(-g)) * u);
+          }
+        }
+      } else {
+        OUT* o = out + (size_t)m * N + n;
+        if (n + 3 < N && (N % 4) == 0) {
+          if constexpr (sizeof(OUT) == 4) {
+            *reinterpret_cast<float4*>(o) = make_float4(c[0], c[1], c[2], c[3]);
+          } else {
+            *reinterpret_cast<uint2*>(o) = pack_bf16x4(c);
+          }
+        } else {
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            if (n + q < N) o[q] = from_float<OUT>(c[q]);
+        }
+      }
+    }
+  }
+}
+
+// The tile shapes on offer: (BM, BN, STAGES).
+constexpr int NUM_CONFIGS = 5;
+
+template <typename OUT, int EPI, int BM, int BN, int WM, int WN, int STAGES>
+int launch_config(const void* x, const void* w, void* out, int M, int N, int K, hipStream_t stream) {
+  typedef Shape<BM, BN, WM, WN, STAGES> S;
+  static bool raised[16] = {};   // the dynamic shared-memory limit, once per device
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 16) return Q3_ERR_BAD_ARGUMENT;
+  auto kernel = gemm_tiles_kernel<OUT, EPI, BM, BN, WM, WN, STAGES>;
+  if (!raised[device]) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, S::SMEM_BYTES);
+    if (e != hipSuccess) return (int)e;
+    raised[device] = true;
+  }
+  const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+  const long total = (long)tiles_m * tiles_n;
+  if (total > (1L << 28)) return Q3_ERR_UNSUPPORTED;
+  const int per_xcd = (int)((total + 7) / 8);
+  hipLaunchKernelGGL(kernel, dim3(8 * per_xcd), dim3(S::THREADS), S::SMEM_BYTES, stream, (const bf16_t*)x, (const bf16_t*)w,
+                     (OUT*)out, M, N, K, tiles_m, (int)total, per_xcd);
+  return q3_launch_status();
+}
+
+template <typename OUT, int EPI>
+int launch(int config, const void* x, const void* w, void* out, int M, int N, int K, hipStream_t stream) {
+  switch (config) {
+    case 0: return launch_config<OUT, EPI, 128, 128, 2, 2, 2>(x, w, out, M, N, K, stream);
+    case 1: return launch_config<OUT, EPI, 128, 128, 2, 2, 3>(x, w, out, M, N, K, stream);
+    case 2: return launch_config<OUT, EPI, 256, 128, 4, 2, 2>(x, w, out, M, N, K, stream);
+    case 3: return launch_config<OUT, EPI, 256, 256, 2, 4, 2>(x, w, out, M, N, K, stream);
+    case 4: return launch_config<OUT, EPI, 256, 256, 4, 2, 2>(x, w, out, M, N, K, stream);
+  }
+  return Q3_ERR_BAD_ARGUMENT;
+}
+
+// Whether the kernel takes a product at all.
+inline bool takes(int M, int N, int K) { return M > 0 && N > 0 && K >= BK && K % BK == 0; }
+
+}  // namespace tiles

@@ -15,11 +15,17 @@
 // cache runs before each timed run. Timed warm, products of few rows pick
 // kernels that are the fastest only while the weight sits in that cache.
 //
+// The hand-written tiled kernel (gemm_tiles.h) stands in the same contest: where it takes a
+// size (K a multiple of 64) three of its tile shapes are timed after the library's candidates,
+// and a size goes to whichever kernel was the fastest. q3_matmul_set_kernels narrows the
+// contest to the library's kernels alone, or to the hand-written ones where they take the size.
+//
 // One workspace and one such buffer per device, allocated at first need and kept. Calls on one
 // device share it and the plans: they are serialised by a lock and are meant
 // to come from one stream at a time.
 
 #include "common.h"
+#include "gemm_tiles.h"
 
 #include <hipblaslt/hipblaslt.h>
 
@@ -52,6 +58,7 @@ struct Plan {
   hipblasLtMatrixLayout_t w = nullptr, x = nullptr, out = nullptr;
   hipblasLtMatmulAlgo_t algo;
   bool tuned = false;
+  int own = -1;            // the hand-written kernel's tile shape, if that was chosen; else `algo`
   int candidates = 0, chosen = 0;
   float first_us = 0.f, best_us = 0.f;
 };
@@ -73,6 +80,11 @@ int rows_class(int M) { return M <= 64 ? M : (M + 31) / 32 * 32; }
 std::mutex g_lock;
 std::map<int, Device> g_devices;
 int g_candidates = 16;
+enum { KERNELS_BOTH = 0, KERNELS_LIBRARY = 1, KERNELS_OWN = 2 };
+int g_kernels = KERNELS_BOTH;
+// the tile shapes that enter the contest (the other two never won a size of the 8B, 14B and 32B models)
+constexpr int OWN_CANDIDATES[] = {0, 2, 4};
+constexpr int NUM_OWN = sizeof(OWN_CANDIDATES) / sizeof(OWN_CANDIDATES[0]);
 
 #define HIP_TRY(call)                    \
   do {                                   \
@@ -107,6 +119,12 @@ void forget(Plan& p) {
   p = Plan();
 }
 
+int run_own(int config, const void* x, const void* w, void* out, int M, int N, int K, int out_dtype,
+            hipStream_t stream) {
+  return out_dtype == Q3_F32 ? tiles::launch<float, tiles::EPI_PLAIN>(config, x, w, out, M, N, K, stream)
+                             : tiles::launch<bf16_t, tiles::EPI_PLAIN>(config, x, w, out, M, N, K, stream);
+}
+
 hipblasStatus_t run(Device& d, const Plan& p, const hipblasLtMatmulAlgo_t& algo, const void* x, const void* w,
                     void* out, hipStream_t stream) {
   const float one = 1.f, zero = 0.f;
@@ -114,14 +132,14 @@ hipblasStatus_t run(Device& d, const Plan& p, const hipblasLtMatmulAlgo_t& algo,
                          WORKSPACE_BYTES, stream);
 }
 
-// The shortest of `reps` runs, each with cold caches, in microseconds; negative if the candidate fails.
-float time_candidate(Device& d, const Plan& p, const hipblasLtMatmulAlgo_t& algo, const void* x, const void* w,
-                     void* out, hipStream_t stream, int reps) {
+// The shortest of `reps` runs of `launch`, each with cold caches, in microseconds; negative if it fails.
+template <typename Launch>
+float time_runs(Device& d, hipStream_t stream, int reps, Launch launch) {
   float best = -1.f;
   for (int r = 0; r < reps; ++r) {
     evict_kernel<<<EVICT_BLOCKS, EVICT_THREADS, 0, stream>>>((float4*)d.evict, EVICT_BYTES / sizeof(float4));
     if (hipEventRecord(d.begin, stream) != hipSuccess) return -1.f;
-    if (run(d, p, algo, x, w, out, stream) != HIPBLAS_STATUS_SUCCESS) return -1.f;
+    if (!launch()) return -1.f;
     if (hipEventRecord(d.end, stream) != hipSuccess || hipEventSynchronize(d.end) != hipSuccess) return -1.f;
     float ms = 0.f;
     if (hipEventElapsedTime(&ms, d.begin, d.end) != hipSuccess) return -1.f;
@@ -130,7 +148,21 @@ float time_candidate(Device& d, const Plan& p, const hipblasLtMatmulAlgo_t& algo
   return best;
 }
 
-int choose(Device& d, Plan& p, const void* x, const void* w, void* out, hipStream_t stream, bool capturing) {
+float time_candidate(Device& d, const Plan& p, const hipblasLtMatmulAlgo_t& algo, const void* x, const void* w,
+                     void* out, hipStream_t stream, int reps) {
+  return time_runs(d, stream, reps, [&] { return run(d, p, algo, x, w, out, stream) == HIPBLAS_STATUS_SUCCESS; });
+}
+
+int choose(Device& d, Plan& p, const void* x, const void* w, void* out, int M, int N, int K, int out_dtype,
+           hipStream_t stream, bool capturing) {
+  const bool own_takes = tiles::takes(M, N, K) && g_kernels != KERNELS_LIBRARY;
+  if (own_takes && g_kernels == KERNELS_OWN && capturing) {   // untimed: the first shape, timed at the next eager call
+    p.candidates = 1;
+    p.chosen = 0;
+    p.own = OWN_CANDIDATES[0];
+    p.tuned = false;
+    return 0;
+  }
   hipblasLtMatmulPreference_t pref = nullptr;
   LT_TRY(hipblasLtMatmulPreferenceCreate(&pref));
   size_t bytes = WORKSPACE_BYTES;
@@ -146,39 +178,81 @@ int choose(Device& d, Plan& p, const void* x, const void* w, void* out, hipStrea
   if (got == 0) return Q3_ERR_UNSUPPORTED;
   p.candidates = got;
   p.chosen = 0;
+  p.own = -1;
   p.algo = found[0].algo;
   p.tuned = !capturing;
-  if (capturing || got == 1) return 0;
+  if (capturing || (got == 1 && !own_takes)) return 0;
   if (!d.evict) {
     HIP_TRY(hipMalloc(&d.evict, EVICT_BYTES));
     HIP_TRY(hipMemsetAsync(d.evict, 0, EVICT_BYTES, stream));
   }
   // two passes: all candidates briefly (the first run of each also loads its code), then those
   // near the front again and longer
-  std::vector<float> us(got, -1.f);
+  // candidates got .. got + NUM_OWN - 1 are the hand-written kernel's tile shapes
+  const int all = got + (own_takes ? NUM_OWN : 0);
+  const int first = g_kernels == KERNELS_OWN && own_takes ? got : 0;
+  auto time_one = [&](int i, int reps) {
+    if (i < got) return time_candidate(d, p, found[i].algo, x, w, out, stream, reps);
+    return time_runs(d, stream, reps, [&] {
+      return run_own(OWN_CANDIDATES[i - got], x, w, out, M, N, K, out_dtype, stream) == 0;
+    });
+  };
+  std::vector<float> us(all, -1.f);
   float best = -1.f;
-  for (int i = 0; i < got; ++i) {
-    if (run(d, p, found[i].algo, x, w, out, stream) != HIPBLAS_STATUS_SUCCESS) continue;
-    us[i] = time_candidate(d, p, found[i].algo, x, w, out, stream, 2);
+  for (int i = first; i < all; ++i) {
+    if (time_one(i, 1) < 0.f) continue;     // the first run of a kernel also loads its code
+    us[i] = time_one(i, 2);
     if (us[i] > 0.f && (best < 0.f || us[i] < best)) best = us[i];
   }
   if (best < 0.f) return Q3_ERR_UNSUPPORTED;
-  for (int i = 0; i < got; ++i) {
+  for (int i = first; i < all; ++i) {
     if (us[i] < 0.f || us[i] > 1.2f * best) continue;
-    const float again = time_candidate(d, p, found[i].algo, x, w, out, stream, 5);
+    const float again = time_one(i, 5);
     if (again > 0.f && again < us[i]) us[i] = again;
   }
   int chosen = -1;
-  for (int i = 0; i < got; ++i)
+  for (int i = first; i < all; ++i)
     if (us[i] > 0.f && (chosen < 0 || us[i] < us[chosen])) chosen = i;
-  p.chosen = chosen;
-  p.algo = found[chosen].algo;
-  p.first_us = us[0];
+  p.candidates = all - first;
+  p.chosen = chosen - first;
+  if (chosen < got) {
+    p.algo = found[chosen].algo;
+  } else {
+    p.own = OWN_CANDIDATES[chosen - got];
+  }
+  p.first_us = us[first];
   p.best_us = us[chosen];
   return 0;
 }
 
+// The product by the plan's kernel.
+int run_plan(Device& d, const Plan& p, const void* x, const void* w, void* out, int M, int N, int K, int out_dtype,
+             hipStream_t stream) {
+  if (p.own >= 0) return run_own(p.own, x, w, out, M, N, K, out_dtype, stream);
+  const hipblasStatus_t s = run(d, p, p.algo, x, w, out, stream);
+  return s == HIPBLAS_STATUS_SUCCESS ? 0 : Q3_ERR_LIBRARY + (int)s;
+}
+
 }  // namespace
+
+// The hand-written tiled kernel alone (gemm_tiles.h), tile shape `config` (0 .. q3_gemm_tiles_configs() - 1):
+// x (M, K) and w (N, K) bfloat16, K a multiple of 64; `epilogue` 0: out (M, N) in `out_dtype`; 1: rows of w
+// interleave gate and up, out (M, N / 2) bfloat16 = silu(gate) * up.
+extern "C" int q3_gemm_tiles_configs() { return tiles::NUM_CONFIGS; }
+
+extern "C" int q3_gemm_tiles(const void* x, const void* w, void* out, int M, int N, int K, int out_dtype,
+                             int epilogue, int config, void* stream_) {
+  if (!x || !w || !out || !tiles::takes(M, N, K)) return Q3_ERR_BAD_ARGUMENT;
+  hipStream_t stream = (hipStream_t)stream_;
+  if (epilogue == tiles::EPI_SWIGLU) {
+    if (out_dtype != Q3_BF16 || N % 2) return Q3_ERR_BAD_ARGUMENT;
+    return tiles::launch<bf16_t, tiles::EPI_SWIGLU>(config, x, w, out, M, N, K, stream);
+  }
+  if (epilogue != tiles::EPI_PLAIN) return Q3_ERR_BAD_ARGUMENT;
+  if (out_dtype == Q3_F32) return tiles::launch<float, tiles::EPI_PLAIN>(config, x, w, out, M, N, K, stream);
+  if (out_dtype == Q3_BF16) return tiles::launch<bf16_t, tiles::EPI_PLAIN>(config, x, w, out, M, N, K, stream);
+  return Q3_ERR_BAD_ARGUMENT;
+}
 
 // How many of the library's candidates are timed for a new problem size (1: take its first choice).
 extern "C" int q3_matmul_set_candidates(int n) {
@@ -188,8 +262,19 @@ extern "C" int q3_matmul_set_candidates(int n) {
   return 0;
 }
 
+// Which kernels enter the contest for a new size: 0 the library's and the hand-written one's (the default),
+// 1 the library's alone, 2 the hand-written ones alone where they take the size. Sizes already met keep their
+// choice.
+extern "C" int q3_matmul_set_kernels(int mode) {
+  if (mode < KERNELS_BOTH || mode > KERNELS_OWN) return Q3_ERR_BAD_ARGUMENT;
+  std::lock_guard<std::mutex> hold(g_lock);
+  g_kernels = mode;
+  return 0;
+}
+
 // What was chosen for a size on the current device: info[0] candidates timed, info[1] index chosen,
-// info[2] microseconds of the first candidate, info[3] of the chosen one. Returns 1 if the size is known.
+// info[2] microseconds of the first candidate, info[3] of the chosen one, info[4] the hand-written kernel's
+// tile shape if that was chosen, else -1. Returns 1 if the size is known.
 extern "C" int q3_matmul_plan(int M, int N, int K, int out_dtype, float* info) {
   std::lock_guard<std::mutex> hold(g_lock);
   int device = 0;
@@ -202,6 +287,7 @@ extern "C" int q3_matmul_plan(int M, int N, int K, int out_dtype, float* info) {
   info[1] = (float)p->second.chosen;
   info[2] = p->second.first_us;
   info[3] = p->second.best_us;
+  info[4] = (float)p->second.own;
   return 1;
 }
 
@@ -235,8 +321,9 @@ extern "C" int q3_matmul(const void* x, const void* w, void* out, int M, int N, 
   if (!p.tuned) {
     auto near = d.chosen_near.find(near_key);
     if (near != d.chosen_near.end()) {   // a neighbour's choice, if the library takes it for this size
-      if (run(d, p, near->second.algo, x, w, out, stream) == HIPBLAS_STATUS_SUCCESS) {
-        p.algo = near->second.algo;
+      p.own = near->second.own;
+      p.algo = near->second.algo;
+      if (run_plan(d, p, x, w, out, M, N, K, out_dtype, stream) == 0) {
         p.candidates = near->second.candidates;
         p.chosen = near->second.chosen;
         p.first_us = near->second.first_us;
@@ -247,7 +334,7 @@ extern "C" int q3_matmul(const void* x, const void* w, void* out, int M, int N, 
     }
   }
   if (!p.candidates || (!p.tuned && !capturing)) {
-    const int status = choose(d, p, x, w, out, stream, capturing);
+    const int status = choose(d, p, x, w, out, M, N, K, out_dtype, stream, capturing);
     if (status) {
       forget(p);
       return status;
@@ -255,12 +342,12 @@ extern "C" int q3_matmul(const void* x, const void* w, void* out, int M, int N, 
     if (p.tuned) {
       Plan& kept = d.chosen_near[near_key];   // the choice only: the descriptors stay with their size
       kept.algo = p.algo;
+      kept.own = p.own;
       kept.candidates = p.candidates;
       kept.chosen = p.chosen;
       kept.first_us = p.first_us;
       kept.best_us = p.best_us;
     }
   }
-  LT_TRY(run(d, p, p.algo, x, w, out, stream));
-  return 0;
+  return run_plan(d, p, x, w, out, M, N, K, out_dtype, stream);
 }

@@ -32,6 +32,9 @@ __all__ = [
     "linear_swiglu",
     "linear_residual_norm",
     "matmul_candidates",
+    "matmul_kernels",
+    "gemm_tiles",
+    "gemm_tiles_configs",
     "matmul_plan",
     "tile_weight",
     "sample",
@@ -79,13 +82,52 @@ def matmul_candidates(n):
     _check(library("matmul").q3_matmul_set_candidates(int(n)), "matmul_candidates")
 
 
+def matmul_kernels(which):
+    """Which kernels a product with many rows may go to when it meets a new size: "both" (the
+    vendor library's candidates and the hand-written tiled kernel's shapes are timed and the
+    fastest is kept; the default), "library", or "own" (the hand-written kernel wherever it
+    takes the size: an inner size that is a multiple of 64). Sizes already met keep their choice."""
+    modes = {"both": 0, "library": 1, "own": 2}
+    _need(which in modes, "which is one of %s" % ", ".join(sorted(modes)))
+    _check(library("matmul").q3_matmul_set_kernels(modes[which]), "matmul_kernels")
+
+
 def matmul_plan(M, N, K, out_dtype=torch.bfloat16):
     """What was chosen for a size on the current device, or None if it has not been met:
-    (candidates timed, index chosen, microseconds of the first candidate, of the chosen one)."""
-    info = (ctypes.c_float * 4)()
+    (candidates timed, index chosen, microseconds of the first candidate, of the chosen one,
+    the hand-written kernel's tile shape if that was chosen, else -1)."""
+    info = (ctypes.c_float * 5)()
     if not library("matmul").q3_matmul_plan(int(M), int(N), int(K), _DT[out_dtype], info):
         return None
-    return int(info[0]), int(info[1]), float(info[2]), float(info[3])
+    return int(info[0]), int(info[1]), float(info[2]), float(info[3]), int(info[4])
+
+
+def gemm_tiles_configs():
+    """How many tile shapes the hand-written tiled product offers."""
+    return int(library("matmul").q3_gemm_tiles_configs())
+
+
+def gemm_tiles(x, weight, config=0, out_dtype=None, swiglu=False, out=None):
+    """The hand-written tiled matrix-core product alone, with tile shape `config`: x (M, K) and
+    weight (N, K) bfloat16, K a multiple of 64; out (M, N) bfloat16 or float32, or with `swiglu`
+    (weight rows interleave gate and up) out (M, N / 2) bfloat16 = silu(gate) * up."""
+    _dev(x, weight, out)
+    _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1], "x (M, K) and weight (N, K)")
+    _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "x and weight must be bfloat16")
+    M, K = x.shape
+    N = weight.shape[0]
+    _need(M > 0 and K >= 64 and K % 64 == 0, "the inner size must be a multiple of 64")
+    _need(0 <= config < gemm_tiles_configs(), "no such tile shape")
+    out_dtype = out_dtype or torch.bfloat16
+    _need(out_dtype in _DT and not (swiglu and (out_dtype != torch.bfloat16 or N % 2)),
+          "out is bfloat16 or float32; with swiglu bfloat16 and an even number of weight rows")
+    shape = (M, N // 2) if swiglu else (M, N)
+    if out is None:
+        out = torch.empty(shape, dtype=out_dtype, device=x.device)
+    _need(out.shape == shape and out.dtype == out_dtype, "out must be %s of out_dtype" % (shape,))
+    _check(library("matmul").q3_gemm_tiles(_ptr(x), _ptr(weight), _ptr(out), M, N, K, _DT[out_dtype],
+                                           1 if swiglu else 0, int(config), _stream()), "gemm_tiles")
+    return out
 
 
 def embed_rows(ids, table, out=None):

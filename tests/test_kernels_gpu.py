@@ -463,6 +463,79 @@ def test_linear_many_rows_first_met_in_a_graph():
     assert ops.matmul_plan(M, N, K)[0] > 1
 
 
+@pytest.mark.parametrize("M,N,K", [(200, 304, 128), (513, 1000, 192), (77, 48, 64), (17, 2, 64), (300, 331, 4096),
+                                   (1024, 1536, 1024)])
+def test_tiled_product_every_shape_and_epilogue(M, N, K):
+    """The hand-written tiled matrix-core product: every tile shape, at sizes whose rows and
+    columns end inside a tile, against a float64 product; float32 and bfloat16 outputs and the
+    SwiGLU epilogue; one row's result does not depend on its neighbours."""
+    ops = _ops()
+    x = _rand((M, K), torch.bfloat16, 51)
+    w = _rand((N, K), torch.bfloat16, 52, scale=0.05)
+    want = x.double() @ w.double().T
+    rounded = want.to(torch.bfloat16).double()
+    gated = torch.nn.functional.silu(rounded[:, 0::2]) * rounded[:, 1::2] if N % 2 == 0 else None
+    first = None
+    for config in range(ops.gemm_tiles_configs()):
+        got = ops.gemm_tiles(x, w, config, out_dtype=torch.float32)
+        torch.testing.assert_close(got.double(), want, rtol=1e-4, atol=1e-4)
+        got16 = ops.gemm_tiles(x, w, config)
+        torch.testing.assert_close(got16.double(), want, rtol=1.6e-2, atol=1e-2)
+        # every shape adds a sum's terms in the same order (k ascending, 32 at a time)
+        first = got if first is None else first
+        assert torch.equal(got, first)
+        if gated is not None:
+            act = ops.gemm_tiles(x, w, config, swiglu=True)
+            torch.testing.assert_close(act.double(), gated, rtol=3.2e-2, atol=2e-2)
+        other = x.clone()
+        other[1:] = _rand((M - 1, K), torch.bfloat16, 53)
+        assert torch.equal(ops.gemm_tiles(other, w, config)[0], got16[0])
+    with pytest.raises(ops.OperandError):
+        ops.gemm_tiles(x[:, :K - 8].contiguous(), w[:, :K - 8].contiguous())      # K no multiple of 64
+
+
+def test_linear_many_rows_by_the_hand_written_kernel_alone():
+    """With the contest narrowed to the hand-written kernel, products with many rows are its:
+    a size it takes, also first met inside a graph, and a size it does not take (the library's)."""
+    ops = _ops()
+    ops.linear(_rand((20, 64), torch.bfloat16, 1), _rand((64, 64), torch.bfloat16, 2))   # the device's set-up is eager
+    ops.matmul_kernels("own")
+    try:
+        M, N, K = 150, 840, 320
+        x = _rand((M, K), torch.bfloat16, 54)
+        w = _rand((N, K), torch.bfloat16, 55, scale=0.05)
+        want = x.double() @ w.double().T
+        got = ops.linear(x, w, out_dtype=torch.float32)
+        torch.testing.assert_close(got.double(), want, rtol=1e-4, atol=1e-4)
+        plan = ops.matmul_plan(M, N, K, torch.float32)
+        assert plan[4] >= 0 and plan[0] >= 1
+        assert torch.equal(got, ops.gemm_tiles(x, w, plan[4], out_dtype=torch.float32))
+        # first met in a capture: runs untimed there, timed at the next eager call
+        M2 = 90
+        x2 = _rand((M2, K), torch.bfloat16, 56)
+        out = torch.empty((M2, N), dtype=torch.bfloat16, device=x.device)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                ops.linear(x2, w, out=out)
+        torch.cuda.current_stream().wait_stream(side)
+        for _ in range(3):
+            out.zero_()
+            graph.replay()
+            torch.testing.assert_close(out.double(), x2.double() @ w.double().T, rtol=1.6e-2, atol=1e-2)
+            assert torch.equal(ops.linear(x2, w), out)
+        assert ops.matmul_plan(M2, N, K)[4] >= 0
+        # an inner size it does not take goes to the library
+        x3, w3 = _rand((40, 72), torch.bfloat16, 57), _rand((96, 72), torch.bfloat16, 58, scale=0.05)
+        torch.testing.assert_close(ops.linear(x3, w3, out_dtype=torch.float32).double(), x3.double() @ w3.double().T,
+                                   rtol=2e-3, atol=2e-3)
+        assert ops.matmul_plan(40, 96, 72, torch.float32)[4] == -1
+    finally:
+        ops.matmul_kernels("both")
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 6144, 4096), (8, 4096, 12288), (16, 1000, 96), (3, 331, 64), (9, 24, 2048),
                                    (5, 151936, 256)])
 def test_linear_from_the_tiled_copy(M, N, K):

@@ -18,11 +18,13 @@
 // epilogue, eight bytes of bfloat16 for the plain one.
 //
 // What bounds it (2,048 x 24,576 x 4,096, 256 x 256 tiles, eight wavefronts of 64 x 128): with
-// the copies taken out 233 us (1.77 PFLOP/s), with copies that always hit the cache 303, as it is
-// 323 (1.27), the vendor library's best kernel 279: a step's operand reads (192 KB) and the
-// copies' writes (64 KB) keep shared memory busy for as many cycles as the matrix instructions
-// take. Wavefront tiles of 128 x 128 would read a third less but leave one wavefront a SIMD and
-// no registers to read ahead with (the compiler's schedule of that shape: 364 us).
+// the copies taken out 233 us (1.77 PFLOP/s), with copies that always hit the cache 303, with
+// the copies issued and never waited for 328, as it is 323 (1.27; the matrix pipes are busy 59 %
+// of the cycles, no bank conflicts), the vendor library's best kernel 279. So it is the copies'
+// passage itself, not their latency, that takes the time from the operand reads. Tried and not
+// kept: steps of 32 in four stages with the next step's operands read while the current one is
+// multiplied (385); copies through registers and ds_write (three times slower as the compiler
+// schedules them); wavefront tiles of 128 x 128, one wavefront a SIMD (364).
 //
 // K must be a multiple of 64. Rows of x beyond M and of w beyond N are read from the last
 // valid row and never written. Blocks are numbered so that the eight XCDs each take a
@@ -69,6 +71,49 @@ __device__ inline uint2 pack_bf16x4(f32x4_t c) {
   } pk;
   pk.v = __builtin_convertvector(c, bf16x4_t);
   return pk.u;
+}
+
+// A wavefront's outputs to memory: lane (col, grp) of block (i, j) holds out[m][n .. n + 3] with
+// m = m_base + 16 i + col, n = n_base + 16 j + 4 grp.
+template <typename OUT, int EPI, int MI, int NJ>
+__device__ inline void store_tile(const f32x4_t (&acc)[MI][NJ], OUT* __restrict__ out, int M, int N, int m_base,
+                                  int n_base, int col, int grp) {
+#pragma unroll
+  for (int i = 0; i < MI; ++i) {
+    const int m = m_base + 16 * i + col;
+    if (m >= M) continue;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      const int n = n_base + 16 * j + 4 * grp;
+      if (n >= N) continue;
+      const f32x4_t c = acc[i][j];
+      if constexpr (EPI == EPI_SWIGLU) {
+        // rows of w interleave gate and up (row 2 i gate, row 2 i + 1 up); both are rounded to
+        // the activation type first, as a separate activation kernel would have read them
+        OUT* o = out + (size_t)m * (N / 2) + n / 2;
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+          if (n + 2 * p + 1 < N) {
+            const float g = to_float(from_float<OUT>(c[2 * p])), u = to_float(from_float<OUT>(c[2 * p + 1]));
+            o[p] = from_float<OUT>(g / (1.f + expf(-g)) * u);
+          }
+        }
+      } else {
+        OUT* o = out + (size_t)m * N + n;
+        if (n + 3 < N && (N % 4) == 0) {
+          if constexpr (sizeof(OUT) == 4) {
+            *reinterpret_cast<float4*>(o) = make_float4(c[0], c[1], c[2], c[3]);
+          } else {
+            *reinterpret_cast<uint2*>(o) = pack_bf16x4(c);
+          }
+        } else {
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            if (n + q < N) o[q] = from_float<OUT>(c[q]);
+        }
+      }
+    }
+  }
 }
 
 template <typename OUT, int EPI, int BM, int BN, int WM, int WN, int STAGES>
@@ -136,16 +181,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiles_kernel(const bf16_t* 
     for (int j = 0; j < S::NJ; ++j) acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
   const int steps = K / BK;
-#pragma unroll
-  for (int ahead = 0; ahead < STAGES - 1; ++ahead)
-    if (ahead < steps) copy_step(ahead, ahead);
-  for (int kt = 0; kt < steps; ++kt) {
-    // step kt has landed in every thread's view, and nobody still reads the stage that the
-    // next copy overwrites (step kt - 1's)
-    wait_for_step(min(kt + STAGES - 2, steps - 1) - kt);
-    __syncthreads();
-    const unsigned char* st = smem + (kt % STAGES) * S::STAGE_BYTES;
-    if (kt + STAGES - 1 < steps) copy_step(kt + STAGES - 1, (kt + STAGES - 1) % STAGES);
+  auto multiply_stage = [&](const unsigned char* st) {
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
       Frag xf[S::MI], wf[S::NJ];
@@ -161,45 +197,21 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiles_kernel(const bf16_t* 
         for (int j = 0; j < S::NJ; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j].v, xf[i].v, acc[i][j], 0, 0, 0);
     }
-  }
-
-  // lane (col, grp) of block (i, j) holds out[m][n .. n + 3]
+  };
+  {
 #pragma unroll
-  for (int i = 0; i < S::MI; ++i) {
-    const int m = m0 + wm * (BM / WM) + 16 * i + col;
-    if (m >= M) continue;
-#pragma unroll
-    for (int j = 0; j < S::NJ; ++j) {
-      const int n = n0 + wn * (BN / WN) + 16 * j + 4 * grp;
-      if (n >= N) continue;
-      const f32x4_t c = acc[i][j];
-      if constexpr (EPI == EPI_SWIGLU) {
-        // rows of w interleave gate and up (row 2 i gate, row 2 i + 1 up); both are rounded to
-        // the activation type first, as a separate activation kernel would have read them
-        OUT* o = out + (size_t)m * (N / 2) + n / 2;
-#pragma unroll
-        for (int p = 0; p < 2; ++p) {
-          if (n + 2 * p + 1 < N) {
-            const float g = to_float(from_float<OUT>(c[2 * p])), u = to_float(from_float<OUT>(c[2 * p + 1]));
-            o[p] = from_float<OUT>(g / (1.f + expf(-g)) * u);
-          }
-        }
-      } else {
-        OUT* o = out + (size_t)m * N + n;
-        if (n + 3 < N && (N % 4) == 0) {
-          if constexpr (sizeof(OUT) == 4) {
-            *reinterpret_cast<float4*>(o) = make_float4(c[0], c[1], c[2], c[3]);
-          } else {
-            *reinterpret_cast<uint2*>(o) = pack_bf16x4(c);
-          }
-        } else {
-#pragma unroll
-          for (int q = 0; q < 4; ++q)
-            if (n + q < N) o[q] = from_float<OUT>(c[q]);
-        }
-      }
+    for (int ahead = 0; ahead < STAGES - 1; ++ahead)
+      if (ahead < steps) copy_step(ahead, ahead);
+    for (int kt = 0; kt < steps; ++kt) {
+      // step kt has landed in every thread's view, and nobody still reads the stage that the
+      // next copy overwrites (step kt - 1's)
+      wait_for_step(min(kt + STAGES - 2, steps - 1) - kt);
+      __syncthreads();
+      if (kt + STAGES - 1 < steps) copy_step(kt + STAGES - 1, (kt + STAGES - 1) % STAGES);
+      multiply_stage(smem + (kt % STAGES) * S::STAGE_BYTES);
     }
   }
+  store_tile<OUT, EPI, S::MI, S::NJ>(acc, out, M, N, m0 + wm * (BM / WM), n0 + wn * (BN / WN), col, grp);
 }
 
 // The tile shapes on offer: (BM, BN, STAGES).

@@ -1,5 +1,6 @@
-"""An architecture defined in tests/toy_architecture.py, with config.json keys of its own and a
-mixer that keeps a state per request, goes through the framework's model folder writer, loader,
+"""An architecture defined in tests/toy_architecture.py, with config.json keys of its own, a
+mixer that keeps a state per request and, in its second example, a norm and a block arrangement
+of its own, goes through the framework's model folder writer, loader,
 cache manager, step function, engine and replay program without a change to the framework."""
 
 import json
@@ -21,9 +22,12 @@ from qwen3_from_scratch_amd.weights import write_random_model
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-@pytest.fixture(scope="module")
-def folder(tmp_path_factory):
-    config = toy.ToyHybridConfig.from_dict(toy.EXAMPLE)
+EXAMPLES = {"sequential": toy.EXAMPLE, "parallel": toy.EXAMPLE_PARALLEL}
+
+
+@pytest.fixture(scope="module", params=sorted(EXAMPLES))
+def folder(request, tmp_path_factory):
+    config = toy.ToyHybridConfig.from_dict(EXAMPLES[request.param])
     return write_random_model(str(tmp_path_factory.mktemp("hybrid")), config, seed=9, std=0.08, norm_jitter=0.2)
 
 
@@ -33,8 +37,9 @@ def _plain(folder, requests):
     return config, w, {rid: toy.plain_logits(config, w, toks) for rid, toks in requests.items()}
 
 
-def _requests():
-    return {"h%d" % i: random_tokens(n, toy.EXAMPLE["vocab"], 60 + i) for i, n in enumerate([70, 9, 41, 130, 25])}
+def _requests(folder):
+    vocab = load_model_config(folder).vocab
+    return {"h%d" % i: random_tokens(n, vocab, 60 + i) for i, n in enumerate([70, 9, 41, 130, 25])}
 
 
 def _worst(got, want):
@@ -45,15 +50,19 @@ def _worst(got, want):
 def test_folder_is_read_by_its_architectures_own_keys(folder):
     assert toy.NAME in architectures()
     config = load_model_config(folder)
-    assert isinstance(config, toy.ToyHybridConfig) and config == toy.ToyHybridConfig.from_dict(toy.EXAMPLE)
+    example = EXAMPLES[config.arrangement]
+    assert isinstance(config, toy.ToyHybridConfig) and config == toy.ToyHybridConfig.from_dict(example)
     with open(os.path.join(folder, "config.json")) as fh:
-        assert set(json.load(fh)) == set(toy.EXAMPLE)
+        assert set(json.load(fh)) == set(example)
     names = set(load_file(os.path.join(folder, "model.safetensors")))
-    assert "hybrid.layers.1.self_attn.mix.weight" in names and "hybrid.layers.0.self_attn.q_proj.weight" in names
+    mean_layer, attention_layer = config.pattern.index("s"), config.pattern.index("a")
+    assert "hybrid.layers.%d.self_attn.mix.weight" % mean_layer in names
+    assert "hybrid.layers.%d.self_attn.q_proj.weight" % attention_layer in names
+    assert ("hybrid.norm.bias" in names) == (config.norm == "centred")
 
 
 def test_every_cutting_and_generation_on_the_host(cpu_ops, folder):
-    requests = _requests()
+    requests = _requests(folder)
     config, w, want = _plain(folder, requests)
     for make in (trace_tail_decoded, trace_portions, trace_mixed):
         steps = make(requests)
@@ -90,7 +99,7 @@ def _replay(folder, dtype, steps, out, max_tokens, plugins):
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype,tol", [("float32", 5e-4), ("bfloat16", 0.25)])
 def test_replay_program_takes_the_architecture_as_a_plugin(folder, tmp_path, dtype, tol):
-    requests = _requests()
+    requests = _requests(folder)
     _, _, want = _plain(folder, requests)
     steps = trace_mixed(requests, seed=2)
     out = str(tmp_path / dtype)

@@ -2,7 +2,9 @@
 own configuration class, a function from that configuration to a ModelSpec, and one
 `register_architecture` call. Layers follow a pattern string: `a` is the framework's
 attention (with a window), `s` the running-mean mixer of test_toy_parts.py, which keeps a
-state of fixed size per request. It is no model of anyone's; it shows that the loader, the
+state of fixed size per request. Two more keys choose between the framework's RMS norm and a
+mean-subtracting norm with a bias defined here, and between the framework's sequential block
+and a block defined here whose mixer and feed-forward read the same stream. It is no model of anyone's; it shows that the loader, the
 random-weights writer, the cache manager, the step function, the engine and the replay
 program take an architecture they have never heard of.
 
@@ -17,14 +19,67 @@ import torch
 
 import plain_qwen3 as plain
 import test_toy_parts  # registers the mixer "toy_running_mean"  # noqa: F401
-from qwen3_from_scratch_amd.config import register_architecture
+from qwen3_from_scratch_amd.config import register_architecture, register_part
 from qwen3_from_scratch_amd.config.model_config import ConfigError
 from qwen3_from_scratch_amd.models import LayerSpec, ModelSpec, RunStep
-from qwen3_from_scratch_amd.parts import PartSpec
+from qwen3_from_scratch_amd.parts import Part, PartSpec
 
 NAME = "ToyHybridForCausalLM"
 KEYS = (("vocab", int), ("width", int), ("inner", int), ("heads", int), ("kv_heads", int), ("head_size", int),
-        ("pattern", str), ("window", int), ("eps", float), ("theta", float), ("max_position_embeddings", int))
+        ("pattern", str), ("window", int), ("eps", float), ("theta", float), ("max_position_embeddings", int),
+        ("norm", str), ("arrangement", str))
+
+
+@register_part("norm", "toy_centred")
+class CentredNorm(Part):
+    """y = (x - mean(x)) * rsqrt(var(x) + eps) * weight + bias over the last dimension, in
+    float32, rounded once. The contract of a norm: it reads the float32 stream, and with
+    `delta` adds it into the stream first (in place, unless `rows` selects a subset)."""
+
+    def __init__(self, prefix, precision, device, size, eps):
+        super().__init__(prefix, precision, device)
+        self.size, self.eps = size, float(eps)
+        self.weight = self.bias = None
+
+    def tensors(self):
+        return {self._name("weight"): (self.size,), self._name("bias"): (self.size,)}
+
+    def load(self, fetch):
+        self.weight = fetch(self._name("weight"), torch.float32)
+        self.bias = fetch(self._name("bias"), torch.float32)
+
+    def forward(self, x, delta=None, rows=None):
+        if rows is not None:
+            picked = x[rows.long()]
+            if delta is not None:
+                picked = picked + delta[rows.long()].float()
+        else:
+            if delta is not None:
+                x.add_(delta.float())
+            picked = x
+        centred = picked - picked.mean(dim=-1, keepdim=True)
+        y = centred * torch.rsqrt(centred.pow(2).mean(dim=-1, keepdim=True) + self.eps)
+        return (y * self.weight + self.bias).to(self.precision.act)
+
+
+@register_part("block", "toy_parallel")
+class ParallelBlock(Part):
+    """x = x + mixer(norm_1(x)) + feed_forward(norm_2(x)): both branches read the stream as it
+    entered the block. The contract of a block: the float32 stream and an addend it still lacks
+    come in, the stream and the next such addend go out."""
+
+    def __init__(self, prefix, precision, device):
+        super().__init__(prefix, precision, device)
+
+    def attach(self, mixer, feed_forward, mixer_norm, feed_forward_norm):
+        self.mixer, self.feed_forward = mixer, feed_forward
+        self.mixer_norm, self.feed_forward_norm = mixer_norm, feed_forward_norm
+
+    def forward(self, x, pending, batch, cache, next_norm=None):
+        h1 = self.mixer_norm.forward(x, delta=pending)          # the stream is whole from here on
+        h2 = self.feed_forward_norm.forward(x)
+        mixed = self.mixer.forward(h1, batch, cache)
+        return x, mixed.float() + self.feed_forward.forward(h2, batch).float()
 
 
 @dataclasses.dataclass(frozen=True)
@@ -41,6 +96,8 @@ class ToyHybridConfig:
     eps: float
     theta: float
     max_position_embeddings: int
+    norm: str
+    arrangement: str
     eos_token_ids: tuple = ()
 
     @classmethod
@@ -50,6 +107,8 @@ class ToyHybridConfig:
             raise ConfigError("config.json of %s lacks %s" % (NAME, ", ".join(missing)))
         if not data["pattern"] or set(data["pattern"]) - set("as"):
             raise ConfigError("pattern must be a string of 'a' and 's'")
+        if data["norm"] not in ("rms", "centred") or data["arrangement"] not in ("sequential", "parallel"):
+            raise ConfigError("norm is rms or centred, arrangement sequential or parallel")
         return cls(architecture=data["architectures"][0], **{k: kind(data[k]) for k, kind in KEYS})
 
     def to_dict(self):
@@ -60,13 +119,14 @@ class ToyHybridConfig:
 
 
 def toy_hybrid_spec(c):
-    norm = PartSpec.of("norm", "rms", size=c.width, eps=c.eps)
+    norm = PartSpec.of("norm", "rms" if c.norm == "rms" else "toy_centred", size=c.width, eps=c.eps)
+    block = PartSpec.of("block", "pre_norm" if c.arrangement == "sequential" else "toy_parallel")
     attention = PartSpec.of("mixer", "attention", hidden_size=c.width, num_heads=c.heads, num_kv_heads=c.kv_heads,
                             head_dim=c.head_size, qk_norm=False, qk_norm_eps=c.eps, window=c.window)
     mean = PartSpec.of("mixer", "toy_running_mean", hidden_size=c.width)
     ff = PartSpec.of("feed_forward", "swiglu", hidden_size=c.width, intermediate_size=c.inner)
     layers = tuple(LayerSpec(prefix="hybrid.layers.%d" % i, mixer=attention if kind == "a" else mean, feed_forward=ff,
-                             mixer_norm=norm, feed_forward_norm=norm) for i, kind in enumerate(c.pattern))
+                             mixer_norm=norm, feed_forward_norm=norm, block=block) for i, kind in enumerate(c.pattern))
     return ModelSpec(
         hidden_size=c.width, vocab_size=c.vocab,
         embedding=PartSpec.of("embedding", "token", vocab_size=c.vocab, hidden_size=c.width),
@@ -81,7 +141,18 @@ def toy_hybrid_spec(c):
 register_architecture(NAME, ToyHybridConfig, toy_hybrid_spec)
 
 EXAMPLE = dict(architectures=[NAME], vocab=211, width=40, inner=72, heads=6, kv_heads=2, head_size=16, pattern="asa",
-               window=21, eps=1e-5, theta=10000.0, max_position_embeddings=512)
+               window=21, eps=1e-5, theta=10000.0, max_position_embeddings=512, norm="rms", arrangement="sequential")
+# every size and option differs; the norm and the block are the ones defined above
+EXAMPLE_PARALLEL = dict(architectures=[NAME], vocab=157, width=56, inner=100, heads=4, kv_heads=4, head_size=32,
+                        pattern="saas", window=0, eps=1e-6, theta=500000.0, max_position_embeddings=300,
+                        norm="centred", arrangement="parallel")
+
+
+def _norm(c, x, w, name):
+    if c.norm == "rms":
+        return plain.rms_norm(x, w[name + ".weight"], c.eps)
+    centred = x - x.mean(dim=-1, keepdim=True)
+    return centred * torch.rsqrt(centred.pow(2).mean(dim=-1, keepdim=True) + c.eps) * w[name + ".weight"] + w[name + ".bias"]
 
 
 def plain_logits(c, w, tokens):
@@ -92,10 +163,10 @@ def plain_logits(c, w, tokens):
     x = w["hybrid.embed.weight"][torch.tensor(tokens)]
     for i, kind in enumerate(c.pattern):
         p = "hybrid.layers.%d" % i
-        h = plain.rms_norm(x, w[p + ".input_layernorm.weight"], c.eps)
+        h = _norm(c, x, w, p + ".input_layernorm")
         if kind == "s":
             mean = torch.cumsum(h, dim=0) / torch.arange(1, T + 1)[:, None]
-            x = x + mean @ w[p + ".self_attn.mix.weight"].T
+            mixed = mean @ w[p + ".self_attn.mix.weight"].T
         else:
             a = p + ".self_attn"
             ang = plain.rotary_angles(pos, c.head_size, c.theta, torch.float32)
@@ -103,7 +174,10 @@ def plain_logits(c, w, tokens):
             k = plain.apply_rotary((h @ w[a + ".k_proj.weight"].T).view(T, c.kv_heads, c.head_size), ang)
             v = (h @ w[a + ".v_proj.weight"].T).view(T, c.kv_heads, c.head_size)
             o = plain.causal_attention(q, k, v, 1.0 / math.sqrt(c.head_size), c.window or None)
-            x = x + o.reshape(T, c.heads * c.head_size) @ w[a + ".o_proj.weight"].T
-        h = plain.rms_norm(x, w[p + ".post_attention_layernorm.weight"], c.eps)
-        x = x + plain.swiglu_mlp(h, w, p + ".mlp")
-    return plain.rms_norm(x, w["hybrid.norm.weight"], c.eps) @ w["hybrid.embed.weight"].T
+            mixed = o.reshape(T, c.heads * c.head_size) @ w[a + ".o_proj.weight"].T
+        if c.arrangement == "parallel":
+            x = x + mixed + plain.swiglu_mlp(_norm(c, x, w, p + ".post_attention_layernorm"), w, p + ".mlp")
+        else:
+            x = x + mixed
+            x = x + plain.swiglu_mlp(_norm(c, x, w, p + ".post_attention_layernorm"), w, p + ".mlp")
+    return _norm(c, x, w, "hybrid.norm") @ w["hybrid.embed.weight"].T

@@ -63,6 +63,8 @@ class EngineConfig:
     block_size: int = 16
     gpu_utilization: float = 0.5
     chunked_prefill_size: int = 512
+    # requests take over the cached blocks of a prefix they share with earlier ones (batch_config.py:147)
+    enable_prefix_cache: bool = True
     # an explicit number of cache pages; overrides gpu_utilization when set
     num_blocks: int = 0
     seed: int = 0
@@ -128,7 +130,7 @@ class EngineConfig:
             generation=generation,
         )
         for key in ("max_num_seqs", "max_num_tokens", "block_size", "gpu_utilization",
-                    "chunked_prefill_size", "num_blocks"):
+                    "chunked_prefill_size", "num_blocks", "enable_prefix_cache"):
             if key in sched:
                 kwargs[key] = sched[key]
         kwargs.update(overrides)

@@ -119,10 +119,10 @@ class ModelRunner:
     code, kernels and cache as any other step.
     """
 
-    def __init__(self, model, page_size, num_pages, max_requests, use_graphs=True):
+    def __init__(self, model, page_size, num_pages, max_requests, use_graphs=True, prefix_cache=False):
         self.model = model
         self.device = model.device
-        self.manager = CacheManager(model.plane_needs, page_size, num_pages, max_requests)
+        self.manager = CacheManager(model.plane_needs, page_size, num_pages, max_requests, prefix_cache=prefix_cache)
         self.storage = CacheStorage(self.manager, model.precision.act, self.device)
         self.vocab_size = model.spec.vocab_size
         self.max_positions = getattr(model.position, "max_positions", None)

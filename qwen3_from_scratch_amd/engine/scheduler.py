@@ -11,6 +11,12 @@ drops them, :155-162). Waiting requests are admitted in arrival order without
 overtaking, and a preempted request returns to the front of the queue. And if
 no request at all can advance because prompts in progress hold every page, the
 newest of them is preempted, so that a step can always be made.
+
+With the cache manager's prefix index on, a request that is admitted first takes
+over the leading full blocks that the index already holds for its tokens
+(the reference's `share_prefix`, scheduler.py:121-135) and starts its prompt
+behind them; after every step the blocks a request has filled are registered. A
+preempted request finds its own blocks again if nobody needed their pages meanwhile.
 """
 
 from collections import deque
@@ -38,6 +44,7 @@ class Request:
     status: RequestStatus = RequestStatus.WAITING
     last_token_id: int = -1
     preemptions: int = 0
+    blocks_offered: int = 0        # full blocks that the prefix index has been offered
 
     def __post_init__(self):
         self.prompt = list(self.prompt)
@@ -158,8 +165,12 @@ class Scheduler:
         while self.waiting and len(scheduled) < max_seqs and tokens < max_tokens \
                 and len(self.running) < self.max_num_seqs:
             req = self.waiting[0]
+            shared = self._share_prefix(req)
             n = min(req.prefill_target - req.computed, self.chunked_prefill_size, max_tokens - tokens)
             if not self.manager.can_grow(req.request_id, n, spare):
+                if shared:                              # it waits on: what it took over goes back
+                    self.manager.release(req.request_id)
+                    req.computed = req.blocks_offered = 0
                 break                                   # no overtaking
             self.waiting.popleft()
             req.status = RequestStatus.RUNNING
@@ -168,11 +179,29 @@ class Scheduler:
             tokens += n
         return scheduled
 
+    def _share_prefix(self, req):
+        """A waiting request that holds nothing yet is admitted to the cache and
+        takes over what the prefix index has of its tokens. True if it did."""
+        m = self.manager
+        if not getattr(m, "prefix_cache", False) or req.computed or m.has(req.request_id):
+            return False
+        try:
+            m.admit(req.request_id)
+        except Exception:
+            return False                                # no slot: can_grow says so next
+        req.computed = m.share_prefix(req.request_id, req.tokens[:req.prefill_target])
+        req.blocks_offered = req.computed // m.page_size
+        if not req.computed:
+            m.release(req.request_id)                   # nothing found: the step admits it as usual
+            return False
+        return True
+
     def _preempt(self, req, keep_in_running=True):
         self.release(req.request_id)
         if req in self.running:
             self.running.remove(req)
         req.computed = 0
+        req.blocks_offered = 0
         req.prefill_target = req.num_tokens
         req.status = RequestStatus.WAITING
         req.preemptions += 1
@@ -187,6 +216,11 @@ class Scheduler:
         for s in plan:
             req = s.request
             req.computed += s.num_tokens
+            full = req.computed // self.manager.page_size
+            if full > req.blocks_offered and getattr(self.manager, "prefix_cache", False) \
+                    and self.manager.has(req.request_id):
+                self.manager.register_prefix(req.request_id, req.tokens)
+                req.blocks_offered = full
             if not s.samples:
                 continue
             token = int(next(it))

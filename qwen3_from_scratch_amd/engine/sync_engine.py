@@ -88,7 +88,7 @@ class SyncEngine:
         self.max_len = min(config.max_len, mc.max_position_embeddings)
         num_blocks = config.num_blocks or self._blocks_from_memory()
         self.runner = ModelRunner(self.model, config.block_size, num_blocks, max_requests=config.max_num_seqs,
-                                  use_graphs=config.use_graphs)
+                                  use_graphs=config.use_graphs, prefix_cache=config.enable_prefix_cache)
         self.sampler = Sampler(self.model.device)
         self.scheduler = Scheduler(
             self.runner.manager, config.max_num_seqs, config.max_num_tokens, config.chunked_prefill_size,

@@ -173,6 +173,7 @@ models:
 scheduler:
   max_num_seqs: 8
   chunked_prefill_size: 24
+  enable_prefix_cache: false
 kv_cache_dtype: bfloat16
 """ % model_folders["B"]
     path = tmp_path / "engine.yaml"
@@ -182,6 +183,7 @@ kv_cache_dtype: bfloat16
     assert cfg.max_num_tokens == 3000 and cfg.block_size == 16 and cfg.gpu_utilization == 0.5
     assert cfg.generation.temperature == 0.7 and cfg.generation.top_k == 40
     assert cfg.generation.max_new_tokens == 512 and cfg.max_len == 2048
+    assert cfg.enable_prefix_cache is False and EngineConfig().enable_prefix_cache is True
     with pytest.raises(KeyError):
         EngineConfig.from_yaml(str(path), "other")
     with pytest.raises(ConfigError):

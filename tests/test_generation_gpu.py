@@ -45,6 +45,31 @@ def test_chunked_generation_with_preemption_equals_plain(model_folders):
     assert sum(r.preemptions for r in requests) > 0
 
 
+@pytest.mark.parametrize("name,block_size,num_blocks", [("B", 8, 60), ("B", 8, 14), ("D", 16, 30)])
+def test_shared_prefixes_change_no_token(model_folders, name, block_size, num_blocks):
+    """Requests that begin alike take over each other's cached blocks, at once, later and after
+    a preemption, through prompt steps and graph replays; float32 tokens are the plain
+    implementation's."""
+    vocab = TINY[name]["config"]["vocab_size"]
+    stem = random_tokens(50, vocab, 90)
+    prompts = [stem + random_tokens(n, vocab, 91 + n) for n in (3, 11, 1)] + [stem[:33], random_tokens(20, vocab, 99)]
+    want = _plain_greedy(model_folders[name], prompts, 8)
+    engine = SyncEngine(path=model_folders[name], dtype="float32", block_size=block_size, num_blocks=num_blocks,
+                        max_num_seqs=3, max_num_tokens=40, chunked_prefill_size=24)
+    manager = engine.runner.manager
+    requests = [engine.add_request(p, engine.default_params(8, temperature=0.0, ignore_eos=True)) for p in prompts]
+    while engine.scheduler.has_work():
+        engine.step()
+        manager.audit()
+    assert [r.generated for r in requests] == want
+    assert manager.prefix_hits >= 48 + 32 and manager.num_free() == num_blocks      # at least two requests found the stem
+    if num_blocks == 14:
+        assert sum(r.preemptions for r in requests) > 0
+    before = manager.prefix_hits
+    assert engine.generate_ids([prompts[1]], max_new_tokens=8, temperature=0.0, ignore_eos=True) == [want[1]]
+    assert manager.prefix_hits > before
+
+
 def test_bfloat16_generation_and_seeded_sampling(model_folders):
     vocab = TINY["B"]["config"]["vocab_size"]
     prompts = [random_tokens(n, vocab, 50 + n) for n in (1, 9, 64, 130)]

@@ -165,3 +165,40 @@ def test_a_step_ahead_under_random_arrivals(cpu_ops, model_folders, seed):
     plain = run(False)
     rng.setstate(state)
     assert run(True) == plain
+
+
+def test_shared_prefixes_change_no_token(cpu_ops, model_folders):
+    """Requests that begin alike take over each other's cached blocks (at once, later, and after
+    a preemption) and generate what the plain implementation generates; the index saves prompt
+    tokens and loses no page."""
+    vocab = TINY["B"]["config"]["vocab_size"]
+    stem = random_tokens(50, vocab, 90)
+    prompts = [stem + random_tokens(n, vocab, 91 + n) for n in (3, 11, 1)] + [stem[:33], random_tokens(20, vocab, 99)]
+    want = _plain_greedy(model_folders["B"], prompts, 8)
+    kw = dict(path=model_folders["B"], dtype="float32", device="cpu", block_size=8, max_num_seqs=3,
+              max_num_tokens=40, chunked_prefill_size=24)
+    for num_blocks in (60, 14):                  # room for all; so little that requests are preempted
+        engine = SyncEngine(num_blocks=num_blocks, **kw)
+        manager = engine.runner.manager
+        assert manager.prefix_cache
+        requests = [engine.add_request(p, engine.default_params(8, temperature=0.0, ignore_eos=True)) for p in prompts]
+        steps = 0
+        while engine.scheduler.has_work():
+            engine.step()
+            manager.audit()
+            steps += 1
+        assert [r.generated for r in requests] == want, num_blocks
+        assert manager.prefix_hits >= 48 + 32                      # at least two requests found the stem
+        assert manager.num_free() == num_blocks
+        if num_blocks == 14:
+            assert sum(r.preemptions for r in requests) > 0
+        # a later request finds what the ended ones left
+        before = manager.prefix_hits
+        again = engine.generate_ids([prompts[1]], max_new_tokens=8, temperature=0.0, ignore_eos=True)
+        assert again == [want[1]]
+        if num_blocks == 60:
+            assert manager.prefix_hits - before == 56              # 61 tokens: seven full blocks of eight
+    # with the index off the same tokens, and nothing is taken over
+    engine = SyncEngine(num_blocks=60, enable_prefix_cache=False, **kw)
+    assert engine.generate_ids(prompts, max_new_tokens=8, temperature=0.0, ignore_eos=True) == want
+    assert engine.runner.manager.prefix_hits == 0 and not engine.runner.manager.prefix_cache

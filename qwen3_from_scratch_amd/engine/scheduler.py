@@ -169,6 +169,7 @@ class Scheduler:
             n = min(req.prefill_target - req.computed, self.chunked_prefill_size, max_tokens - tokens)
             if not self.manager.can_grow(req.request_id, n, spare):
                 if shared:                              # it waits on: what it took over goes back
+                    self.manager.prefix_hits -= req.computed
                     self.manager.release(req.request_id)
                     req.computed = req.blocks_offered = 0
                 break                                   # no overtaking

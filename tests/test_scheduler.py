@@ -198,3 +198,34 @@ def test_every_request_finishes_within_budgets_under_random_load(seed):
         ids = [e.request.request_id for e in plan]
         assert len(set(ids)) == len(ids)
     assert m.num_free() == m.num_pages()
+
+
+def test_a_request_starts_behind_the_blocks_the_prefix_index_holds():
+    """The reference's share_prefix (scheduler.py:121-135; test_scheduler.py's prefix cases): a
+    request whose first blocks are cached is scheduled from behind them; a whole hit keeps its
+    last block to compute; one that cannot get its remaining pages gives back what it took over
+    and waits."""
+    m = CacheManager([CacheNeed(2, 16)], page_size=4, num_pages=8, max_requests=4, prefix_cache=True)
+    s = Scheduler(m, 4, 100, 100)
+    s.add(Request("a", list(range(10)), SamplingParams(max_new_tokens=1)))
+    plan = run_step(m, s)
+    assert [(e.num_tokens, e.samples) for e in plan] == [(10, True)] and not s.has_work()
+    assert m.num_free() == 8 and m.groups[0].pool.num_free == 6       # two nodes keep their pages
+    s.add(Request("b", list(range(8)) + [50, 51, 52], SamplingParams(max_new_tokens=2)))
+    s.add(Request("c", list(range(8)), SamplingParams(max_new_tokens=2)))
+    plan = s.schedule()
+    assert [(e.request.request_id, e.request.computed, e.num_tokens) for e in plan] == [("b", 8, 3), ("c", 4, 4)]
+    for e in plan:
+        m.reserve(e.request.request_id, e.num_tokens)
+        m.commit(e.request.request_id, e.num_tokens)
+    s.after_step(plan, [7, 7])
+    m.audit()
+    assert m.prefix_hits == 12
+    # five pages are in use (two nodes, b's third block, c's second, which stays its own); d's whole
+    # prompt is cached, but the four more pages that its remaining tokens and d2 ask for are not there
+    s.add(Request("d", list(range(8)) + [50, 51, 52] + list(range(60, 72)), SamplingParams(max_new_tokens=1)))
+    before = m.prefix_hits
+    plan = s.schedule()
+    assert [e.request.request_id for e in plan] == ["b", "c"] and s.waiting[0].computed == 0
+    assert not m.has("d") and m.prefix_hits == before
+    m.audit()

@@ -80,3 +80,35 @@ def test_schedules_agree_at_real_sizes(folder):
     assert [len(t) for t in roomy] == news
     assert preemptions > 0
     assert tight == roomy
+
+
+def test_long_prompt_in_portions_at_real_sizes(folder):
+    """A prompt of 3,000 tokens whole, in portions of 512 and in portions of 300: the later
+    portions run over thousands of cached keys, where the prompt kernel shares a row tile's keys
+    out over several blocks. bfloat16 against the float32 engine at a few places."""
+    tokens = random_tokens(3000, 151936, 7)
+    places = [0, 1499, 2559, 2998, 2999]
+
+    def run(dtype, portion):
+        runner = load_runner(folder, dtype=dtype, page_size=16, max_tokens=3008, max_requests=2)
+        got, at = {}, 0
+        while at < len(tokens):
+            part = tokens[at:at + portion]
+            want = [p - at for p in places if at <= p < at + len(part)]
+            logits = runner.step([StepEntry("long", part, want)])
+            for row, p in enumerate(p for p in places if at <= p < at + len(part)):
+                got[p] = logits[row].float().cpu()
+            at += len(part)
+        runner.finish("long")
+        assert runner.manager.num_free() == runner.manager.num_pages()
+        return got
+
+    truth = run("float32", 3000)
+    for portion in (3000, 512, 300):
+        got = run("bfloat16", portion)
+        for p in places:
+            scale = max(1.0, float(truth[p].abs().max()))
+            assert float((got[p] - truth[p]).abs().max()) <= 6e-2 * scale, (portion, p)
+    again = run("float32", 700)
+    for p in places:
+        assert float((again[p] - truth[p]).abs().max()) <= 3e-4 * max(1.0, float(truth[p].abs().max())), p

@@ -7,7 +7,7 @@ Random bfloat16 weights, uniform-random prompts of 2,048 tokens, greedy decoding
 through the engine's own step loop (scheduler, step function, sampling). A
 "step" is one decode step of the whole batch. One JSON line is printed:
 `value` is decoded tokens per second at the default batch; `prefill` is one
-2,048-token prompt in one step; `roofline` prices the decode step against HBM
+2,048-token prompt in one step (the median of three); `roofline` prices the decode step against HBM
 bandwidth; `points` holds decoding at batch 1 and 64. The default run is the
 8B shape with prompts of 2,048 in a context of 8,192; `--shape`, `--prompt` and
 `--context` move the decode measurement to the larger shapes and to longer
@@ -70,7 +70,8 @@ def continuous(args, config, model, shape_name, gen, sync):
     sizes = [(rng.randint(128, 4096), rng.randint(64, 512)) for _ in range(requests)]
     engine = SyncEngine(model=model, path="", dtype=args.dtype, device="cuda:0", max_len=context, block_size=BLOCK,
                         num_blocks=requests * context // BLOCK // 2, max_num_seqs=requests,
-                        max_num_tokens=portion + requests, chunked_prefill_size=portion)
+                        max_num_tokens=portion + requests, chunked_prefill_size=portion,
+                        enable_prefix_cache=False)         # the second pass computes every prompt again
     for _ in range(2):
         for prompt, generated in sizes:
             engine.add_request(torch.randint(0, config.vocab_size, (prompt,), generator=gen).tolist(),
@@ -147,7 +148,8 @@ def main():
         pages = batch * (context // BLOCK)
         return SyncEngine(model=model, path="", dtype=args.dtype, device="cuda:0", max_len=context,
                           block_size=BLOCK, num_blocks=pages, max_num_seqs=batch,
-                          max_num_tokens=max(PREFILL, batch), chunked_prefill_size=PREFILL)
+                          max_num_tokens=max(PREFILL, batch), chunked_prefill_size=PREFILL,
+                          enable_prefix_cache=False)       # every token of every prompt is computed
 
     def sync():
         torch.cuda.synchronize()
@@ -157,18 +159,19 @@ def main():
 
     # ---- prefill: one prompt of 2,048 tokens in one step ----
     engine = engine_for(1)
-    prefill_s = None
-    for _ in range(0 if args.skip_prefill else 2):   # warm-up, then the timed one
+    timings = []
+    for _ in range(0 if args.skip_prefill else 4):   # a warm-up, then three timed ones, each a new prompt
         engine.add_request(prompts(1, PREFILL)[0], engine.default_params(1, temperature=0.0, ignore_eos=True))
         sync()
         t0 = time.perf_counter()
         plan = engine.step()
         sync()
-        prefill_s = time.perf_counter() - t0
+        timings.append(time.perf_counter() - t0)
         assert len(plan) == 1 and plan[0].num_tokens == PREFILL
         while engine.scheduler.has_work():
             engine.step()
     prefill = None
+    prefill_s = sorted(timings[1:])[1] if timings else None      # the median of the timed three
     if prefill_s is not None:
         prefill = {"value": round(PREFILL / prefill_s, 1), "tokens": PREFILL, "ms": round(prefill_s * 1e3, 3),
                    "frac": round(prefill_flops(config, PREFILL) / prefill_s / PEAK_FLOPS[args.dtype], 4)}

@@ -1,8 +1,8 @@
 """Compile the HIP sources under csrc/ for gfx950 and load them with ctypes.
 
 Each `<module>.hip` becomes `csrc/lib/<module>.so`. A module is built when its
-library is missing or was built from other sources or flags (a digest is kept
-beside it), at the first call of an operation that lives in it; nothing else
+library is missing or was built from other sources or flags (a digest of the
+file, the headers it includes and the flags is kept beside it), at the first call of an operation that lives in it; nothing else
 is compiled. If the package folder cannot be written, libraries go to a
 temporary folder. There is no other implementation to fall back to: a failure
 to build or load raises.
@@ -11,6 +11,7 @@ to build or load raises.
 import ctypes
 import hashlib
 import os
+import re
 import shutil
 import subprocess
 import sys
@@ -52,14 +53,27 @@ def _hipcc():
     raise ExtensionError("hipcc was not found (looked at $HIPCC, PATH and /opt/rocm/bin)")
 
 
+def _sources(module):
+    """The module's .hip file and the headers of this folder that it includes, directly or
+    through another header."""
+    found, todo = [], [module + ".hip"]
+    while todo:
+        name = todo.pop()
+        if name in found or not os.path.isfile(os.path.join(CSRC, name)):
+            continue
+        found.append(name)
+        with open(os.path.join(CSRC, name), encoding="utf-8", errors="replace") as fh:
+            todo += re.findall(r'^\s*#\s*include\s+"([^"]+)"', fh.read(), flags=re.MULTILINE)
+    return sorted(found)
+
+
 def _digest(module):
     h = hashlib.sha256()
     h.update(" ".join(FLAGS + LINKS.get(module, [])).encode())
-    for name in sorted(os.listdir(CSRC)):
-        if name.endswith(".h") or name == module + ".hip":
-            with open(os.path.join(CSRC, name), "rb") as fh:
-                h.update(name.encode())
-                h.update(fh.read())
+    for name in _sources(module):
+        with open(os.path.join(CSRC, name), "rb") as fh:
+            h.update(name.encode())
+            h.update(fh.read())
     return h.hexdigest()
 
 

@@ -23,8 +23,8 @@
 // of the cycles, no bank conflicts), the vendor library's best kernel 279. So it is the copies'
 // passage itself, not their latency, that takes the time from the operand reads. Tried and not
 // kept: steps of 32 in four stages with the next step's operands read while the current one is
-// multiplied (385); copies through registers and ds_write (three times slower as the compiler
-// schedules them); wavefront tiles of 128 x 128, one wavefront a SIMD (364).
+// multiplied (385); copies through registers and ds_write (365); wavefront tiles of 128 x 128,
+// one wavefront a SIMD (364).
 //
 // K must be a multiple of 64. Rows of x beyond M and of w beyond N are read from the last
 // valid row and never written. Blocks are numbered so that the eight XCDs each take a

@@ -244,6 +244,7 @@ extern "C" int q3_gemm_tiles(const void* x, const void* w, void* out, int M, int
                              int epilogue, int config, void* stream_) {
   if (!x || !w || !out || !tiles::takes(M, N, K)) return Q3_ERR_BAD_ARGUMENT;
   hipStream_t stream = (hipStream_t)stream_;
+  std::lock_guard<std::mutex> hold(g_lock);   // the launchers keep a per-device flag
   if (epilogue == tiles::EPI_SWIGLU) {
     if (out_dtype != Q3_BF16 || N % 2) return Q3_ERR_BAD_ARGUMENT;
     return tiles::launch<bf16_t, tiles::EPI_SWIGLU>(config, x, w, out, M, N, K, stream);

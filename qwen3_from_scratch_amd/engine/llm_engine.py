@@ -59,7 +59,7 @@ class LLMEngine:
         config_path, model_name, config, model, overrides = self._arguments
         try:
             self.engine = SyncEngine(config_path, model_name, config=config, model=model, **overrides)
-        except BaseException as exc:            # the callers learn of it in wait_ready()
+        except Exception as exc:                # the callers learn of it in wait_ready()
             self._failure = exc
             self._ready.set()
             return
@@ -71,7 +71,7 @@ class LLMEngine:
                 continue
             try:
                 plan = engine.step()
-            except BaseException as exc:        # nothing can go on: every caller is told
+            except Exception as exc:            # nothing can go on: every caller is told
                 for stream in self._streams.values():
                     stream.send(exc)
                 self._streams.clear()
@@ -119,7 +119,7 @@ class LLMEngine:
                 prompt = engine.tokenizer.apply_chat_template(prompt, tokenize=False, **template)
             stream.request = engine.add_request(prompt, engine.default_params(max_new_tokens, **sampling),
                                                 request_id=request_id)
-        except BaseException as exc:            # a prompt that cannot be served: its caller alone is told
+        except Exception as exc:                # a prompt that cannot be served: its caller alone is told
             stream.send(exc)
             return
         self._streams[request_id] = stream

@@ -23,6 +23,7 @@ from collections import deque
 from dataclasses import dataclass, field
 from enum import Enum
 
+from ..cache import OutOfPages
 from ..sampling import SamplingParams
 
 
@@ -188,7 +189,7 @@ class Scheduler:
             return False
         try:
             m.admit(req.request_id)
-        except Exception:
+        except OutOfPages:
             return False                                # no slot: can_grow says so next
         req.computed = m.share_prefix(req.request_id, req.tokens[:req.prefill_target])
         req.blocks_offered = req.computed // m.page_size

@@ -1,7 +1,7 @@
 """Decode and prefill throughput of the Qwen3-8B-shaped model on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L]
-                    [--shape 8b|14b|32b] [--prompt P] [--context C] [--workload decode|continuous]
+                    [--shape 8b|14b|32b] [--prompt P] [--context C] [--workload decode|continuous|prefix]
 
 Random bfloat16 weights, uniform-random prompts of 2,048 tokens, greedy decoding
 through the engine's own step loop (scheduler, step function, sampling). A
@@ -99,6 +99,55 @@ def continuous(args, config, model, shape_name, gen, sync):
     return 0
 
 
+def shared_prefix(args, config, model, shape_name, gen, sync):
+    """64 requests that begin with the same 2,048 tokens (a system prompt, say) and go on with 32
+    to 256 tokens of their own, 64 generated tokens each, with the prefix index on and off. Each
+    engine serves such a load twice, with new tokens behind the shared ones each time; the second
+    pass is the one reported (with the index on it finds the shared blocks of the first pass, as
+    a server that has seen the system prompt before would)."""
+    import random
+
+    import torch
+
+    from qwen3_from_scratch_amd.engine import SyncEngine
+
+    requests, stem_len, context = 64, 2048, 4096
+    rng = random.Random(0)
+    stem = torch.randint(0, config.vocab_size, (stem_len,), generator=gen).tolist()
+    tails = [rng.randint(32, 256) for _ in range(requests)]
+    seconds, hits = {}, {}
+    for on in (False, True):
+        engine = SyncEngine(model=model, path="", dtype=args.dtype, device="cuda:0", max_len=context, block_size=BLOCK,
+                            num_blocks=requests * context // BLOCK // 2, max_num_seqs=requests,
+                            max_num_tokens=512 + requests, chunked_prefill_size=512, enable_prefix_cache=on)
+        for _ in range(2):
+            before = engine.runner.manager.prefix_hits
+            # every pass has new tokens behind the shared ones: only those can be found again
+            prompts = [stem + torch.randint(0, config.vocab_size, (n,), generator=gen).tolist() for n in tails]
+            for p in prompts:
+                engine.add_request(p, engine.default_params(64, temperature=0.0, ignore_eos=True))
+            sync()
+            t0 = time.perf_counter()
+            while engine.scheduler.has_work():
+                engine.step()
+            sync()
+            seconds[on] = time.perf_counter() - t0
+            hits[on] = engine.runner.manager.prefix_hits - before
+        del engine
+    tokens_in = sum(len(p) for p in prompts)
+    print(json.dumps({
+        "metric": "shared-prefix load, seconds, %s %s" % (shape_name, "bf16" if args.dtype == "bfloat16" else "fp32"),
+        "value": round(seconds[True], 3), "unit": "s", "n_gpus": 1, "higher_is_better": False,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
+        "seconds_without_prefix_index": round(seconds[False], 3), "prompt_tokens": tokens_in,
+        "prompt_tokens_taken_over": hits[True], "generated_tokens": 64 * requests,
+        "config": {"model": "%s-shaped, random weights N(0, 0.02)" % shape_name, "requests": requests,
+                   "shared_tokens": stem_len, "prefill_portion": 512, "context_len": context, "kv_block_size": BLOCK,
+                   "layers": config.num_hidden_layers, "sampling": "greedy"},
+    }))
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -110,9 +159,10 @@ def main():
     ap.add_argument("--shape", default="8b", choices=sorted(SHAPES))
     ap.add_argument("--prompt", type=int, default=2048, help="tokens every request holds when decoding starts")
     ap.add_argument("--context", type=int, default=8192, help="tokens of cache per request")
-    ap.add_argument("--workload", default="decode", choices=["decode", "continuous"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "prefix"],
                     help="continuous: 64 requests at once, prompts of 128 to 4,096 tokens, 64 to 512 generated "
-                         "tokens each, prompts in portions of 512 (its own JSON line; --steps and --warmup unused)")
+                         "tokens each, prompts in portions of 512 (its own JSON line; --steps and --warmup unused); "
+                         "prefix: 64 requests that share their first 2,048 tokens, with the prefix index on and off")
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 points")
     ap.add_argument("--skip-prefill", action="store_true",
                     help="skip the prefill measurement (for profiles of decoding alone; the line then has no value for it)")
@@ -156,6 +206,8 @@ def main():
 
     if args.workload == "continuous":
         return continuous(args, config, model, shape_name, gen, sync)
+    if args.workload == "prefix":
+        return shared_prefix(args, config, model, shape_name, gen, sync)
 
     # ---- prefill: one prompt of 2,048 tokens in one step ----
     engine = engine_for(1)

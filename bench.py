@@ -1,7 +1,7 @@
 """Decode and prefill throughput of the Qwen3-8B-shaped model on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L]
-                    [--shape 8b|14b|32b] [--prompt P] [--context C] [--workload decode|continuous|prefix]
+                    [--shape 8b|14b|32b] [--prompt P] [--context C] [--workload decode|continuous|prefix|products]
 
 Random bfloat16 weights, uniform-random prompts of 2,048 tokens, greedy decoding
 through the engine's own step loop (scheduler, step function, sampling). A
@@ -99,6 +99,56 @@ def continuous(args, config, model, shape_name, gen, sync):
     return 0
 
 
+def products(args, config, shape_name, sync):
+    """The four products of a layer at 2,048, 576 and 64 rows: the kernel that the contest
+    chose (library candidates and the hand-written tiled kernel, timed with cold caches) beside
+    every tile shape of the hand-written kernel, microseconds with the weight coming from
+    memory (three weights in turn)."""
+    import torch
+
+    from qwen3_from_scratch_amd import ops
+
+    c = config
+    shapes = [("qkv", (c.num_attention_heads + 2 * c.num_key_value_heads) * c.head_dim, c.hidden_size),
+              ("o", c.hidden_size, c.num_attention_heads * c.head_dim),
+              ("gate_up", 2 * c.intermediate_size, c.hidden_size), ("down", c.hidden_size, c.intermediate_size)]
+
+    def timed(f, n=10):
+        for _ in range(2):
+            f()
+        sync()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            f()
+        sync()
+        return (time.perf_counter() - t0) / n * 1e6
+
+    rows = {}
+    for M in (2048, 576, 64):
+        for name, N, K in shapes:
+            x = torch.randn(M, K, device="cuda:0").to(torch.bfloat16)
+            ws = [(torch.randn(N, K, device="cuda:0") * 0.02).to(torch.bfloat16) for _ in range(3)]
+            out = torch.empty(M, N, device="cuda:0", dtype=torch.bfloat16)
+            turn = [0]
+
+            def chosen():
+                turn[0] = (turn[0] + 1) % 3
+                ops.linear(x, ws[turn[0]], out=out)
+
+            entry = {"chosen_us": round(min(timed(chosen), timed(chosen)), 1), "plan": ops.matmul_plan(M, N, K),
+                     "us_at_1_pflops": round(2.0 * M * N * K / 1e9, 1)}
+            for shape in range(ops.gemm_tiles_configs()):
+                def own():
+                    turn[0] = (turn[0] + 1) % 3
+                    ops.gemm_tiles(x, ws[turn[0]], shape, out=out)
+                entry["tiles_%d_us" % shape] = round(min(timed(own), timed(own)), 1)
+            rows["%s_%d" % (name, M)] = entry
+            del ws
+    print(json.dumps({"metric": "products of a layer, microseconds, %s bf16" % shape_name, "unit": "us", "n_gpus": 1,
+                      "higher_is_better": False, "dtype": "bf16", "data": "synthetic", "products": rows}))
+    return 0
+
+
 def shared_prefix(args, config, model, shape_name, gen, sync):
     """64 requests that begin with the same 2,048 tokens (a system prompt, say) and go on with 32
     to 256 tokens of their own, 64 generated tokens each, with the prefix index on and off. Each
@@ -159,10 +209,12 @@ def main():
     ap.add_argument("--shape", default="8b", choices=sorted(SHAPES))
     ap.add_argument("--prompt", type=int, default=2048, help="tokens every request holds when decoding starts")
     ap.add_argument("--context", type=int, default=8192, help="tokens of cache per request")
-    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "prefix"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "prefix", "products"],
                     help="continuous: 64 requests at once, prompts of 128 to 4,096 tokens, 64 to 512 generated "
                          "tokens each, prompts in portions of 512 (its own JSON line; --steps and --warmup unused); "
-                         "prefix: 64 requests that share their first 2,048 tokens, with the prefix index on and off")
+                         "prefix: 64 requests that share their first 2,048 tokens, with the prefix index on and off; "
+                         "products: a layer's four products by the chosen kernel and by each tile shape of the "
+                         "hand-written one")
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 points")
     ap.add_argument("--skip-prefill", action="store_true",
                     help="skip the prefill measurement (for profiles of decoding alone; the line then has no value for it)")
@@ -188,6 +240,8 @@ def main():
     config = ModelConfig.from_dict(raw)
     itemsize = 2 if args.dtype == "bfloat16" else 4
     torch.cuda.set_device(0)
+    if args.workload == "products":
+        return products(args, config, shape_name, torch.cuda.synchronize)
     model = random_model(config, dtype=args.dtype, device="cuda:0", seed=0, std=0.02)
     gen = torch.Generator().manual_seed(1)
 

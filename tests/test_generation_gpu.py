@@ -139,3 +139,25 @@ def test_trace_run_program(model_folders, tmp_path, dtype):
             scale = max(1.0, float(logits.abs().max()))
             for p in range(logits.shape[0]):
                 assert float((got[(rid, p)] - logits[p]).abs().max()) <= tol * scale, (label, rid, p)
+
+
+def test_trace_run_answers_step_by_step(model_folders, tmp_path):
+    """The program reads a step, runs it, writes its file and prints `done <step>` before the
+    next step is sent; it exits with 0 when its input ends."""
+    out = str(tmp_path / "out")
+    proc = subprocess.Popen(
+        [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", model_folders["D"], "--dtype", "bfloat16",
+         "--out", out, "--max-tokens", "256"], stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
+    try:
+        for step in range(4):
+            record = {"step": step, "entries": [{"id": "a", "tokens": [5, 2, 3] if step == 0 else [step], "want": [0]}],
+                      "end": ["a"] if step == 3 else []}
+            proc.stdin.write(json.dumps(record) + "\n")
+            proc.stdin.flush()
+            assert proc.stdout.readline().strip() == "done %d" % step
+            assert os.path.getsize(os.path.join(out, "%d.f32" % step)) == 4 * TINY["D"]["config"]["vocab_size"]
+        proc.stdin.close()
+        assert proc.wait(timeout=60) == 0
+    finally:
+        if proc.poll() is None:
+            proc.kill()

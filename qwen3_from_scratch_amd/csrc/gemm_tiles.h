@@ -26,6 +26,10 @@
 // multiplied (385); copies through registers and ds_write (365); wavefront tiles of 128 x 128,
 // one wavefront a SIMD (364).
 //
+// A product with few tiles (576 x 4,096 x 12,288: 160 tiles of 128 x 128 on 256 CUs) shares K
+// out over several blocks per tile, whose float32 partial products a second kernel adds in a
+// fixed order.
+//
 // K must be a multiple of 64. Rows of x beyond M and of w beyond N are read from the last
 // valid row and never written. Blocks are numbered so that the eight XCDs each take a
 // contiguous run of tiles, M fastest: the blocks that share a slice of w run on one XCD at
@@ -119,7 +123,8 @@ __device__ inline void store_tile(const f32x4_t (&acc)[MI][NJ], OUT* __restrict_
 template <typename OUT, int EPI, int BM, int BN, int WM, int WN, int STAGES>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_tiles_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                          OUT* __restrict__ out, int M, int N, int K, int tiles_m,
-                                                         int tiles_total, int tiles_per_xcd) {
+                                                         int tiles_total, int tiles_per_xcd, int steps_per_split,
+                                                         float* __restrict__ partials) {
   typedef Shape<BM, BN, WM, WN, STAGES> S;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   // block -> tile: XCD x (blocks x, x + 8, ...) takes tiles [x * per, (x + 1) * per)
@@ -180,7 +185,9 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiles_kernel(const bf16_t* 
 #pragma unroll
     for (int j = 0; j < S::NJ; ++j) acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-  const int steps = K / BK;
+  // with K shared out over gridDim.y blocks, this one walks steps first .. first + steps - 1
+  const int first = blockIdx.y * steps_per_split;
+  const int steps = min(K / BK - first, steps_per_split);
   auto multiply_stage = [&](const unsigned char* st) {
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
@@ -201,24 +208,50 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiles_kernel(const bf16_t* 
   {
 #pragma unroll
     for (int ahead = 0; ahead < STAGES - 1; ++ahead)
-      if (ahead < steps) copy_step(ahead, ahead);
+      if (ahead < steps) copy_step(first + ahead, ahead);
     for (int kt = 0; kt < steps; ++kt) {
       // step kt has landed in every thread's view, and nobody still reads the stage that the
       // next copy overwrites (step kt - 1's)
       wait_for_step(min(kt + STAGES - 2, steps - 1) - kt);
       __syncthreads();
-      if (kt + STAGES - 1 < steps) copy_step(kt + STAGES - 1, (kt + STAGES - 1) % STAGES);
+      if (kt + STAGES - 1 < steps) copy_step(first + kt + STAGES - 1, (kt + STAGES - 1) % STAGES);
       multiply_stage(smem + (kt % STAGES) * S::STAGE_BYTES);
     }
   }
-  store_tile<OUT, EPI, S::MI, S::NJ>(acc, out, M, N, m0 + wm * (BM / WM), n0 + wn * (BN / WN), col, grp);
+  if (partials)   // a share of K: float32 sums for gemm_tiles_reduce_kernel
+    store_tile<float, EPI_PLAIN, S::MI, S::NJ>(acc, partials + (size_t)blockIdx.y * M * N, M, N, m0 + wm * (BM / WM),
+                                               n0 + wn * (BN / WN), col, grp);
+  else
+    store_tile<OUT, EPI, S::MI, S::NJ>(acc, out, M, N, m0 + wm * (BM / WM), n0 + wn * (BN / WN), col, grp);
+}
+
+// out = the sum of `splits` float32 partial products (each M x N, N a multiple of 4), added in the
+// splits' order: a fixed order of additions.
+template <typename OUT>
+__global__ __launch_bounds__(256) void gemm_tiles_reduce_kernel(const float* __restrict__ partials, OUT* __restrict__ out,
+                                                                size_t quads, int splits) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= quads) return;
+  float4 sum = reinterpret_cast<const float4*>(partials)[i];
+  for (int s = 1; s < splits; ++s) {
+    const float4 v = reinterpret_cast<const float4*>(partials)[(size_t)s * quads + i];
+    sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
+  }
+  if constexpr (sizeof(OUT) == 4)
+    reinterpret_cast<float4*>(out)[i] = sum;
+  else
+    reinterpret_cast<uint2*>(out)[i] = pack_bf16x4(f32x4_t{sum.x, sum.y, sum.z, sum.w});
 }
 
 // The tile shapes on offer: (BM, BN, STAGES).
 constexpr int NUM_CONFIGS = 5;
 
+// `splits` > 1: K is shared out over that many blocks per tile, which leave float32 partial
+// products in `partials` (splits x M x N floats) for a second kernel to add; plain epilogue
+// only, N a multiple of 4.
 template <typename OUT, int EPI, int BM, int BN, int WM, int WN, int STAGES>
-int launch_config(const void* x, const void* w, void* out, int M, int N, int K, hipStream_t stream) {
+int launch_config(const void* x, const void* w, void* out, int M, int N, int K, int splits, float* partials,
+                  hipStream_t stream) {
   typedef Shape<BM, BN, WM, WN, STAGES> S;
   static bool raised[16] = {};   // the dynamic shared-memory limit, once per device
   int device = 0;
@@ -234,19 +267,43 @@ int launch_config(const void* x, const void* w, void* out, int M, int N, int K, 
   const long total = (long)tiles_m * tiles_n;
   if (total > (1L << 28)) return Q3_ERR_UNSUPPORTED;
   const int per_xcd = (int)((total + 7) / 8);
-  hipLaunchKernelGGL(kernel, dim3(8 * per_xcd), dim3(S::THREADS), S::SMEM_BYTES, stream, (const bf16_t*)x, (const bf16_t*)w,
-                     (OUT*)out, M, N, K, tiles_m, (int)total, per_xcd);
+  const int steps = K / BK;
+  if (splits < 1 || splits > steps || splits > 64) return Q3_ERR_BAD_ARGUMENT;
+  if (splits > 1 && (EPI != EPI_PLAIN || N % 4 || partials == nullptr)) return Q3_ERR_BAD_ARGUMENT;
+  const int per_split = (steps + splits - 1) / splits;
+  const int used = (steps + per_split - 1) / per_split;     // no block without a step
+  hipLaunchKernelGGL(kernel, dim3(8 * per_xcd, used), dim3(S::THREADS), S::SMEM_BYTES, stream, (const bf16_t*)x,
+                     (const bf16_t*)w, (OUT*)out, M, N, K, tiles_m, (int)total, per_xcd, per_split,
+                     used > 1 ? partials : nullptr);
+  if (used > 1) {
+    const size_t quads = (size_t)M * N / 4;
+    hipLaunchKernelGGL(gemm_tiles_reduce_kernel<OUT>, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream,
+                       partials, (OUT*)out, quads, used);
+  }
   return q3_launch_status();
 }
 
+// The number of shares of K that fills the chip once for this size and tile shape (1: the
+// tiles alone do, or the steps are too few to share out).
+inline int splits_that_fill(int config, int M, int N, int K) {
+  const int bm = config < 2 ? 128 : 256, bn = config < 3 ? 128 : 256;
+  const int slots = config < 2 ? 512 : 256;                  // blocks resident at once on 256 CUs
+  const long tiles = (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
+  int splits = (int)(slots / tiles);
+  const int steps = K / BK;
+  while (splits > 1 && steps / splits < 8) --splits;           // a share keeps eight steps at least
+  return splits < 2 || N % 4 ? 1 : (splits > 16 ? 16 : splits);
+}
+
 template <typename OUT, int EPI>
-int launch(int config, const void* x, const void* w, void* out, int M, int N, int K, hipStream_t stream) {
+int launch(int config, const void* x, const void* w, void* out, int M, int N, int K, hipStream_t stream,
+           int splits = 1, float* partials = nullptr) {
   switch (config) {
-    case 0: return launch_config<OUT, EPI, 128, 128, 2, 2, 2>(x, w, out, M, N, K, stream);
-    case 1: return launch_config<OUT, EPI, 128, 128, 2, 2, 3>(x, w, out, M, N, K, stream);
-    case 2: return launch_config<OUT, EPI, 256, 128, 4, 2, 2>(x, w, out, M, N, K, stream);
-    case 3: return launch_config<OUT, EPI, 256, 256, 2, 4, 2>(x, w, out, M, N, K, stream);
-    case 4: return launch_config<OUT, EPI, 256, 256, 4, 2, 2>(x, w, out, M, N, K, stream);
+    case 0: return launch_config<OUT, EPI, 128, 128, 2, 2, 2>(x, w, out, M, N, K, splits, partials, stream);
+    case 1: return launch_config<OUT, EPI, 128, 128, 2, 2, 3>(x, w, out, M, N, K, splits, partials, stream);
+    case 2: return launch_config<OUT, EPI, 256, 128, 4, 2, 2>(x, w, out, M, N, K, splits, partials, stream);
+    case 3: return launch_config<OUT, EPI, 256, 256, 2, 4, 2>(x, w, out, M, N, K, splits, partials, stream);
+    case 4: return launch_config<OUT, EPI, 256, 256, 4, 2, 2>(x, w, out, M, N, K, splits, partials, stream);
   }
   return Q3_ERR_BAD_ARGUMENT;
 }

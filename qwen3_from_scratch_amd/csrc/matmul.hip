@@ -40,6 +40,7 @@ namespace {
 
 constexpr size_t WORKSPACE_BYTES = 128u << 20;
 constexpr size_t EVICT_BYTES = 512u << 20;     // twice the 256 MB last-level cache
+constexpr size_t PARTIALS_BYTES = 128u << 20;  // float32 partial products of the hand-written kernel's K shares
 constexpr int EVICT_BLOCKS = 2048, EVICT_THREADS = 256;
 constexpr int MAX_CANDIDATES = 64;
 
@@ -59,6 +60,7 @@ struct Plan {
   hipblasLtMatmulAlgo_t algo;
   bool tuned = false;
   int own = -1;            // the hand-written kernel's tile shape, if that was chosen; else `algo`
+  int own_splits = 1;      // and over how many blocks it shares K out
   int candidates = 0, chosen = 0;
   float first_us = 0.f, best_us = 0.f;
 };
@@ -67,6 +69,7 @@ struct Device {
   hipblasLtHandle_t handle = nullptr;
   void* workspace = nullptr;
   void* evict = nullptr;
+  float* partials = nullptr;
   hipEvent_t begin = nullptr, end = nullptr;
   std::map<std::tuple<int, int, int, int>, Plan> plans;
   // what was chosen for a size, by its rows rounded up to a multiple of 32: sizes beyond 64
@@ -82,9 +85,11 @@ std::map<int, Device> g_devices;
 int g_candidates = 16;
 enum { KERNELS_BOTH = 0, KERNELS_LIBRARY = 1, KERNELS_OWN = 2 };
 int g_kernels = KERNELS_BOTH;
-// the tile shapes that enter the contest (the other two never won a size of the 8B, 14B and 32B models)
+// the tile shapes that enter the contest (the other two never won a size of the 8B, 14B and 32B models);
+// the first two enter a second time with K shared out where their tiles alone would not fill the chip
 constexpr int OWN_CANDIDATES[] = {0, 2, 4};
 constexpr int NUM_OWN = sizeof(OWN_CANDIDATES) / sizeof(OWN_CANDIDATES[0]);
+constexpr int MAX_OWN = NUM_OWN + 2;
 
 #define HIP_TRY(call)                    \
   do {                                   \
@@ -119,10 +124,12 @@ void forget(Plan& p) {
   p = Plan();
 }
 
-int run_own(int config, const void* x, const void* w, void* out, int M, int N, int K, int out_dtype,
-            hipStream_t stream) {
-  return out_dtype == Q3_F32 ? tiles::launch<float, tiles::EPI_PLAIN>(config, x, w, out, M, N, K, stream)
-                             : tiles::launch<bf16_t, tiles::EPI_PLAIN>(config, x, w, out, M, N, K, stream);
+int run_own(Device& d, int config, int splits, const void* x, const void* w, void* out, int M, int N, int K,
+            int out_dtype, hipStream_t stream) {
+  if (splits > 1 && (!d.partials || (size_t)splits * M * N * sizeof(float) > PARTIALS_BYTES)) return Q3_ERR_UNSUPPORTED;
+  return out_dtype == Q3_F32
+             ? tiles::launch<float, tiles::EPI_PLAIN>(config, x, w, out, M, N, K, stream, splits, d.partials)
+             : tiles::launch<bf16_t, tiles::EPI_PLAIN>(config, x, w, out, M, N, K, stream, splits, d.partials);
 }
 
 hipblasStatus_t run(Device& d, const Plan& p, const hipblasLtMatmulAlgo_t& algo, const void* x, const void* w,
@@ -160,6 +167,7 @@ int choose(Device& d, Plan& p, const void* x, const void* w, void* out, int M, i
     p.candidates = 1;
     p.chosen = 0;
     p.own = OWN_CANDIDATES[0];
+    p.own_splits = 1;
     p.tuned = false;
     return 0;
   }
@@ -179,6 +187,7 @@ int choose(Device& d, Plan& p, const void* x, const void* w, void* out, int M, i
   p.candidates = got;
   p.chosen = 0;
   p.own = -1;
+  p.own_splits = 1;
   p.algo = found[0].algo;
   p.tuned = !capturing;
   if (capturing || (got == 1 && !own_takes)) return 0;
@@ -188,13 +197,27 @@ int choose(Device& d, Plan& p, const void* x, const void* w, void* out, int M, i
   }
   // two passes: all candidates briefly (the first run of each also loads its code), then those
   // near the front again and longer
-  // candidates got .. got + NUM_OWN - 1 are the hand-written kernel's tile shapes
-  const int all = got + (own_takes ? NUM_OWN : 0);
+  // candidates from `got` on are the hand-written kernel's: (tile shape, shares of K)
+  int own_config[MAX_OWN], own_splits[MAX_OWN], owns = 0;
+  if (own_takes) {
+    for (int i = 0; i < NUM_OWN; ++i) {
+      own_config[owns] = OWN_CANDIDATES[i];
+      own_splits[owns++] = 1;
+    }
+    for (int i = 0; i < 2; ++i) {
+      const int splits = tiles::splits_that_fill(OWN_CANDIDATES[i], M, N, K);
+      if (splits < 2 || (size_t)splits * M * N * sizeof(float) > PARTIALS_BYTES) continue;
+      if (!d.partials) HIP_TRY(hipMalloc((void**)&d.partials, PARTIALS_BYTES));
+      own_config[owns] = OWN_CANDIDATES[i];
+      own_splits[owns++] = splits;
+    }
+  }
+  const int all = got + owns;
   const int first = g_kernels == KERNELS_OWN && own_takes ? got : 0;
   auto time_one = [&](int i, int reps) {
     if (i < got) return time_candidate(d, p, found[i].algo, x, w, out, stream, reps);
     return time_runs(d, stream, reps, [&] {
-      return run_own(OWN_CANDIDATES[i - got], x, w, out, M, N, K, out_dtype, stream) == 0;
+      return run_own(d, own_config[i - got], own_splits[i - got], x, w, out, M, N, K, out_dtype, stream) == 0;
     });
   };
   std::vector<float> us(all, -1.f);
@@ -218,7 +241,8 @@ int choose(Device& d, Plan& p, const void* x, const void* w, void* out, int M, i
   if (chosen < got) {
     p.algo = found[chosen].algo;
   } else {
-    p.own = OWN_CANDIDATES[chosen - got];
+    p.own = own_config[chosen - got];
+    p.own_splits = own_splits[chosen - got];
   }
   p.first_us = us[first];
   p.best_us = us[chosen];
@@ -228,7 +252,7 @@ int choose(Device& d, Plan& p, const void* x, const void* w, void* out, int M, i
 // The product by the plan's kernel.
 int run_plan(Device& d, const Plan& p, const void* x, const void* w, void* out, int M, int N, int K, int out_dtype,
              hipStream_t stream) {
-  if (p.own >= 0) return run_own(p.own, x, w, out, M, N, K, out_dtype, stream);
+  if (p.own >= 0) return run_own(d, p.own, p.own_splits, x, w, out, M, N, K, out_dtype, stream);
   const hipblasStatus_t s = run(d, p, p.algo, x, w, out, stream);
   return s == HIPBLAS_STATUS_SUCCESS ? 0 : Q3_ERR_LIBRARY + (int)s;
 }
@@ -240,18 +264,29 @@ int run_plan(Device& d, const Plan& p, const void* x, const void* w, void* out, 
 // interleave gate and up, out (M, N / 2) bfloat16 = silu(gate) * up.
 extern "C" int q3_gemm_tiles_configs() { return tiles::NUM_CONFIGS; }
 
+// `splits` > 1 (plain epilogue, N a multiple of 4): K is shared out over that many blocks per tile and
+// `partials` (splits * M * N floats) takes their partial products; q3_gemm_tiles_splits says how many fill the
+// chip once.
+extern "C" int q3_gemm_tiles_splits(int config, int M, int N, int K) {
+  return tiles::takes(M, N, K) && config >= 0 && config < tiles::NUM_CONFIGS ? tiles::splits_that_fill(config, M, N, K)
+                                                                            : 1;
+}
+
 extern "C" int q3_gemm_tiles(const void* x, const void* w, void* out, int M, int N, int K, int out_dtype,
-                             int epilogue, int config, void* stream_) {
+                             int epilogue, int config, int splits, float* partials, void* stream_) {
   if (!x || !w || !out || !tiles::takes(M, N, K)) return Q3_ERR_BAD_ARGUMENT;
   hipStream_t stream = (hipStream_t)stream_;
   std::lock_guard<std::mutex> hold(g_lock);   // the launchers keep a per-device flag
   if (epilogue == tiles::EPI_SWIGLU) {
     if (out_dtype != Q3_BF16 || N % 2) return Q3_ERR_BAD_ARGUMENT;
+    if (splits != 1) return Q3_ERR_BAD_ARGUMENT;
     return tiles::launch<bf16_t, tiles::EPI_SWIGLU>(config, x, w, out, M, N, K, stream);
   }
   if (epilogue != tiles::EPI_PLAIN) return Q3_ERR_BAD_ARGUMENT;
-  if (out_dtype == Q3_F32) return tiles::launch<float, tiles::EPI_PLAIN>(config, x, w, out, M, N, K, stream);
-  if (out_dtype == Q3_BF16) return tiles::launch<bf16_t, tiles::EPI_PLAIN>(config, x, w, out, M, N, K, stream);
+  if (out_dtype == Q3_F32)
+    return tiles::launch<float, tiles::EPI_PLAIN>(config, x, w, out, M, N, K, stream, splits, partials);
+  if (out_dtype == Q3_BF16)
+    return tiles::launch<bf16_t, tiles::EPI_PLAIN>(config, x, w, out, M, N, K, stream, splits, partials);
   return Q3_ERR_BAD_ARGUMENT;
 }
 
@@ -275,7 +310,8 @@ extern "C" int q3_matmul_set_kernels(int mode) {
 
 // What was chosen for a size on the current device: info[0] candidates timed, info[1] index chosen,
 // info[2] microseconds of the first candidate, info[3] of the chosen one, info[4] the hand-written kernel's
-// tile shape if that was chosen, else -1. Returns 1 if the size is known.
+// tile shape if that was chosen, else -1, info[5] over how many blocks it shares K out. Returns 1 if the size
+// is known.
 extern "C" int q3_matmul_plan(int M, int N, int K, int out_dtype, float* info) {
   std::lock_guard<std::mutex> hold(g_lock);
   int device = 0;
@@ -289,6 +325,7 @@ extern "C" int q3_matmul_plan(int M, int N, int K, int out_dtype, float* info) {
   info[2] = p->second.first_us;
   info[3] = p->second.best_us;
   info[4] = (float)p->second.own;
+  info[5] = (float)p->second.own_splits;
   return 1;
 }
 
@@ -323,6 +360,7 @@ extern "C" int q3_matmul(const void* x, const void* w, void* out, int M, int N, 
     auto near = d.chosen_near.find(near_key);
     if (near != d.chosen_near.end()) {   // a neighbour's choice, if the library takes it for this size
       p.own = near->second.own;
+      p.own_splits = near->second.own_splits;
       p.algo = near->second.algo;
       if (run_plan(d, p, x, w, out, M, N, K, out_dtype, stream) == 0) {
         p.candidates = near->second.candidates;
@@ -344,6 +382,7 @@ extern "C" int q3_matmul(const void* x, const void* w, void* out, int M, int N, 
       Plan& kept = d.chosen_near[near_key];   // the choice only: the descriptors stay with their size
       kept.algo = p.algo;
       kept.own = p.own;
+      kept.own_splits = p.own_splits;
       kept.candidates = p.candidates;
       kept.chosen = p.chosen;
       kept.first_us = p.first_us;

@@ -35,6 +35,7 @@ __all__ = [
     "matmul_kernels",
     "gemm_tiles",
     "gemm_tiles_configs",
+    "gemm_tiles_splits",
     "matmul_plan",
     "tile_weight",
     "sample",
@@ -95,11 +96,12 @@ def matmul_kernels(which):
 def matmul_plan(M, N, K, out_dtype=torch.bfloat16):
     """What was chosen for a size on the current device, or None if it has not been met:
     (candidates timed, index chosen, microseconds of the first candidate, of the chosen one,
-    the hand-written kernel's tile shape if that was chosen, else -1)."""
-    info = (ctypes.c_float * 5)()
+    the hand-written kernel's tile shape if that was chosen, else -1, and over how many blocks
+    it shares K out)."""
+    info = (ctypes.c_float * 6)()
     if not library("matmul").q3_matmul_plan(int(M), int(N), int(K), _DT[out_dtype], info):
         return None
-    return int(info[0]), int(info[1]), float(info[2]), float(info[3]), int(info[4])
+    return int(info[0]), int(info[1]), float(info[2]), float(info[3]), int(info[4]), int(info[5])
 
 
 def gemm_tiles_configs():
@@ -107,10 +109,18 @@ def gemm_tiles_configs():
     return int(library("matmul").q3_gemm_tiles_configs())
 
 
-def gemm_tiles(x, weight, config=0, out_dtype=None, swiglu=False, out=None):
+def gemm_tiles_splits(config, M, N, K):
+    """Over how many blocks per tile the tiled product would share K out so that the chip is
+    filled once (1: its tiles alone do)."""
+    return int(library("matmul").q3_gemm_tiles_splits(int(config), int(M), int(N), int(K)))
+
+
+def gemm_tiles(x, weight, config=0, out_dtype=None, swiglu=False, out=None, splits=1):
     """The hand-written tiled matrix-core product alone, with tile shape `config`: x (M, K) and
     weight (N, K) bfloat16, K a multiple of 64; out (M, N) bfloat16 or float32, or with `swiglu`
-    (weight rows interleave gate and up) out (M, N / 2) bfloat16 = silu(gate) * up."""
+    (weight rows interleave gate and up) out (M, N / 2) bfloat16 = silu(gate) * up. With
+    `splits` > 1 (not with swiglu; N a multiple of 4) K is shared out over that many blocks per
+    tile and their float32 partial products are added by a second kernel."""
     _dev(x, weight, out)
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1], "x (M, K) and weight (N, K)")
     _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "x and weight must be bfloat16")
@@ -121,12 +131,16 @@ def gemm_tiles(x, weight, config=0, out_dtype=None, swiglu=False, out=None):
     out_dtype = out_dtype or torch.bfloat16
     _need(out_dtype in _DT and not (swiglu and (out_dtype != torch.bfloat16 or N % 2)),
           "out is bfloat16 or float32; with swiglu bfloat16 and an even number of weight rows")
+    _need(1 <= splits <= min(64, K // 64) and (splits == 1 or (not swiglu and N % 4 == 0)),
+          "K is shared out over 1 to min(64, K / 64) blocks, not with swiglu, N a multiple of 4")
     shape = (M, N // 2) if swiglu else (M, N)
     if out is None:
         out = torch.empty(shape, dtype=out_dtype, device=x.device)
     _need(out.shape == shape and out.dtype == out_dtype, "out must be %s of out_dtype" % (shape,))
+    partials = torch.empty((splits * M * N,), dtype=torch.float32, device=x.device) if splits > 1 else None
     _check(library("matmul").q3_gemm_tiles(_ptr(x), _ptr(weight), _ptr(out), M, N, K, _DT[out_dtype],
-                                           1 if swiglu else 0, int(config), _stream()), "gemm_tiles")
+                                           1 if swiglu else 0, int(config), int(splits), _ptr(partials), _stream()),
+           "gemm_tiles")
     return out
 
 

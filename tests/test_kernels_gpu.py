@@ -464,7 +464,7 @@ def test_linear_many_rows_first_met_in_a_graph():
 
 
 @pytest.mark.parametrize("M,N,K", [(200, 304, 128), (513, 1000, 192), (77, 48, 64), (17, 2, 64), (300, 331, 4096),
-                                   (1024, 1536, 1024)])
+                                   (1024, 1536, 1024), (150, 260, 640)])
 def test_tiled_product_every_shape_and_epilogue(M, N, K):
     """The hand-written tiled matrix-core product: every tile shape, at sizes whose rows and
     columns end inside a tile, against a float64 product; float32 and bfloat16 outputs and the
@@ -490,8 +490,18 @@ def test_tiled_product_every_shape_and_epilogue(M, N, K):
         other = x.clone()
         other[1:] = _rand((M - 1, K), torch.bfloat16, 53)
         assert torch.equal(ops.gemm_tiles(other, w, config)[0], got16[0])
+        # K shared out over several blocks per tile, their partial products added by a second kernel
+        for splits in (2, 3, 5):
+            if K // 64 >= splits and N % 4 == 0:
+                shared = ops.gemm_tiles(x, w, config, out_dtype=torch.float32, splits=splits)
+                torch.testing.assert_close(shared.double(), want, rtol=1e-4, atol=1e-4)
+                shared16 = ops.gemm_tiles(x, w, config, splits=splits)
+                torch.testing.assert_close(shared16.double(), want, rtol=1.6e-2, atol=1e-2)
+                assert torch.equal(ops.gemm_tiles(other, w, config, splits=splits)[0], shared16[0])
     with pytest.raises(ops.OperandError):
         ops.gemm_tiles(x[:, :K - 8].contiguous(), w[:, :K - 8].contiguous())      # K no multiple of 64
+    with pytest.raises(ops.OperandError):
+        ops.gemm_tiles(x, w, 0, splits=K // 64 + 1)
 
 
 def test_linear_many_rows_by_the_hand_written_kernel_alone():
@@ -527,6 +537,14 @@ def test_linear_many_rows_by_the_hand_written_kernel_alone():
             torch.testing.assert_close(out.double(), x2.double() @ w.double().T, rtol=1.6e-2, atol=1e-2)
             assert torch.equal(ops.linear(x2, w), out)
         assert ops.matmul_plan(M2, N, K)[4] >= 0
+        # few tiles and many steps: the shapes that share K out stand in the contest too
+        M4, N4, K4 = 300, 512, 4096
+        assert ops.gemm_tiles_splits(0, M4, N4, K4) > 1
+        x4, w4 = _rand((M4, K4), torch.bfloat16, 59), _rand((N4, K4), torch.bfloat16, 60, scale=0.05)
+        torch.testing.assert_close(ops.linear(x4, w4, out_dtype=torch.float32).double(), x4.double() @ w4.double().T,
+                                   rtol=1e-4, atol=1e-4)
+        plan4 = ops.matmul_plan(M4, N4, K4, torch.float32)
+        assert plan4[0] == 5 and plan4[4] >= 0 and plan4[5] >= 1
         # an inner size it does not take goes to the library
         x3, w3 = _rand((40, 72), torch.bfloat16, 57), _rand((96, 72), torch.bfloat16, 58, scale=0.05)
         torch.testing.assert_close(ops.linear(x3, w3, out_dtype=torch.float32).double(), x3.double() @ w3.double().T,

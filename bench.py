@@ -137,7 +137,7 @@ def products(args, config, shape_name, sync):
         return (time.perf_counter() - t0) / (replays * calls) * 1e6
 
     rows = {}
-    for M in (2048, 576, 64):
+    for M in [int(m) for m in __import__("os").environ.get("Q3_ROWS", "2048,576,64").split(",")]:
         for name, N, K in shapes:
             x = torch.randn(M, K, device="cuda:0").to(torch.bfloat16)
             copies = max(3, -(-600_000_000 // (N * K * 2)))    # more than the 256 MB cache holds, in turn

@@ -244,7 +244,7 @@ __global__ __launch_bounds__(256) void gemm_tiles_reduce_kernel(const float* __r
 }
 
 // The tile shapes on offer: (BM, BN, STAGES).
-constexpr int NUM_CONFIGS = 5;
+constexpr int NUM_CONFIGS = 8;
 
 // `splits` > 1: K is shared out over that many blocks per tile, which leave float32 partial
 // products in `partials` (splits x M x N floats) for a second kernel to add; plain epilogue
@@ -286,8 +286,11 @@ int launch_config(const void* x, const void* w, void* out, int M, int N, int K, 
 // The number of shares of K that fills the chip once for this size and tile shape (1: the
 // tiles alone do, or the steps are too few to share out).
 inline int splits_that_fill(int config, int M, int N, int K) {
-  const int bm = config < 2 ? 128 : 256, bn = config < 3 ? 128 : 256;
-  const int slots = config < 2 ? 512 : 256;                  // blocks resident at once on 256 CUs
+  // tile rows, tile columns, blocks resident at once on 256 CUs (what shared memory allows)
+  static const int shape[NUM_CONFIGS][3] = {{128, 128, 512}, {128, 128, 256}, {256, 128, 256}, {256, 256, 256},
+                                            {256, 256, 256}, {64, 128, 512}, {64, 128, 768}, {64, 256, 512}};
+  if (config < 0 || config >= NUM_CONFIGS) return 1;
+  const int bm = shape[config][0], bn = shape[config][1], slots = shape[config][2];
   const long tiles = (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
   int splits = (int)(slots / tiles);
   const int steps = K / BK;
@@ -304,6 +307,9 @@ int launch(int config, const void* x, const void* w, void* out, int M, int N, in
     case 2: return launch_config<OUT, EPI, 256, 128, 4, 2, 2>(x, w, out, M, N, K, splits, partials, stream);
     case 3: return launch_config<OUT, EPI, 256, 256, 2, 4, 2>(x, w, out, M, N, K, splits, partials, stream);
     case 4: return launch_config<OUT, EPI, 256, 256, 4, 2, 2>(x, w, out, M, N, K, splits, partials, stream);
+    case 5: return launch_config<OUT, EPI, 64, 128, 1, 4, 3>(x, w, out, M, N, K, splits, partials, stream);
+    case 6: return launch_config<OUT, EPI, 64, 128, 1, 4, 2>(x, w, out, M, N, K, splits, partials, stream);
+    case 7: return launch_config<OUT, EPI, 64, 256, 1, 8, 2>(x, w, out, M, N, K, splits, partials, stream);
   }
   return Q3_ERR_BAD_ARGUMENT;
 }

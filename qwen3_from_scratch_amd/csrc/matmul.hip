@@ -85,11 +85,20 @@ std::map<int, Device> g_devices;
 int g_candidates = 16;
 enum { KERNELS_BOTH = 0, KERNELS_LIBRARY = 1, KERNELS_OWN = 2 };
 int g_kernels = KERNELS_BOTH;
-// the tile shapes that enter the contest (the other two never won a size of the 8B, 14B and 32B models);
-// the first two enter a second time with K shared out where their tiles alone would not fill the chip
-constexpr int OWN_CANDIDATES[] = {0, 2, 4};
-constexpr int NUM_OWN = sizeof(OWN_CANDIDATES) / sizeof(OWN_CANDIDATES[0]);
-constexpr int MAX_OWN = NUM_OWN + 2;
+// The tile shapes that enter the contest, by the product's rows (the others never won a size of the 8B, 14B
+// and 32B models there): small tiles with three stages where the weights' passage bounds the product, the
+// largest where the matrix units do. Each enters a second time with K shared out where its tiles alone would
+// not fill the chip.
+constexpr int OWN_FEW_ROWS[] = {1, 5}, OWN_SOME_ROWS[] = {0, 1, 2}, OWN_MANY_ROWS[] = {0, 2, 4};
+constexpr int MAX_OWN = 6;
+inline const int* own_shapes(int M, int& count) {
+  if (M <= 256) {
+    count = 2;
+    return OWN_FEW_ROWS;
+  }
+  count = 3;
+  return M <= 1024 ? OWN_SOME_ROWS : OWN_MANY_ROWS;
+}
 
 #define HIP_TRY(call)                    \
   do {                                   \
@@ -166,7 +175,8 @@ int choose(Device& d, Plan& p, const void* x, const void* w, void* out, int M, i
   if (own_takes && g_kernels == KERNELS_OWN && capturing) {   // untimed: the first shape, timed at the next eager call
     p.candidates = 1;
     p.chosen = 0;
-    p.own = OWN_CANDIDATES[0];
+    int count = 0;
+    p.own = own_shapes(M, count)[0];
     p.own_splits = 1;
     p.tuned = false;
     return 0;
@@ -200,15 +210,15 @@ int choose(Device& d, Plan& p, const void* x, const void* w, void* out, int M, i
   // candidates from `got` on are the hand-written kernel's: (tile shape, shares of K)
   int own_config[MAX_OWN], own_splits[MAX_OWN], owns = 0;
   if (own_takes) {
-    for (int i = 0; i < NUM_OWN; ++i) {
-      own_config[owns] = OWN_CANDIDATES[i];
+    int count = 0;
+    const int* shapes = own_shapes(M, count);
+    for (int i = 0; i < count; ++i) {
+      own_config[owns] = shapes[i];
       own_splits[owns++] = 1;
-    }
-    for (int i = 0; i < 2; ++i) {
-      const int splits = tiles::splits_that_fill(OWN_CANDIDATES[i], M, N, K);
+      const int splits = tiles::splits_that_fill(shapes[i], M, N, K);
       if (splits < 2 || (size_t)splits * M * N * sizeof(float) > PARTIALS_BYTES) continue;
       if (!d.partials) HIP_TRY(hipMalloc((void**)&d.partials, PARTIALS_BYTES));
-      own_config[owns] = OWN_CANDIDATES[i];
+      own_config[owns] = shapes[i];
       own_splits[owns++] = splits;
     }
   }

@@ -544,7 +544,7 @@ def test_linear_many_rows_by_the_hand_written_kernel_alone():
         torch.testing.assert_close(ops.linear(x4, w4, out_dtype=torch.float32).double(), x4.double() @ w4.double().T,
                                    rtol=1e-4, atol=1e-4)
         plan4 = ops.matmul_plan(M4, N4, K4, torch.float32)
-        assert plan4[0] == 5 and plan4[4] >= 0 and plan4[5] >= 1
+        assert plan4[0] >= 4 and plan4[4] >= 0 and plan4[5] >= 1
         # an inner size it does not take goes to the library
         x3, w3 = _rand((40, 72), torch.bfloat16, 57), _rand((96, 72), torch.bfloat16, 58, scale=0.05)
         torch.testing.assert_close(ops.linear(x3, w3, out_dtype=torch.float32).double(), x3.double() @ w3.double().T,

@@ -16,11 +16,13 @@
 // kernels that are the fastest only while the weight sits in that cache.
 //
 // The hand-written tiled kernel (gemm_tiles.h) stands in the same contest: where it takes a
-// size (K a multiple of 64) three of its tile shapes are timed after the library's candidates,
-// and a size goes to whichever kernel was the fastest. q3_matmul_set_kernels narrows the
+// size (K a multiple of 64) two or three of its tile shapes, chosen by the rows, are timed after
+// the library's candidates, each also with K shared out over several blocks per tile where its
+// tiles alone would not fill the chip, and a size goes to whichever kernel was the fastest. q3_matmul_set_kernels narrows the
 // contest to the library's kernels alone, or to the hand-written ones where they take the size.
 //
-// One workspace and one such buffer per device, allocated at first need and kept. Calls on one
+// One workspace, one such buffer and one buffer for the hand-written kernel's partial products
+// per device, allocated at first need and kept. Calls on one
 // device share it and the plans: they are serialised by a lock and are meant
 // to come from one stream at a time.
 

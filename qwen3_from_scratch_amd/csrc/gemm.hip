@@ -148,6 +148,9 @@ struct SkinnyFusion {
   float* sums_out;
 };
 
+#ifndef SKINNY_PAIR_SLABS
+#define SKINNY_PAIR_SLABS 384   // from this many slabs on, and with more than eight rows of x, two slabs share a block
+#endif
 #define SKINNY_PRE 4  // float4 loads of partial sums a thread has in flight beside the main loop's
 
 template <typename OUT, int EPI, bool TILED, bool SCALED>
@@ -310,6 +313,143 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
   }
 }
 
+// Two slabs per block from the tile-ordered copy: a wavefront's rows of x (the second operand)
+// serve two matrix instructions, so a block reads x once for 32 weight rows instead of 16.
+// With 8 to 16 rows of x the one-slab kernel moves as many bytes of x out of the L2 as weights
+// out of memory, and that passage, about 7 TB/s over all CUs, is what bounds it (8, 12 and 16
+// rows of the 8B layer's products: 85, 97 and 109 us; reading x from several copies changes
+// nothing, so it is the volume, not a hot address). With pairs the gate/up product takes 41.6,
+// 42.6 and 44.3 us at 8, 12 and 16 rows (one slab a block: 40.7, 46.1, 51.1) and the q/k/v
+// product 13.1, 14.8, 15.8 (13.5, 15.7, 17.7): used with more than eight rows, where the pairs
+// still give most CUs a block (384 slabs or more). Epilogues: plain and SwiGLU.
+#define PAIR_PRE 2  // fewer partial sums in flight than the one-slab kernel: the registers go to the second slab
+template <typename OUT, int EPI, bool SCALED>
+__global__ __launch_bounds__(512, 4) void gemm_skinny_pair_kernel(const bf16_t* __restrict__ x,
+                                                               const bf16_t* __restrict__ w, OUT* __restrict__ out,
+                                                               int M, int N, int K, int kw, int k_per_wave,
+                                                               SkinnyFusion fu) {
+  static_assert(EPI == EPI_PLAIN || EPI == EPI_SWIGLU, "plain and SwiGLU epilogues");
+  extern __shared__ float red[];  // [waves][2][64][4], then [waves][16] for the rows' sums
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = lane & 15, grp = lane >> 4;
+  const int nwaves = blockDim.x >> 6;      // = kw: the block's wavefronts share K
+  const int slabs = (N + 15) / 16;
+  const int slab0 = 2 * blockIdx.x;
+  const bool second = slab0 + 1 < slabs;
+  const int k_begin = wave * k_per_wave;
+  const int k_end = min(K, k_begin + k_per_wave);
+  f32x4_t acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+
+  constexpr bool scaled = SCALED;
+  float4 pre[PAIR_PRE];
+  if (scaled) {
+    const int q = threadIdx.x & 3, i0 = threadIdx.x >> 2, stride = blockDim.x >> 2;
+#pragma unroll
+    for (int u = 0; u < PAIR_PRE; ++u) {
+      const int i = i0 + u * stride;
+      pre[u] = i < fu.sums_rows ? reinterpret_cast<const float4*>(fu.row_sums)[i * 4 + q] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+  }
+  const bool x_ok = col < M;
+  const size_t slab_elems = (size_t)(K / 32) * 512;
+  const bf16_t* wp0 = w + (size_t)slab0 * slab_elems + lane * 8;
+  const bf16_t* wp1 = second ? wp0 + slab_elems : wp0;
+  const bf16_t* xp = x + (size_t)(x_ok ? col : 0) * K + 8 * grp;
+  for (int k = k_begin; k < k_end; k += 32 * SKINNY_U) {
+    Pack16 a0[SKINNY_U], a1[SKINNY_U], b[SKINNY_U];
+#pragma unroll
+    for (int u = 0; u < SKINNY_U; ++u) {
+      const int kk = k + 32 * u;
+      const bool k_ok = kk + 8 * grp + 8 <= k_end;
+      a0[u].u = k_ok ? *reinterpret_cast<const uint4*>(wp0 + (size_t)(kk / 32) * 512) : make_uint4(0, 0, 0, 0);
+      a1[u].u = k_ok ? *reinterpret_cast<const uint4*>(wp1 + (size_t)(kk / 32) * 512) : make_uint4(0, 0, 0, 0);
+      b[u].u = (x_ok && k_ok) ? *reinterpret_cast<const uint4*>(xp + kk) : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int u = 0; u < SKINNY_U; ++u) {
+      acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0[u].v, b[u].v, acc[0], 0, 0, 0);
+      acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1[u].v, b[u].v, acc[1], 0, 0, 0);
+    }
+  }
+  float* sums = red + (size_t)nwaves * 512;
+  if (scaled) {
+    float4 s = pre[0];
+#pragma unroll
+    for (int u = 1; u < PAIR_PRE; ++u) {
+      s.x += pre[u].x; s.y += pre[u].y; s.z += pre[u].z; s.w += pre[u].w;
+    }
+    const int q = threadIdx.x & 3, stride = blockDim.x >> 2;
+    for (int i = (threadIdx.x >> 2) + PAIR_PRE * stride; i < fu.sums_rows; i += stride) {
+      const float4 v = reinterpret_cast<const float4*>(fu.row_sums)[i * 4 + q];
+      s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+    }
+#pragma unroll
+    for (int off = 4; off < 64; off <<= 1) {
+      s.x += __shfl_xor(s.x, off, 64); s.y += __shfl_xor(s.y, off, 64);
+      s.z += __shfl_xor(s.z, off, 64); s.w += __shfl_xor(s.w, off, 64);
+    }
+    if (lane < 4) *reinterpret_cast<float4*>(sums + wave * 16 + 4 * lane) = s;
+  }
+  if (nwaves > 1) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) red[((wave * 2 + h) * 64 + lane) * 4 + j] = acc[h][j];
+  }
+  if (nwaves > 1 || scaled) __syncthreads();
+  if (wave != 0) return;
+  // the wavefronts' sums in their order, as the one-slab kernel adds them
+  for (int s = 1; s < nwaves; ++s)
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[h][j] += red[((s * 2 + h) * 64 + lane) * 4 + j];
+  if (scaled) {
+    float total = 0.f;
+    for (int wv = 0; wv < nwaves; ++wv) total += sums[wv * 16 + col];
+    const float r = rsqrtf(total * fu.inv_width + fu.eps);
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[h][j] *= r;
+  }
+  if (col >= M) return;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    if (h == 1 && !second) break;
+    const int n = (slab0 + h) * 16 + 4 * grp;
+    if constexpr (EPI == EPI_SWIGLU) {
+      OUT* o = out + (size_t)col * (N / 2) + n / 2;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        if (n + 2 * j + 1 < N) {
+          const float g = to_float(from_float<OUT>(acc[h][2 * j])), u = to_float(from_float<OUT>(acc[h][2 * j + 1]));
+          o[j] = from_float<OUT>(g / (1.f + expf(-g)) * u);
+        }
+      }
+    } else {
+      OUT* o = out + (size_t)col * N + n;
+      if (n + 3 < N && (N % 4) == 0) {
+        if constexpr (sizeof(OUT) == 4) {
+          *reinterpret_cast<float4*>(o) = make_float4(acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
+        } else {
+          union {
+            uint2 u;
+            bf16_t e[4];
+          } pk;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) pk.e[j] = float_to_bf16(acc[h][j]);
+          *reinterpret_cast<uint2*>(o) = pk.u;
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (n + j < N) o[j] = from_float<OUT>(acc[h][j]);
+      }
+    }
+  }
+}
+
 template <typename OUT, int EPI, bool TILED = false, bool SCALED = false>
 static int launch_skinny(const void* x, const void* w, void* out, int M, int N, int K, hipStream_t stream,
                          SkinnyFusion fu = SkinnyFusion{}) {
@@ -326,6 +466,14 @@ static int launch_skinny(const void* x, const void* w, void* out, int M, int N, 
   const int step = 32 * SKINNY_U;
   int k_per_wave = (K + kw - 1) / kw;
   k_per_wave = (k_per_wave + step - 1) / step * step;
+  if constexpr (TILED && (EPI == EPI_PLAIN || EPI == EPI_SWIGLU)) {
+    if (slabs >= SKINNY_PAIR_SLABS && sw == 1 && M > 8) {
+      const size_t pair_smem = (size_t)kw * (2 * 64 * 4 + 16) * sizeof(float);
+      hipLaunchKernelGGL((gemm_skinny_pair_kernel<OUT, EPI, SCALED>), dim3((slabs + 1) / 2), dim3(64 * kw), pair_smem,
+                         stream, (const bf16_t*)x, (const bf16_t*)w, (OUT*)out, M, N, K, kw, k_per_wave, fu);
+      return q3_launch_status();
+    }
+  }
   const int blocks = (slabs + sw - 1) / sw;
   const size_t smem = (size_t)sw * kw * (64 * 4 + 16) * sizeof(float);
   hipLaunchKernelGGL((gemm_skinny_kernel<OUT, EPI, TILED, SCALED>), dim3(blocks), dim3(64 * sw * kw), smem, stream,

@@ -555,10 +555,13 @@ def test_linear_many_rows_by_the_hand_written_kernel_alone():
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 6144, 4096), (8, 4096, 12288), (16, 1000, 96), (3, 331, 64), (9, 24, 2048),
-                                   (5, 151936, 256)])
+                                   (5, 151936, 256), (12, 6144, 4096), (16, 24576, 512), (9, 6168, 160),
+                                   (13, 6150, 4096)])
 def test_linear_from_the_tiled_copy(M, N, K):
     """The tile-ordered copy gives the very sums of the row-major kernel: the same numbers
-    are added in the same order, only their addresses differ."""
+    are added in the same order, only their addresses differ. That holds for the kernel that
+    gives two slabs to a block too (more than eight rows, 384 slabs or more; also with an odd
+    number of slabs and a last slab that is not whole)."""
     ops = _ops()
     x = _rand((M, K), torch.bfloat16, 23)
     w = _rand((N, K), torch.bfloat16, 24, scale=0.05)
@@ -592,7 +595,8 @@ def test_linear_swiglu(dtype, M, I, K):
 
 @pytest.mark.parametrize("norm_dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("M,H,K,N2", [(1, 4096, 4096, 6144), (8, 4096, 12288, 24576), (16, 96, 224, 160),
-                                      (5, 992, 64, 330), (3, 32, 32, 48)])
+                                      (5, 992, 64, 330), (3, 32, 32, 48), (12, 4096, 1024, 24576),
+                                      (16, 1024, 512, 6152)])
 def test_linear_residual_norm_and_unscaled_rows(M, H, K, N2, norm_dtype):
     """A product that adds itself into the residual stream and prepares the next norm, and the
     product after it, which applies the norm's division: together they give what the product,

@@ -77,20 +77,36 @@ __device__ inline uint2 pack_bf16x4(f32x4_t c) {
   return pk.u;
 }
 
+// The rows of x may still lack the factor of the norm before this product: they hold
+// stream * norm_weight, and `sums` (chunks, rows) holds the rows' sums of squares of the stream in
+// partial sums of column chunks (tiles_residual_kernel leaves them so). Row m of the product is
+// then multiplied by rsqrt(sum_m * inv_width + eps): (x / rms) @ W^T = (x @ W^T) / rms.
+struct RowScale {
+  const float* sums = nullptr;
+  int chunks = 0, rows = 0;
+  float eps = 0.f, inv_width = 0.f;
+  __device__ float of(int m) const {
+    float total = 0.f;
+    for (int c = 0; c < chunks; ++c) total += sums[(size_t)c * rows + m];   // in the chunks' order
+    return rsqrtf(total * inv_width + eps);
+  }
+};
+
 // A wavefront's outputs to memory: lane (col, grp) of block (i, j) holds out[m][n .. n + 3] with
 // m = m_base + 16 i + col, n = n_base + 16 j + 4 grp.
 template <typename OUT, int EPI, int MI, int NJ>
 __device__ inline void store_tile(const f32x4_t (&acc)[MI][NJ], OUT* __restrict__ out, int M, int N, int m_base,
-                                  int n_base, int col, int grp) {
+                                  int n_base, int col, int grp, const RowScale& scale = RowScale()) {
 #pragma unroll
   for (int i = 0; i < MI; ++i) {
     const int m = m_base + 16 * i + col;
     if (m >= M) continue;
+    const float r = scale.sums ? scale.of(m) : 1.f;
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
       const int n = n_base + 16 * j + 4 * grp;
       if (n >= N) continue;
-      const f32x4_t c = acc[i][j];
+      const f32x4_t c = acc[i][j] * r;
       if constexpr (EPI == EPI_SWIGLU) {
         // rows of w interleave gate and up (row 2 i gate, row 2 i + 1 up); both are rounded to
         // the activation type first, as a separate activation kernel would have read them
@@ -124,7 +140,7 @@ template <typename OUT, int EPI, int BM, int BN, int WM, int WN, int STAGES>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_tiles_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                          OUT* __restrict__ out, int M, int N, int K, int tiles_m,
                                                          int tiles_total, int tiles_per_xcd, int steps_per_split,
-                                                         float* __restrict__ partials) {
+                                                         float* __restrict__ partials, RowScale scale) {
   typedef Shape<BM, BN, WM, WN, STAGES> S;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   // block -> tile: XCD x (blocks x, x + 8, ...) takes tiles [x * per, (x + 1) * per)
@@ -222,14 +238,16 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiles_kernel(const bf16_t* 
     store_tile<float, EPI_PLAIN, S::MI, S::NJ>(acc, partials + (size_t)blockIdx.y * M * N, M, N, m0 + wm * (BM / WM),
                                                n0 + wn * (BN / WN), col, grp);
   else
-    store_tile<OUT, EPI, S::MI, S::NJ>(acc, out, M, N, m0 + wm * (BM / WM), n0 + wn * (BN / WN), col, grp);
+    store_tile<OUT, EPI, S::MI, S::NJ>(acc, out, M, N, m0 + wm * (BM / WM), n0 + wn * (BN / WN), col, grp, scale);
 }
 
 // out = the sum of `splits` float32 partial products (each M x N, N a multiple of 4), added in the
-// splits' order: a fixed order of additions.
-template <typename OUT>
+// splits' order: a fixed order of additions. With `scale`, row m is multiplied by its factor
+// (see RowScale); with SWIGLU the columns are (gate, up) pairs and out is (M, N / 2).
+template <typename OUT, bool SWIGLU>
 __global__ __launch_bounds__(256) void gemm_tiles_reduce_kernel(const float* __restrict__ partials, OUT* __restrict__ out,
-                                                                size_t quads, int splits) {
+                                                                size_t quads, int quads_per_row, int splits,
+                                                                RowScale scale) {
   const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= quads) return;
   float4 sum = reinterpret_cast<const float4*>(partials)[i];
@@ -237,21 +255,77 @@ __global__ __launch_bounds__(256) void gemm_tiles_reduce_kernel(const float* __r
     const float4 v = reinterpret_cast<const float4*>(partials)[(size_t)s * quads + i];
     sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
   }
-  if constexpr (sizeof(OUT) == 4)
+  if (scale.sums) {
+    const float r = scale.of((int)(i / quads_per_row));
+    sum.x *= r; sum.y *= r; sum.z *= r; sum.w *= r;
+  }
+  if constexpr (SWIGLU) {
+    // both rounded to the activation type first, as a separate activation kernel would have read them
+    const float g0 = to_float(from_float<OUT>(sum.x)), u0 = to_float(from_float<OUT>(sum.y));
+    const float g1 = to_float(from_float<OUT>(sum.z)), u1 = to_float(from_float<OUT>(sum.w));
+    OUT* o = out + 2 * i;
+    o[0] = from_float<OUT>(g0 / (1.f + expf(-g0)) * u0);
+    o[1] = from_float<OUT>(g1 / (1.f + expf(-g1)) * u1);
+  } else if constexpr (sizeof(OUT) == 4) {
     reinterpret_cast<float4*>(out)[i] = sum;
-  else
+  } else {
     reinterpret_cast<uint2*>(out)[i] = pack_bf16x4(f32x4_t{sum.x, sum.y, sum.z, sum.w});
+  }
+}
+
+// The product as a residual stream's next addend, with the next norm prepared: the sum of the
+// partial products is rounded to bfloat16 (what a separate addition would have read), added
+// into `residual` (M, N) float32 in place, (residual * norm_weight) goes to `values` as
+// bfloat16, and the row's sum of squares over this block's 1,024 columns to sums[chunk][row].
+// Grid (chunks of 1,024 columns, rows), 256 threads, four columns a thread; N a multiple of 4.
+constexpr int CHUNK_COLUMNS = 1024;
+template <typename NW>
+__global__ __launch_bounds__(256) void tiles_residual_kernel(const float* __restrict__ partials, int splits,
+                                                             float* __restrict__ residual,
+                                                             const NW* __restrict__ norm_weight,
+                                                             bf16_t* __restrict__ values, float* __restrict__ sums,
+                                                             int M, int N) {
+  __shared__ float scratch[17];
+  const int m = blockIdx.y, n = blockIdx.x * CHUNK_COLUMNS + 4 * threadIdx.x;
+  float ss = 0.f;
+  if (n < N) {
+    const size_t at = (size_t)m * N + n;
+    float4 sum = *reinterpret_cast<const float4*>(partials + at);
+    for (int s = 1; s < splits; ++s) {
+      const float4 v = *reinterpret_cast<const float4*>(partials + (size_t)s * M * N + at);
+      sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
+    }
+    float4 r = *reinterpret_cast<const float4*>(residual + at);
+    r.x += bf16_to_float(float_to_bf16(sum.x)); r.y += bf16_to_float(float_to_bf16(sum.y));
+    r.z += bf16_to_float(float_to_bf16(sum.z)); r.w += bf16_to_float(float_to_bf16(sum.w));
+    *reinterpret_cast<float4*>(residual + at) = r;
+    union {
+      uint2 u;
+      bf16_t e[4];
+    } pk;
+    pk.e[0] = float_to_bf16(r.x * to_float(norm_weight[n]));
+    pk.e[1] = float_to_bf16(r.y * to_float(norm_weight[n + 1]));
+    pk.e[2] = float_to_bf16(r.z * to_float(norm_weight[n + 2]));
+    pk.e[3] = float_to_bf16(r.w * to_float(norm_weight[n + 3]));
+    *reinterpret_cast<uint2*>(values + at) = pk.u;
+    ss = r.x * r.x + r.y * r.y + r.z * r.z + r.w * r.w;
+  }
+  const float total = block_sum(ss, scratch);
+  if (threadIdx.x == 0) sums[(size_t)blockIdx.x * M + m] = total;
 }
 
 // The tile shapes on offer: (BM, BN, STAGES).
 constexpr int NUM_CONFIGS = 8;
 
 // `splits` > 1: K is shared out over that many blocks per tile, which leave float32 partial
-// products in `partials` (splits x M x N floats) for a second kernel to add; plain epilogue
-// only, N a multiple of 4.
+// products in `partials` (splits x M x N floats) for a second kernel to add, which also applies
+// the epilogue; N a multiple of 4.
+// `keep_partials`: the partial products (also a single one) stay in `partials` for the caller's
+// own second kernel. `scale`: see RowScale.
 template <typename OUT, int EPI, int BM, int BN, int WM, int WN, int STAGES>
 int launch_config(const void* x, const void* w, void* out, int M, int N, int K, int splits, float* partials,
-                  hipStream_t stream) {
+                  hipStream_t stream, const RowScale& scale = RowScale(), bool keep_partials = false,
+                  int* splits_used = nullptr) {
   typedef Shape<BM, BN, WM, WN, STAGES> S;
   static bool raised[16] = {};   // the dynamic shared-memory limit, once per device
   int device = 0;
@@ -269,16 +343,18 @@ int launch_config(const void* x, const void* w, void* out, int M, int N, int K, 
   const int per_xcd = (int)((total + 7) / 8);
   const int steps = K / BK;
   if (splits < 1 || splits > steps || splits > 64) return Q3_ERR_BAD_ARGUMENT;
-  if (splits > 1 && (EPI != EPI_PLAIN || N % 4 || partials == nullptr)) return Q3_ERR_BAD_ARGUMENT;
+  if ((splits > 1 || keep_partials) && (N % 4 || partials == nullptr)) return Q3_ERR_BAD_ARGUMENT;
   const int per_split = (steps + splits - 1) / splits;
   const int used = (steps + per_split - 1) / per_split;     // no block without a step
+  const bool to_partials = used > 1 || keep_partials;
   hipLaunchKernelGGL(kernel, dim3(8 * per_xcd, used), dim3(S::THREADS), S::SMEM_BYTES, stream, (const bf16_t*)x,
                      (const bf16_t*)w, (OUT*)out, M, N, K, tiles_m, (int)total, per_xcd, per_split,
-                     used > 1 ? partials : nullptr);
-  if (used > 1) {
+                     to_partials ? partials : nullptr, to_partials ? RowScale() : scale);
+  if (splits_used) *splits_used = used;
+  if (to_partials && !keep_partials) {
     const size_t quads = (size_t)M * N / 4;
-    hipLaunchKernelGGL(gemm_tiles_reduce_kernel<OUT>, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream,
-                       partials, (OUT*)out, quads, used);
+    hipLaunchKernelGGL((gemm_tiles_reduce_kernel<OUT, EPI == EPI_SWIGLU>), dim3((unsigned)((quads + 255) / 256)),
+                       dim3(256), 0, stream, partials, (OUT*)out, quads, N / 4, used, scale);
   }
   return q3_launch_status();
 }
@@ -300,16 +376,17 @@ inline int splits_that_fill(int config, int M, int N, int K) {
 
 template <typename OUT, int EPI>
 int launch(int config, const void* x, const void* w, void* out, int M, int N, int K, hipStream_t stream,
-           int splits = 1, float* partials = nullptr) {
+           int splits = 1, float* partials = nullptr, const RowScale& scale = RowScale(), bool keep_partials = false,
+           int* splits_used = nullptr) {
   switch (config) {
-    case 0: return launch_config<OUT, EPI, 128, 128, 2, 2, 2>(x, w, out, M, N, K, splits, partials, stream);
-    case 1: return launch_config<OUT, EPI, 128, 128, 2, 2, 3>(x, w, out, M, N, K, splits, partials, stream);
-    case 2: return launch_config<OUT, EPI, 256, 128, 4, 2, 2>(x, w, out, M, N, K, splits, partials, stream);
-    case 3: return launch_config<OUT, EPI, 256, 256, 2, 4, 2>(x, w, out, M, N, K, splits, partials, stream);
-    case 4: return launch_config<OUT, EPI, 256, 256, 4, 2, 2>(x, w, out, M, N, K, splits, partials, stream);
-    case 5: return launch_config<OUT, EPI, 64, 128, 1, 4, 3>(x, w, out, M, N, K, splits, partials, stream);
-    case 6: return launch_config<OUT, EPI, 64, 128, 1, 4, 2>(x, w, out, M, N, K, splits, partials, stream);
-    case 7: return launch_config<OUT, EPI, 64, 256, 1, 8, 2>(x, w, out, M, N, K, splits, partials, stream);
+    case 0: return launch_config<OUT, EPI, 128, 128, 2, 2, 2>(x, w, out, M, N, K, splits, partials, stream, scale, keep_partials, splits_used);
+    case 1: return launch_config<OUT, EPI, 128, 128, 2, 2, 3>(x, w, out, M, N, K, splits, partials, stream, scale, keep_partials, splits_used);
+    case 2: return launch_config<OUT, EPI, 256, 128, 4, 2, 2>(x, w, out, M, N, K, splits, partials, stream, scale, keep_partials, splits_used);
+    case 3: return launch_config<OUT, EPI, 256, 256, 2, 4, 2>(x, w, out, M, N, K, splits, partials, stream, scale, keep_partials, splits_used);
+    case 4: return launch_config<OUT, EPI, 256, 256, 4, 2, 2>(x, w, out, M, N, K, splits, partials, stream, scale, keep_partials, splits_used);
+    case 5: return launch_config<OUT, EPI, 64, 128, 1, 4, 3>(x, w, out, M, N, K, splits, partials, stream, scale, keep_partials, splits_used);
+    case 6: return launch_config<OUT, EPI, 64, 128, 1, 4, 2>(x, w, out, M, N, K, splits, partials, stream, scale, keep_partials, splits_used);
+    case 7: return launch_config<OUT, EPI, 64, 256, 1, 8, 2>(x, w, out, M, N, K, splits, partials, stream, scale, keep_partials, splits_used);
   }
   return Q3_ERR_BAD_ARGUMENT;
 }

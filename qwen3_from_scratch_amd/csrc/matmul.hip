@@ -78,6 +78,8 @@ struct Device {
   // rows that differ only within such a step take the choice of the first one that was timed
   // (a serving loop meets dozens of them, a prompt's portion plus however many requests decode)
   std::map<std::tuple<int, int, int, int>, Plan> chosen_near;
+  // (kind, M, N, K) -> (tile shape, shares of K) of the products that carry a norm (q3_tiles_*)
+  std::map<std::tuple<int, int, int, int>, std::pair<int, int>> fused;
 };
 
 int rows_class(int M) { return M <= 64 ? M : (M + 31) / 32 * 32; }
@@ -269,7 +271,137 @@ int run_plan(Device& d, const Plan& p, const void* x, const void* w, void* out, 
   return s == HIPBLAS_STATUS_SUCCESS ? 0 : Q3_ERR_LIBRARY + (int)s;
 }
 
+// Tile shape and shares of K for a product of 17 to 64 rows that carries a norm. `kind` tells the
+// variants apart (0 plain, 1 SwiGLU, 2 residual); `launch(config, splits)` runs one without
+// side effects and returns its status. Timed once per size with cold caches outside a graph
+// capture; a capture that meets a new size takes the rule of thumb and leaves the timing to the
+// next eager call.
+template <typename Launch>
+int choose_fused(Device& d, int kind, int M, int N, int K, hipStream_t stream, Launch launch, int& config, int& splits) {
+  const auto key = std::make_tuple(kind, M, N, K);
+  auto known = d.fused.find(key);
+  if (known != d.fused.end()) {
+    config = known->second.first;
+    splits = known->second.second;
+    return 0;
+  }
+  int configs[4], shares[4], n = 0;
+  for (int shape : OWN_FEW_ROWS) {   // the 64 x 256 tiles lose here too (gate/up at 64 rows: 67 us against 51)
+    const int fill = tiles::splits_that_fill(shape, M, N, K);
+    if (fill > 1 && (size_t)fill * M * N * sizeof(float) <= PARTIALS_BYTES) {
+      configs[n] = shape;
+      shares[n++] = fill;
+    }
+    configs[n] = shape;
+    shares[n++] = 1;
+  }
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  HIP_TRY(hipStreamIsCapturing(stream, &capture));
+  if (!d.partials) {
+    if (capture != hipStreamCaptureStatusNone) return (int)hipErrorStreamCaptureUnsupported;
+    HIP_TRY(hipMalloc((void**)&d.partials, PARTIALS_BYTES));
+  }
+  config = configs[0];
+  splits = shares[0];
+  if (capture != hipStreamCaptureStatusNone) return 0;
+  if (!d.begin) {
+    HIP_TRY(hipEventCreate(&d.begin));
+    HIP_TRY(hipEventCreate(&d.end));
+  }
+  if (!d.evict) {
+    HIP_TRY(hipMalloc(&d.evict, EVICT_BYTES));
+    HIP_TRY(hipMemsetAsync(d.evict, 0, EVICT_BYTES, stream));
+  }
+  float best = -1.f;
+  for (int i = 0; i < n; ++i) {
+    auto one = [&] { return launch(configs[i], shares[i]) == 0; };
+    if (time_runs(d, stream, 1, one) < 0.f) continue;   // the first run also loads the code
+    const float us = time_runs(d, stream, 4, one);
+    if (us > 0.f && (best < 0.f || us < best)) {
+      best = us;
+      config = configs[i];
+      splits = shares[i];
+    }
+  }
+  if (best < 0.f) return Q3_ERR_UNSUPPORTED;
+  d.fused[key] = std::make_pair(config, splits);
+  return 0;
+}
+
 }  // namespace
+
+// Products of 17 to 64 rows that carry a norm, by the hand-written tiled kernel (the few-row kernel of
+// gemm.hip does the same for up to 16 rows). x (M, K) and w (N, K) bfloat16, K a multiple of 64, N of 4.
+//
+// q3_tiles_scaled: the rows of x hold stream * norm_weight and still lack the norm's division; `sums`
+// (chunks, M) float32 holds the rows' sums of squares of the stream in partial sums, `width` the stream's
+// width (= K). out = (x @ w^T) * rsqrt(sum / width + eps) row by row: epilogue 0 gives (M, N) in `out_dtype`,
+// 1 (rows of w interleave gate and up) gives (M, N / 2) bfloat16 = silu(gate) * up.
+extern "C" int q3_tiles_scaled(const void* x, const void* w, void* out, int M, int N, int K, int out_dtype,
+                               int epilogue, const float* sums, int chunks, float eps, int width, void* stream_) {
+  if (!x || !w || !out || !sums || M < 1 || M > 64 || N % 4 || !tiles::takes(M, N, K)) return Q3_ERR_BAD_ARGUMENT;
+  if (chunks < 1 || width != K) return Q3_ERR_BAD_ARGUMENT;
+  const bool swiglu = epilogue == tiles::EPI_SWIGLU;
+  if (!swiglu && epilogue != tiles::EPI_PLAIN) return Q3_ERR_BAD_ARGUMENT;
+  if (swiglu ? out_dtype != Q3_BF16 : (out_dtype != Q3_BF16 && out_dtype != Q3_F32)) return Q3_ERR_BAD_ARGUMENT;
+  hipStream_t stream = (hipStream_t)stream_;
+  std::lock_guard<std::mutex> hold(g_lock);
+  int device = 0;
+  HIP_TRY(hipGetDevice(&device));
+  Device& d = g_devices[device];
+  tiles::RowScale scale;
+  scale.sums = sums;
+  scale.chunks = chunks;
+  scale.rows = M;
+  scale.eps = eps;
+  scale.inv_width = 1.f / (float)width;
+  auto launch = [&](int config, int splits) {
+    if (swiglu)
+      return tiles::launch<bf16_t, tiles::EPI_SWIGLU>(config, x, w, out, M, N, K, stream, splits, d.partials, scale);
+    if (out_dtype == Q3_F32)
+      return tiles::launch<float, tiles::EPI_PLAIN>(config, x, w, out, M, N, K, stream, splits, d.partials, scale);
+    return tiles::launch<bf16_t, tiles::EPI_PLAIN>(config, x, w, out, M, N, K, stream, splits, d.partials, scale);
+  };
+  int config = 0, splits = 1;
+  const int status = choose_fused(d, swiglu ? 1 : 0, M, N, K, stream, launch, config, splits);
+  return status ? status : launch(config, splits);
+}
+
+// q3_tiles_residual: residual (M, N) float32 += bfloat16(x @ w^T) in place; values (M, N) bfloat16 =
+// residual * norm_weight; sums (ceil(N / 1024), M) float32 = the rows' sums of squares of the new residual over
+// chunks of 1,024 columns: what q3_tiles_scaled takes for the next product.
+extern "C" int q3_tiles_residual_chunks(int N) { return (N + tiles::CHUNK_COLUMNS - 1) / tiles::CHUNK_COLUMNS; }
+
+extern "C" int q3_tiles_residual(const void* x, const void* w, int M, int N, int K, float* residual,
+                                 const void* norm_weight, int norm_weight_dtype, void* values, float* sums,
+                                 void* stream_) {
+  if (!x || !w || !residual || !norm_weight || !values || !sums) return Q3_ERR_BAD_ARGUMENT;
+  if (M < 1 || M > 64 || N % 4 || !tiles::takes(M, N, K)) return Q3_ERR_BAD_ARGUMENT;
+  if (norm_weight_dtype != Q3_BF16 && norm_weight_dtype != Q3_F32) return Q3_ERR_BAD_ARGUMENT;
+  hipStream_t stream = (hipStream_t)stream_;
+  std::lock_guard<std::mutex> hold(g_lock);
+  int device = 0;
+  HIP_TRY(hipGetDevice(&device));
+  Device& d = g_devices[device];
+  int config = 0, splits = 1;
+  // timed by the product into `values`, which the real run overwrites: the residual is not touched
+  int status = choose_fused(d, 2, M, N, K, stream, [&](int c, int s) {
+    return tiles::launch<bf16_t, tiles::EPI_PLAIN>(c, x, w, values, M, N, K, stream, s, d.partials);
+  }, config, splits);
+  if (status) return status;
+  int used = 1;
+  status = tiles::launch<bf16_t, tiles::EPI_PLAIN>(config, x, w, values, M, N, K, stream, splits, d.partials,
+                                                   tiles::RowScale(), true, &used);
+  if (status) return status;
+  const dim3 grid(q3_tiles_residual_chunks(N), M);
+  if (norm_weight_dtype == Q3_F32)
+    hipLaunchKernelGGL(tiles::tiles_residual_kernel<float>, grid, dim3(256), 0, stream, d.partials, used, residual,
+                       (const float*)norm_weight, (bf16_t*)values, sums, M, N);
+  else
+    hipLaunchKernelGGL(tiles::tiles_residual_kernel<bf16_t>, grid, dim3(256), 0, stream, d.partials, used, residual,
+                       (const bf16_t*)norm_weight, (bf16_t*)values, sums, M, N);
+  return q3_launch_status();
+}
 
 // The hand-written tiled kernel alone (gemm_tiles.h), tile shape `config` (0 .. q3_gemm_tiles_configs() - 1):
 // x (M, K) and w (N, K) bfloat16, K a multiple of 64; `epilogue` 0: out (M, N) in `out_dtype`; 1: rows of w
@@ -291,8 +423,7 @@ extern "C" int q3_gemm_tiles(const void* x, const void* w, void* out, int M, int
   std::lock_guard<std::mutex> hold(g_lock);   // the launchers keep a per-device flag
   if (epilogue == tiles::EPI_SWIGLU) {
     if (out_dtype != Q3_BF16 || N % 2) return Q3_ERR_BAD_ARGUMENT;
-    if (splits != 1) return Q3_ERR_BAD_ARGUMENT;
-    return tiles::launch<bf16_t, tiles::EPI_SWIGLU>(config, x, w, out, M, N, K, stream);
+    return tiles::launch<bf16_t, tiles::EPI_SWIGLU>(config, x, w, out, M, N, K, stream, splits, partials);
   }
   if (epilogue != tiles::EPI_PLAIN) return Q3_ERR_BAD_ARGUMENT;
   if (out_dtype == Q3_F32)
@@ -355,8 +486,10 @@ extern "C" int q3_matmul(const void* x, const void* w, void* out, int M, int N, 
   if (!d.handle) {
     if (capturing) return (int)hipErrorStreamCaptureUnsupported;   // the first call on a device allocates
     HIP_TRY(hipMalloc(&d.workspace, WORKSPACE_BYTES));
-    HIP_TRY(hipEventCreate(&d.begin));
-    HIP_TRY(hipEventCreate(&d.end));
+    if (!d.begin) {
+      HIP_TRY(hipEventCreate(&d.begin));
+      HIP_TRY(hipEventCreate(&d.end));
+    }
     LT_TRY(hipblasLtCreate(&d.handle));
   }
   Plan& p = d.plans[std::make_tuple(M, N, K, out_dtype)];

@@ -119,8 +119,8 @@ def gemm_tiles(x, weight, config=0, out_dtype=None, swiglu=False, out=None, spli
     """The hand-written tiled matrix-core product alone, with tile shape `config`: x (M, K) and
     weight (N, K) bfloat16, K a multiple of 64; out (M, N) bfloat16 or float32, or with `swiglu`
     (weight rows interleave gate and up) out (M, N / 2) bfloat16 = silu(gate) * up. With
-    `splits` > 1 (not with swiglu; N a multiple of 4) K is shared out over that many blocks per
-    tile and their float32 partial products are added by a second kernel."""
+    `splits` > 1 (N a multiple of 4) K is shared out over that many blocks per tile and their
+    float32 partial products are added by a second kernel, which then also applies the activation."""
     _dev(x, weight, out)
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1], "x (M, K) and weight (N, K)")
     _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "x and weight must be bfloat16")
@@ -131,8 +131,8 @@ def gemm_tiles(x, weight, config=0, out_dtype=None, swiglu=False, out=None, spli
     out_dtype = out_dtype or torch.bfloat16
     _need(out_dtype in _DT and not (swiglu and (out_dtype != torch.bfloat16 or N % 2)),
           "out is bfloat16 or float32; with swiglu bfloat16 and an even number of weight rows")
-    _need(1 <= splits <= min(64, K // 64) and (splits == 1 or (not swiglu and N % 4 == 0)),
-          "K is shared out over 1 to min(64, K / 64) blocks, not with swiglu, N a multiple of 4")
+    _need(1 <= splits <= min(64, K // 64) and (splits == 1 or N % 4 == 0),
+          "K is shared out over 1 to min(64, K / 64) blocks, and then N is a multiple of 4")
     shape = (M, N // 2) if swiglu else (M, N)
     if out is None:
         out = torch.empty(shape, dtype=out_dtype, device=x.device)
@@ -452,6 +452,30 @@ def _row_sums_args(unscaled, M, K):
     return _ptr(sums), sums.shape[0], ctypes.c_float(eps), int(width)
 
 
+FUSED_ROWS_FEW, FUSED_ROWS_MOST = 16, 64
+
+
+def fused_rows_take(weight, M):
+    """Whether the tiled kernel carries a norm for `M` rows of a product with `weight` (N, K):
+    more rows than the few-row kernel takes, at most 64, bfloat16, K a multiple of 64 and N of 4."""
+    return (FUSED_ROWS_FEW < M <= FUSED_ROWS_MOST and weight.dtype == torch.bfloat16 and weight.dim() == 2
+            and weight.shape[1] % 64 == 0 and weight.shape[0] % 4 == 0 and weight.is_contiguous())
+
+
+def _tiles_scaled(x, weight, out, unscaled, swiglu, what):
+    sums, eps, width = unscaled
+    M, K = x.shape
+    _dev(sums)
+    _need(sums.dtype == torch.float32 and sums.dim() == 2 and sums.shape[1] == M and sums.shape[0] > 0
+          and sums.is_contiguous(), "row sums must be float32 (chunks, M)")
+    _need(width == K, "the rows' width must be the product's inner size")
+    _need(x.is_contiguous() and out.is_contiguous(), "operands must be contiguous")
+    _check(library("matmul").q3_tiles_scaled(
+        _ptr(x), _ptr(weight), _ptr(out), M, weight.shape[0], K, _DT[out.dtype], 1 if swiglu else 0, _ptr(sums),
+        sums.shape[0], ctypes.c_float(eps), int(width), _stream()), what)
+    return out
+
+
 def linear(x, weight, out_dtype=None, out=None, tiled=None, unscaled=None):
     """out = x @ weight^T with float32 accumulation. x (M, K), weight (N, K).
     `tiled` is `tile_weight(weight)`, if the caller keeps one: few rows are then served from it.
@@ -479,7 +503,10 @@ def linear(x, weight, out_dtype=None, out=None, tiled=None, unscaled=None):
             _ptr(x), _ptr(tiled), _ptr(out), M, N, K, _DT[out_dtype], 0, sums, sums_rows, eps, width,
             None, None, 0, None, _stream()), "linear")
         return out
-    _need(unscaled is None, "unscaled rows need the few-row kernel: bfloat16, at most 16 rows, a tiled weight")
+    if unscaled is not None and x.dtype == torch.bfloat16 and fused_rows_take(weight, M):
+        return _tiles_scaled(x, weight, out, unscaled, False, "linear")
+    _need(unscaled is None, "unscaled rows need bfloat16 and at most 16 rows with a tiled weight, or 17 to 64 rows "
+          "with an inner size that is a multiple of 64")
     if M and x.dtype == torch.bfloat16 and not library("gemm").q3_linear_is_skinny(M, N, K, 1):
         # bfloat16 products with many rows go to the vendor library (hipBLASLt), as the
         # reference's engine uses its vendor library for them; accumulation is float32.
@@ -520,7 +547,11 @@ def linear_swiglu(x, weight, tiled=None, unscaled=None):
             _ptr(x), _ptr(tiled), _ptr(out), M, N, K, 1, 1, sums, sums_rows, eps, width,
             None, None, 0, None, _stream()), "linear_swiglu")
         return out
-    _need(unscaled is None, "unscaled rows need the few-row kernel: bfloat16, at most 16 rows, a tiled weight")
+    if unscaled is not None and x.dtype == torch.bfloat16 and fused_rows_take(weight, M):
+        out = torch.empty((M, N // 2), dtype=x.dtype, device=x.device)
+        return _tiles_scaled(x, weight, out, unscaled, True, "linear_swiglu")
+    _need(unscaled is None, "unscaled rows need bfloat16 and at most 16 rows with a tiled weight, or 17 to 64 rows "
+          "with an inner size that is a multiple of 64")
     if M and library("gemm").q3_linear_is_skinny(M, N, K, _DT[x.dtype]):
         out = torch.empty((M, N // 2), dtype=x.dtype, device=x.device)
         _check(library("gemm").q3_linear_swiglu(_ptr(x), _ptr(weight), _ptr(out), M, N, K, _DT[x.dtype], _stream()),
@@ -539,17 +570,29 @@ def linear_residual_norm(x, weight, tiled, residual, norm_weight):
     float32, the rows' sums of squares of the new residual in partial sums of 16 columns (row m
     of the stream in column m). The norm's result is values * rsqrt(sum / N + eps) row by row;
     `linear` and `linear_swiglu` apply that factor to their products when given
-    `unscaled=(sums, eps, N)`."""
+    `unscaled=(sums, eps, N)`.
+
+    With 17 to 64 rows (`fused_rows_take`; `tiled` is not used) the tiled kernel's partial
+    products are added by a second kernel that does the same; sums is then (ceil(N / 1024), M),
+    partial sums over 1,024 columns, row m of the stream in column m."""
     _dev(x, weight, tiled, residual, norm_weight)
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1], "x (M, K) and weight (N, K)")
     M, K = x.shape
     N = weight.shape[0]
-    _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and _tiled_ok(tiled, weight, M) and N % 16 == 0,
-          "bfloat16, 1 to 16 rows, a tiled weight and a width that is a multiple of 16")
     _need(residual.shape == (M, N) and residual.dtype == torch.float32 and residual.is_contiguous(),
           "residual must be float32 (M, N)")
     _need(norm_weight.shape == (N,) and norm_weight.dtype in _DT and norm_weight.is_contiguous(), "norm weight (N,)")
     values = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    if x.dtype == torch.bfloat16 and fused_rows_take(weight, M):
+        _need(x.is_contiguous(), "x must be contiguous")
+        lib = library("matmul")
+        sums = torch.empty((lib.q3_tiles_residual_chunks(N), M), dtype=torch.float32, device=x.device)
+        _check(lib.q3_tiles_residual(
+            _ptr(x), _ptr(weight), M, N, K, _ptr(residual), _ptr(norm_weight), _DT[norm_weight.dtype], _ptr(values),
+            _ptr(sums), _stream()), "linear_residual_norm")
+        return values, sums
+    _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and _tiled_ok(tiled, weight, M) and N % 16 == 0,
+          "bfloat16, 1 to 16 rows, a tiled weight and a width that is a multiple of 16")
     sums = torch.empty((N // 16, 16), dtype=torch.float32, device=x.device)
     _check(library("gemm").q3_linear_tiled(
         _ptr(x), _ptr(tiled), _ptr(values), M, N, K, 1, 2, None, 0, ctypes.c_float(0.0), 0,

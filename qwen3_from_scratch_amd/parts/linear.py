@@ -32,15 +32,19 @@ class LinearWeight:
 
     @property
     def fuses(self):
-        """Whether steps of at most 16 rows go through the few-row kernel, whose
-        epilogues carry the norm fusion: UnscaledRows in, a NormSink out."""
-        return self.tiled is not None
+        """Whether steps of few rows go through kernels whose epilogues carry the
+        norm fusion, UnscaledRows in, a NormSink out: up to 16 rows the few-row
+        kernel on the tiled copy, up to 64 the tiled matrix-core kernel. A
+        reader of UnscaledRows must have output rows in steps of 4."""
+        return self.tiled is not None and self.weight.shape[0] % 4 == 0
 
     def forward_into(self, x, sink):
         """x @ W^T added into the sink's residual and prepared for its norm, as
-        UnscaledRows; or, where the kernel does not take the case, returned."""
+        UnscaledRows; or, where the kernels do not take the case, returned."""
         norm = sink.norm
-        if not self.fuses or x.shape[0] > 16 or self.weight.shape[0] % 16:
+        rows = x.shape[0]
+        if self.tiled is None or not (ops.fused_rows_take(self.weight, rows) if rows > ops.FUSED_ROWS_FEW
+                                      else self.weight.shape[0] % 16 == 0):
             return self.forward(x)
         values, sums = ops.linear_residual_norm(x, self.weight, self.tiled, sink.residual, norm.weight)
         return UnscaledRows(values, sums, norm.eps, norm.size)

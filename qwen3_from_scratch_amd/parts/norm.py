@@ -38,9 +38,11 @@ class RMSNorm(Part):
     def sink_for(self, x):
         """A NormSink for the residual `x` if this step may have the addition
         and this norm fused into the neighbouring products (bfloat16 with
-        tiled matrices, at most 16 rows), else None."""
-        if self.precision.act != torch.bfloat16 or not self.precision.tiled or not 1 <= x.shape[0] <= 16:
+        tiled matrices; at most 16 rows and a width in steps of 16, or up to
+        64 rows and a width in steps of 64), else None."""
+        rows = x.shape[0]
+        if self.precision.act != torch.bfloat16 or not self.precision.tiled or self.weight is None:
             return None
-        if self.size % 16 or self.weight is None:
+        if not 1 <= rows <= ops.FUSED_ROWS_MOST or self.size % (16 if rows <= ops.FUSED_ROWS_FEW else 64):
             return None
         return NormSink(x, self)

@@ -647,6 +647,60 @@ def test_linear_residual_norm_and_unscaled_rows(M, H, K, N2, norm_dtype):
         ops.linear(values, w2, unscaled=(sums, eps, H))
 
 
+@pytest.mark.parametrize("norm_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,H,K,N2", [(17, 4096, 4096, 6144), (64, 4096, 12288, 24576), (40, 1024, 512, 6152),
+                                      (33, 192, 64, 332), (64, 5120, 3200, 1000), (25, 1088, 17408, 128)])
+def test_linear_residual_norm_and_unscaled_rows_beyond_sixteen(M, H, K, N2, norm_dtype):
+    """The same pair of fusions for 17 to 64 rows, where the tiled kernel carries them: its
+    partial products go through a second kernel that adds them into the stream, and the next
+    product's epilogue (or the kernel that adds its partial products) divides by the rows' rms."""
+    ops = _ops()
+    x = _rand((M, K), torch.bfloat16, 41)
+    w1 = _rand((H, K), torch.bfloat16, 42, scale=0.05)
+    w2 = _rand((N2, H), torch.bfloat16, 43, scale=0.05)
+    nw = (1.0 + _rand((H,), torch.float32, 44, scale=0.2)).to(norm_dtype)
+    residual = _rand((M, H), torch.float32, 45, scale=2.0)
+    residual[M // 2] *= 30.0                                       # a row whose factor is far from the others'
+    eps = 1e-5
+    assert ops.fused_rows_take(w1, M) and ops.fused_rows_take(w2, M)
+
+    exact_delta = (x.double() @ w1.double().T)
+    fused_stream = residual.clone()
+    values, sums = ops.linear_residual_norm(x, w1, None, fused_stream, nw)
+    # the stream: the product rounded to bfloat16 once, then added in float32
+    stream = residual + exact_delta.float().bfloat16().float()
+    differs = fused_stream != stream
+    assert float(differs.float().mean()) < 0.02                   # roundings at a bfloat16 tie aside
+    torch.testing.assert_close(fused_stream, stream, rtol=0, atol=2 ** -7 * float(exact_delta.abs().max()))
+    stream = fused_stream
+    assert sums.shape == (-(-H // 1024), M)
+    torch.testing.assert_close(sums.double().sum(dim=0), (stream.double() ** 2).sum(dim=1), rtol=1e-5, atol=1e-6)
+    assert torch.equal(values, (stream * nw.float()).bfloat16())
+
+    h = ops.rmsnorm(stream.clone(), nw, eps, torch.bfloat16)
+    want = ops.linear(h, w2, out_dtype=torch.float32)
+    got = ops.linear(values, w2, out_dtype=torch.float32, unscaled=(sums, eps, H))
+    exact = (stream.double() * torch.rsqrt((stream.double() ** 2).mean(dim=1, keepdim=True) + eps) * nw.double()) @ w2.double().T
+    for m in range(M):                                             # row by row: their sizes differ
+        scale = float(exact[m].abs().max())
+        assert float((got[m] - want[m]).abs().max()) <= 6e-3 * scale
+        assert float((got[m].double() - exact[m]).abs().max()) <= 6e-3 * scale
+    got_bf16 = ops.linear(values, w2, unscaled=(sums, eps, H))
+    torch.testing.assert_close(got_bf16.float(), got, rtol=8e-3, atol=1e-3)
+    if N2 % 2 == 0:
+        want_act = torch_ops.swiglu(exact.float().bfloat16().float())
+        got_act = ops.linear_swiglu(values, w2, unscaled=(sums, eps, H))
+        assert got_act.shape == (M, N2 // 2)
+        assert float((got_act.float() - want_act).abs().max()) <= 2e-2 * max(1.0, float(want_act.abs().max()))
+    # a second call gives the same bits (the choice of tile shape is kept, the additions are ordered)
+    again_stream = residual.clone()
+    v2, s2 = ops.linear_residual_norm(x, w1, None, again_stream, nw)
+    assert torch.equal(again_stream, fused_stream) and torch.equal(v2, values) and torch.equal(s2, sums)
+    assert torch.equal(ops.linear(values, w2, out_dtype=torch.float32, unscaled=(sums, eps, H)), got)
+    with pytest.raises(ops.OperandError):                          # sums of another number of rows
+        ops.linear(values, w2, unscaled=(sums[:, :-1].contiguous(), eps, H))
+
+
 def test_linear_float32_is_true_float32():
     """Inputs whose products need all 24 bits: a matrix mode of reduced precision
     (bf16 or tf32-like splitting) would be off by far more than float32 rounding."""

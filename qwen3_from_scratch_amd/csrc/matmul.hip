@@ -271,7 +271,7 @@ int run_plan(Device& d, const Plan& p, const void* x, const void* w, void* out, 
   return s == HIPBLAS_STATUS_SUCCESS ? 0 : Q3_ERR_LIBRARY + (int)s;
 }
 
-// Tile shape and shares of K for a product of 17 to 64 rows that carries a norm. `kind` tells the
+// Tile shape and shares of K for a product of some tens of rows that carries a norm. `kind` tells the
 // variants apart (0 plain, 1 SwiGLU, 2 residual); `launch(config, splits)` runs one without
 // side effects and returns its status. Timed once per size with cold caches outside a graph
 // capture; a capture that meets a new size takes the rule of thumb and leaves the timing to the
@@ -330,8 +330,9 @@ int choose_fused(Device& d, int kind, int M, int N, int K, hipStream_t stream, L
 
 }  // namespace
 
-// Products of 17 to 64 rows that carry a norm, by the hand-written tiled kernel (the few-row kernel of
-// gemm.hip does the same for up to 16 rows). x (M, K) and w (N, K) bfloat16, K a multiple of 64, N of 4.
+// Products of up to 256 rows that carry a norm, by the hand-written tiled kernel (the few-row kernel of
+// gemm.hip does the same for up to 16 rows and is faster there; the callers' policy decides which rows come
+// here). x (M, K) and w (N, K) bfloat16, K a multiple of 64, N of 4.
 //
 // q3_tiles_scaled: the rows of x hold stream * norm_weight and still lack the norm's division; `sums`
 // (chunks, M) float32 holds the rows' sums of squares of the stream in partial sums, `width` the stream's
@@ -339,7 +340,7 @@ int choose_fused(Device& d, int kind, int M, int N, int K, hipStream_t stream, L
 // 1 (rows of w interleave gate and up) gives (M, N / 2) bfloat16 = silu(gate) * up.
 extern "C" int q3_tiles_scaled(const void* x, const void* w, void* out, int M, int N, int K, int out_dtype,
                                int epilogue, const float* sums, int chunks, float eps, int width, void* stream_) {
-  if (!x || !w || !out || !sums || M < 1 || M > 64 || N % 4 || !tiles::takes(M, N, K)) return Q3_ERR_BAD_ARGUMENT;
+  if (!x || !w || !out || !sums || M < 1 || M > 256 || N % 4 || !tiles::takes(M, N, K)) return Q3_ERR_BAD_ARGUMENT;
   if (chunks < 1 || width != K) return Q3_ERR_BAD_ARGUMENT;
   const bool swiglu = epilogue == tiles::EPI_SWIGLU;
   if (!swiglu && epilogue != tiles::EPI_PLAIN) return Q3_ERR_BAD_ARGUMENT;
@@ -376,7 +377,7 @@ extern "C" int q3_tiles_residual(const void* x, const void* w, int M, int N, int
                                  const void* norm_weight, int norm_weight_dtype, void* values, float* sums,
                                  void* stream_) {
   if (!x || !w || !residual || !norm_weight || !values || !sums) return Q3_ERR_BAD_ARGUMENT;
-  if (M < 1 || M > 64 || N % 4 || !tiles::takes(M, N, K)) return Q3_ERR_BAD_ARGUMENT;
+  if (M < 1 || M > 256 || N % 4 || !tiles::takes(M, N, K)) return Q3_ERR_BAD_ARGUMENT;
   if (norm_weight_dtype != Q3_BF16 && norm_weight_dtype != Q3_F32) return Q3_ERR_BAD_ARGUMENT;
   hipStream_t stream = (hipStream_t)stream_;
   std::lock_guard<std::mutex> hold(g_lock);

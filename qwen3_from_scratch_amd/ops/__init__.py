@@ -452,12 +452,13 @@ def _row_sums_args(unscaled, M, K):
     return _ptr(sums), sums.shape[0], ctypes.c_float(eps), int(width)
 
 
-FUSED_ROWS_FEW, FUSED_ROWS_MOST = 16, 64
+FUSED_ROWS_FEW, FUSED_ROWS_MOST = 16, 128
 
 
 def fused_rows_take(weight, M):
     """Whether the tiled kernel carries a norm for `M` rows of a product with `weight` (N, K):
-    more rows than the few-row kernel takes, at most 64, bfloat16, K a multiple of 64 and N of 4."""
+    more rows than the few-row kernel takes, at most 128 (beyond that the vendor library's products with the norms as kernels of
+    their own are faster), bfloat16, K a multiple of 64 and N of 4."""
     return (FUSED_ROWS_FEW < M <= FUSED_ROWS_MOST and weight.dtype == torch.bfloat16 and weight.dim() == 2
             and weight.shape[1] % 64 == 0 and weight.shape[0] % 4 == 0 and weight.is_contiguous())
 
@@ -505,7 +506,7 @@ def linear(x, weight, out_dtype=None, out=None, tiled=None, unscaled=None):
         return out
     if unscaled is not None and x.dtype == torch.bfloat16 and fused_rows_take(weight, M):
         return _tiles_scaled(x, weight, out, unscaled, False, "linear")
-    _need(unscaled is None, "unscaled rows need bfloat16 and at most 16 rows with a tiled weight, or 17 to 64 rows "
+    _need(unscaled is None, "unscaled rows need bfloat16 and at most 16 rows with a tiled weight, or 17 to 128 rows "
           "with an inner size that is a multiple of 64")
     if M and x.dtype == torch.bfloat16 and not library("gemm").q3_linear_is_skinny(M, N, K, 1):
         # bfloat16 products with many rows go to the vendor library (hipBLASLt), as the
@@ -550,7 +551,7 @@ def linear_swiglu(x, weight, tiled=None, unscaled=None):
     if unscaled is not None and x.dtype == torch.bfloat16 and fused_rows_take(weight, M):
         out = torch.empty((M, N // 2), dtype=x.dtype, device=x.device)
         return _tiles_scaled(x, weight, out, unscaled, True, "linear_swiglu")
-    _need(unscaled is None, "unscaled rows need bfloat16 and at most 16 rows with a tiled weight, or 17 to 64 rows "
+    _need(unscaled is None, "unscaled rows need bfloat16 and at most 16 rows with a tiled weight, or 17 to 128 rows "
           "with an inner size that is a multiple of 64")
     if M and library("gemm").q3_linear_is_skinny(M, N, K, _DT[x.dtype]):
         out = torch.empty((M, N // 2), dtype=x.dtype, device=x.device)
@@ -572,7 +573,7 @@ def linear_residual_norm(x, weight, tiled, residual, norm_weight):
     `linear` and `linear_swiglu` apply that factor to their products when given
     `unscaled=(sums, eps, N)`.
 
-    With 17 to 64 rows (`fused_rows_take`; `tiled` is not used) the tiled kernel's partial
+    With 17 to 128 rows (`fused_rows_take`; `tiled` is not used) the tiled kernel's partial
     products are added by a second kernel that does the same; sums is then (ceil(N / 1024), M),
     partial sums over 1,024 columns, row m of the stream in column m."""
     _dev(x, weight, tiled, residual, norm_weight)

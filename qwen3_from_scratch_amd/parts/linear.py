@@ -34,7 +34,7 @@ class LinearWeight:
     def fuses(self):
         """Whether steps of few rows go through kernels whose epilogues carry the
         norm fusion, UnscaledRows in, a NormSink out: up to 16 rows the few-row
-        kernel on the tiled copy, up to 64 the tiled matrix-core kernel. A
+        kernel on the tiled copy, up to 128 the tiled matrix-core kernel. A
         reader of UnscaledRows must have output rows in steps of 4."""
         return self.tiled is not None and self.weight.shape[0] % 4 == 0
 

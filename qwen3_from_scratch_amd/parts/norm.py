@@ -39,7 +39,7 @@ class RMSNorm(Part):
         """A NormSink for the residual `x` if this step may have the addition
         and this norm fused into the neighbouring products (bfloat16 with
         tiled matrices; at most 16 rows and a width in steps of 16, or up to
-        64 rows and a width in steps of 64), else None."""
+        128 rows and a width in steps of 64), else None."""
         rows = x.shape[0]
         if self.precision.act != torch.bfloat16 or not self.precision.tiled or self.weight is None:
             return None

@@ -649,9 +649,10 @@ def test_linear_residual_norm_and_unscaled_rows(M, H, K, N2, norm_dtype):
 
 @pytest.mark.parametrize("norm_dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("M,H,K,N2", [(17, 4096, 4096, 6144), (64, 4096, 12288, 24576), (40, 1024, 512, 6152),
-                                      (33, 192, 64, 332), (64, 5120, 3200, 1000), (25, 1088, 17408, 128)])
+                                      (33, 192, 64, 332), (64, 5120, 3200, 1000), (25, 1088, 17408, 128),
+                                      (100, 4096, 4096, 24576), (128, 2048, 1024, 6144)])
 def test_linear_residual_norm_and_unscaled_rows_beyond_sixteen(M, H, K, N2, norm_dtype):
-    """The same pair of fusions for 17 to 64 rows, where the tiled kernel carries them: its
+    """The same pair of fusions for 17 to 128 rows, where the tiled kernel carries them: its
     partial products go through a second kernel that adds them into the stream, and the next
     product's epilogue (or the kernel that adds its partial products) divides by the rows' rms."""
     ops = _ops()

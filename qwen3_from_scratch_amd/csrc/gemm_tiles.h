@@ -183,10 +183,14 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiles_kernel(const bf16_t* 
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     else if (steps_after == 1)
       asm volatile("s_waitcnt vmcnt(%0)" ::"n"(S::LOADS) : "memory");
-    else
+    else if (steps_after == 2 || STAGES <= 4)
       asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * S::LOADS) : "memory");
+    else if (steps_after == 3 || STAGES <= 5)
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(STAGES > 4 ? 3 * S::LOADS : 0) : "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(STAGES > 5 ? 4 * S::LOADS : 0) : "memory");
   };
-  static_assert(STAGES >= 2 && STAGES <= 4 && 2 * S::LOADS < 64, "the wait counts above");
+  static_assert(STAGES >= 2 && STAGES <= 6 && (STAGES - 2) * S::LOADS < 64, "the wait counts above");
 
   // operand reads: row 16 i + col of this wavefront's half of a slice, pieces 4 s + grp
   const int swz = (col >> 1) & 7;
@@ -315,7 +319,7 @@ __global__ __launch_bounds__(256) void tiles_residual_kernel(const float* __rest
 }
 
 // The tile shapes on offer: (BM, BN, STAGES).
-constexpr int NUM_CONFIGS = 8;
+constexpr int NUM_CONFIGS = 9;
 
 // `splits` > 1: K is shared out over that many blocks per tile, which leave float32 partial
 // products in `partials` (splits x M x N floats) for a second kernel to add, which also applies
@@ -364,7 +368,8 @@ int launch_config(const void* x, const void* w, void* out, int M, int N, int K, 
 inline int splits_that_fill(int config, int M, int N, int K) {
   // tile rows, tile columns, blocks resident at once on 256 CUs (what shared memory allows)
   static const int shape[NUM_CONFIGS][3] = {{128, 128, 512}, {128, 128, 256}, {256, 128, 256}, {256, 256, 256},
-                                            {256, 256, 256}, {64, 128, 512}, {64, 128, 768}, {64, 256, 512}};
+                                            {256, 256, 256}, {64, 128, 512}, {64, 128, 768}, {64, 256, 512},
+                                            {64, 128, 256}};
   if (config < 0 || config >= NUM_CONFIGS) return 1;
   const int bm = shape[config][0], bn = shape[config][1], slots = shape[config][2];
   const long tiles = (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
@@ -387,6 +392,7 @@ int launch(int config, const void* x, const void* w, void* out, int M, int N, in
     case 5: return launch_config<OUT, EPI, 64, 128, 1, 4, 3>(x, w, out, M, N, K, splits, partials, stream, scale, keep_partials, splits_used);
     case 6: return launch_config<OUT, EPI, 64, 128, 1, 4, 2>(x, w, out, M, N, K, splits, partials, stream, scale, keep_partials, splits_used);
     case 7: return launch_config<OUT, EPI, 64, 256, 1, 8, 2>(x, w, out, M, N, K, splits, partials, stream, scale, keep_partials, splits_used);
+    case 8: return launch_config<OUT, EPI, 64, 128, 1, 4, 5>(x, w, out, M, N, K, splits, partials, stream, scale, keep_partials, splits_used);
   }
   return Q3_ERR_BAD_ARGUMENT;
 }

@@ -285,8 +285,11 @@ int choose_fused(Device& d, int kind, int M, int N, int K, hipStream_t stream, L
     splits = known->second.second;
     return 0;
   }
-  int configs[4], shares[4], n = 0;
-  for (int shape : OWN_FEW_ROWS) {   // the 64 x 256 tiles lose here too (gate/up at 64 rows: 67 us against 51)
+  // 64 x 128 tiles also with five stages: with K shared out they need fewer shares to fill the chip (q/k/v at
+  // 64 rows 17.7 us in 5 shares against 21.9 in 8). The 64 x 256 tiles lose here too (gate/up 67 us against 51).
+  constexpr int FUSED_SHAPES[] = {1, 5, 8};
+  int configs[6], shares[6], n = 0;
+  for (int shape : FUSED_SHAPES) {
     const int fill = tiles::splits_that_fill(shape, M, N, K);
     if (fill > 1 && (size_t)fill * M * N * sizeof(float) <= PARTIALS_BYTES) {
       configs[n] = shape;

@@ -278,7 +278,8 @@ int run_plan(Device& d, const Plan& p, const void* x, const void* w, void* out, 
 // next eager call.
 template <typename Launch>
 int choose_fused(Device& d, int kind, int M, int N, int K, hipStream_t stream, Launch launch, int& config, int& splits) {
-  const auto key = std::make_tuple(kind, M, N, K);
+  // rows that differ within a step of eight share a choice: a serving loop meets most of them
+  const auto key = std::make_tuple(kind, (M + 7) / 8 * 8, N, K);
   auto known = d.fused.find(key);
   if (known != d.fused.end()) {
     config = known->second.first;
@@ -290,8 +291,8 @@ int choose_fused(Device& d, int kind, int M, int N, int K, hipStream_t stream, L
   constexpr int FUSED_SHAPES[] = {1, 5, 8};
   int configs[6], shares[6], n = 0;
   for (int shape : FUSED_SHAPES) {
-    const int fill = tiles::splits_that_fill(shape, M, N, K);
-    if (fill > 1 && (size_t)fill * M * N * sizeof(float) <= PARTIALS_BYTES) {
+    const int fill = tiles::splits_that_fill(shape, M, N, K);   // the same for all rows that share the choice
+    if (fill > 1 && (size_t)fill * ((M + 7) / 8 * 8) * N * sizeof(float) <= PARTIALS_BYTES) {
       configs[n] = shape;
       shares[n++] = fill;
     }
@@ -393,6 +394,7 @@ extern "C" int q3_tiles_residual(const void* x, const void* w, int M, int N, int
     return tiles::launch<bf16_t, tiles::EPI_PLAIN>(c, x, w, values, M, N, K, stream, s, d.partials);
   }, config, splits);
   if (status) return status;
+  if ((size_t)splits * M * N * sizeof(float) > PARTIALS_BYTES) return Q3_ERR_UNSUPPORTED;   // also a single share
   int used = 1;
   status = tiles::launch<bf16_t, tiles::EPI_PLAIN>(config, x, w, values, M, N, K, stream, splits, d.partials,
                                                    tiles::RowScale(), true, &used);

@@ -37,12 +37,14 @@
 #include <vector>
 
 #define Q3_ERR_LIBRARY 20000   // + the library's status
+#define Q3_DECLINED 1          // q3_tiles_residual: nothing was done, the caller's other way is faster
 
 namespace {
 
 constexpr size_t WORKSPACE_BYTES = 128u << 20;
 constexpr size_t EVICT_BYTES = 512u << 20;     // twice the 256 MB last-level cache
 constexpr size_t PARTIALS_BYTES = 128u << 20;  // float32 partial products of the hand-written kernel's K shares
+constexpr size_t STAGING_BYTES = 64u << 20;
 constexpr int EVICT_BLOCKS = 2048, EVICT_THREADS = 256;
 constexpr int MAX_CANDIDATES = 64;
 
@@ -72,6 +74,7 @@ struct Device {
   void* workspace = nullptr;
   void* evict = nullptr;
   float* partials = nullptr;
+  float* staging = nullptr;   // a float32 product on its way to the kernel that divides its rows (q3_tiles_scaled)
   hipEvent_t begin = nullptr, end = nullptr;
   std::map<std::tuple<int, int, int, int>, Plan> plans;
   // what was chosen for a size, by its rows rounded up to a multiple of 32: sizes beyond 64
@@ -271,221 +274,8 @@ int run_plan(Device& d, const Plan& p, const void* x, const void* w, void* out, 
   return s == HIPBLAS_STATUS_SUCCESS ? 0 : Q3_ERR_LIBRARY + (int)s;
 }
 
-// Tile shape and shares of K for a product of some tens of rows that carries a norm. `kind` tells the
-// variants apart (0 plain, 1 SwiGLU, 2 residual); `launch(config, splits)` runs one without
-// side effects and returns its status. Timed once per size with cold caches outside a graph
-// capture; a capture that meets a new size takes the rule of thumb and leaves the timing to the
-// next eager call.
-template <typename Launch>
-int choose_fused(Device& d, int kind, int M, int N, int K, hipStream_t stream, Launch launch, int& config, int& splits) {
-  // rows that differ within a step of eight share a choice: a serving loop meets most of them
-  const auto key = std::make_tuple(kind, (M + 7) / 8 * 8, N, K);
-  auto known = d.fused.find(key);
-  if (known != d.fused.end()) {
-    config = known->second.first;
-    splits = known->second.second;
-    return 0;
-  }
-  // 64 x 128 tiles also with five stages: with K shared out they need fewer shares to fill the chip (q/k/v at
-  // 64 rows 17.7 us in 5 shares against 21.9 in 8). The 64 x 256 tiles lose here too (gate/up 67 us against 51).
-  constexpr int FUSED_SHAPES[] = {1, 5, 8};
-  int configs[6], shares[6], n = 0;
-  for (int shape : FUSED_SHAPES) {
-    const int fill = tiles::splits_that_fill(shape, M, N, K);   // the same for all rows that share the choice
-    if (fill > 1 && (size_t)fill * ((M + 7) / 8 * 8) * N * sizeof(float) <= PARTIALS_BYTES) {
-      configs[n] = shape;
-      shares[n++] = fill;
-    }
-    configs[n] = shape;
-    shares[n++] = 1;
-  }
-  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
-  HIP_TRY(hipStreamIsCapturing(stream, &capture));
-  if (!d.partials) {
-    if (capture != hipStreamCaptureStatusNone) return (int)hipErrorStreamCaptureUnsupported;
-    HIP_TRY(hipMalloc((void**)&d.partials, PARTIALS_BYTES));
-  }
-  config = configs[0];
-  splits = shares[0];
-  if (capture != hipStreamCaptureStatusNone) return 0;
-  if (!d.begin) {
-    HIP_TRY(hipEventCreate(&d.begin));
-    HIP_TRY(hipEventCreate(&d.end));
-  }
-  if (!d.evict) {
-    HIP_TRY(hipMalloc(&d.evict, EVICT_BYTES));
-    HIP_TRY(hipMemsetAsync(d.evict, 0, EVICT_BYTES, stream));
-  }
-  float best = -1.f;
-  for (int i = 0; i < n; ++i) {
-    auto one = [&] { return launch(configs[i], shares[i]) == 0; };
-    if (time_runs(d, stream, 1, one) < 0.f) continue;   // the first run also loads the code
-    const float us = time_runs(d, stream, 4, one);
-    if (us > 0.f && (best < 0.f || us < best)) {
-      best = us;
-      config = configs[i];
-      splits = shares[i];
-    }
-  }
-  if (best < 0.f) return Q3_ERR_UNSUPPORTED;
-  d.fused[key] = std::make_pair(config, splits);
-  return 0;
-}
-
-}  // namespace
-
-// Products of up to 256 rows that carry a norm, by the hand-written tiled kernel (the few-row kernel of
-// gemm.hip does the same for up to 16 rows and is faster there; the callers' policy decides which rows come
-// here). x (M, K) and w (N, K) bfloat16, K a multiple of 64, N of 4.
-//
-// q3_tiles_scaled: the rows of x hold stream * norm_weight and still lack the norm's division; `sums`
-// (chunks, M) float32 holds the rows' sums of squares of the stream in partial sums, `width` the stream's
-// width (= K). out = (x @ w^T) * rsqrt(sum / width + eps) row by row: epilogue 0 gives (M, N) in `out_dtype`,
-// 1 (rows of w interleave gate and up) gives (M, N / 2) bfloat16 = silu(gate) * up.
-extern "C" int q3_tiles_scaled(const void* x, const void* w, void* out, int M, int N, int K, int out_dtype,
-                               int epilogue, const float* sums, int chunks, float eps, int width, void* stream_) {
-  if (!x || !w || !out || !sums || M < 1 || M > 256 || N % 4 || !tiles::takes(M, N, K)) return Q3_ERR_BAD_ARGUMENT;
-  if (chunks < 1 || width != K) return Q3_ERR_BAD_ARGUMENT;
-  const bool swiglu = epilogue == tiles::EPI_SWIGLU;
-  if (!swiglu && epilogue != tiles::EPI_PLAIN) return Q3_ERR_BAD_ARGUMENT;
-  if (swiglu ? out_dtype != Q3_BF16 : (out_dtype != Q3_BF16 && out_dtype != Q3_F32)) return Q3_ERR_BAD_ARGUMENT;
-  hipStream_t stream = (hipStream_t)stream_;
-  std::lock_guard<std::mutex> hold(g_lock);
-  int device = 0;
-  HIP_TRY(hipGetDevice(&device));
-  Device& d = g_devices[device];
-  tiles::RowScale scale;
-  scale.sums = sums;
-  scale.chunks = chunks;
-  scale.rows = M;
-  scale.eps = eps;
-  scale.inv_width = 1.f / (float)width;
-  auto launch = [&](int config, int splits) {
-    if (swiglu)
-      return tiles::launch<bf16_t, tiles::EPI_SWIGLU>(config, x, w, out, M, N, K, stream, splits, d.partials, scale);
-    if (out_dtype == Q3_F32)
-      return tiles::launch<float, tiles::EPI_PLAIN>(config, x, w, out, M, N, K, stream, splits, d.partials, scale);
-    return tiles::launch<bf16_t, tiles::EPI_PLAIN>(config, x, w, out, M, N, K, stream, splits, d.partials, scale);
-  };
-  int config = 0, splits = 1;
-  const int status = choose_fused(d, swiglu ? 1 : 0, M, N, K, stream, launch, config, splits);
-  return status ? status : launch(config, splits);
-}
-
-// q3_tiles_residual: residual (M, N) float32 += bfloat16(x @ w^T) in place; values (M, N) bfloat16 =
-// residual * norm_weight; sums (ceil(N / 1024), M) float32 = the rows' sums of squares of the new residual over
-// chunks of 1,024 columns: what q3_tiles_scaled takes for the next product.
-extern "C" int q3_tiles_residual_chunks(int N) { return (N + tiles::CHUNK_COLUMNS - 1) / tiles::CHUNK_COLUMNS; }
-
-extern "C" int q3_tiles_residual(const void* x, const void* w, int M, int N, int K, float* residual,
-                                 const void* norm_weight, int norm_weight_dtype, void* values, float* sums,
-                                 void* stream_) {
-  if (!x || !w || !residual || !norm_weight || !values || !sums) return Q3_ERR_BAD_ARGUMENT;
-  if (M < 1 || M > 256 || N % 4 || !tiles::takes(M, N, K)) return Q3_ERR_BAD_ARGUMENT;
-  if (norm_weight_dtype != Q3_BF16 && norm_weight_dtype != Q3_F32) return Q3_ERR_BAD_ARGUMENT;
-  hipStream_t stream = (hipStream_t)stream_;
-  std::lock_guard<std::mutex> hold(g_lock);
-  int device = 0;
-  HIP_TRY(hipGetDevice(&device));
-  Device& d = g_devices[device];
-  int config = 0, splits = 1;
-  // timed by the product into `values`, which the real run overwrites: the residual is not touched
-  int status = choose_fused(d, 2, M, N, K, stream, [&](int c, int s) {
-    return tiles::launch<bf16_t, tiles::EPI_PLAIN>(c, x, w, values, M, N, K, stream, s, d.partials);
-  }, config, splits);
-  if (status) return status;
-  if ((size_t)splits * M * N * sizeof(float) > PARTIALS_BYTES) return Q3_ERR_UNSUPPORTED;   // also a single share
-  int used = 1;
-  status = tiles::launch<bf16_t, tiles::EPI_PLAIN>(config, x, w, values, M, N, K, stream, splits, d.partials,
-                                                   tiles::RowScale(), true, &used);
-  if (status) return status;
-  const dim3 grid(q3_tiles_residual_chunks(N), M);
-  if (norm_weight_dtype == Q3_F32)
-    hipLaunchKernelGGL(tiles::tiles_residual_kernel<float>, grid, dim3(256), 0, stream, d.partials, used, residual,
-                       (const float*)norm_weight, (bf16_t*)values, sums, M, N);
-  else
-    hipLaunchKernelGGL(tiles::tiles_residual_kernel<bf16_t>, grid, dim3(256), 0, stream, d.partials, used, residual,
-                       (const bf16_t*)norm_weight, (bf16_t*)values, sums, M, N);
-  return q3_launch_status();
-}
-
-// The hand-written tiled kernel alone (gemm_tiles.h), tile shape `config` (0 .. q3_gemm_tiles_configs() - 1):
-// x (M, K) and w (N, K) bfloat16, K a multiple of 64; `epilogue` 0: out (M, N) in `out_dtype`; 1: rows of w
-// interleave gate and up, out (M, N / 2) bfloat16 = silu(gate) * up.
-extern "C" int q3_gemm_tiles_configs() { return tiles::NUM_CONFIGS; }
-
-// `splits` > 1 (plain epilogue, N a multiple of 4): K is shared out over that many blocks per tile and
-// `partials` (splits * M * N floats) takes their partial products; q3_gemm_tiles_splits says how many fill the
-// chip once.
-extern "C" int q3_gemm_tiles_splits(int config, int M, int N, int K) {
-  return tiles::takes(M, N, K) && config >= 0 && config < tiles::NUM_CONFIGS ? tiles::splits_that_fill(config, M, N, K)
-                                                                            : 1;
-}
-
-extern "C" int q3_gemm_tiles(const void* x, const void* w, void* out, int M, int N, int K, int out_dtype,
-                             int epilogue, int config, int splits, float* partials, void* stream_) {
-  if (!x || !w || !out || !tiles::takes(M, N, K)) return Q3_ERR_BAD_ARGUMENT;
-  hipStream_t stream = (hipStream_t)stream_;
-  std::lock_guard<std::mutex> hold(g_lock);   // the launchers keep a per-device flag
-  if (epilogue == tiles::EPI_SWIGLU) {
-    if (out_dtype != Q3_BF16 || N % 2) return Q3_ERR_BAD_ARGUMENT;
-    return tiles::launch<bf16_t, tiles::EPI_SWIGLU>(config, x, w, out, M, N, K, stream, splits, partials);
-  }
-  if (epilogue != tiles::EPI_PLAIN) return Q3_ERR_BAD_ARGUMENT;
-  if (out_dtype == Q3_F32)
-    return tiles::launch<float, tiles::EPI_PLAIN>(config, x, w, out, M, N, K, stream, splits, partials);
-  if (out_dtype == Q3_BF16)
-    return tiles::launch<bf16_t, tiles::EPI_PLAIN>(config, x, w, out, M, N, K, stream, splits, partials);
-  return Q3_ERR_BAD_ARGUMENT;
-}
-
-// How many of the library's candidates are timed for a new problem size (1: take its first choice).
-extern "C" int q3_matmul_set_candidates(int n) {
-  if (n < 1 || n > MAX_CANDIDATES) return Q3_ERR_BAD_ARGUMENT;
-  std::lock_guard<std::mutex> hold(g_lock);
-  g_candidates = n;
-  return 0;
-}
-
-// Which kernels enter the contest for a new size: 0 the library's and the hand-written one's (the default),
-// 1 the library's alone, 2 the hand-written ones alone where they take the size. Sizes already met keep their
-// choice.
-extern "C" int q3_matmul_set_kernels(int mode) {
-  if (mode < KERNELS_BOTH || mode > KERNELS_OWN) return Q3_ERR_BAD_ARGUMENT;
-  std::lock_guard<std::mutex> hold(g_lock);
-  g_kernels = mode;
-  return 0;
-}
-
-// What was chosen for a size on the current device: info[0] candidates timed, info[1] index chosen,
-// info[2] microseconds of the first candidate, info[3] of the chosen one, info[4] the hand-written kernel's
-// tile shape if that was chosen, else -1, info[5] over how many blocks it shares K out. Returns 1 if the size
-// is known.
-extern "C" int q3_matmul_plan(int M, int N, int K, int out_dtype, float* info) {
-  std::lock_guard<std::mutex> hold(g_lock);
-  int device = 0;
-  if (hipGetDevice(&device) != hipSuccess) return 0;
-  auto d = g_devices.find(device);
-  if (d == g_devices.end()) return 0;
-  auto p = d->second.plans.find(std::make_tuple(M, N, K, out_dtype));
-  if (p == d->second.plans.end()) return 0;
-  info[0] = (float)p->second.candidates;
-  info[1] = (float)p->second.chosen;
-  info[2] = p->second.first_us;
-  info[3] = p->second.best_us;
-  info[4] = (float)p->second.own;
-  info[5] = (float)p->second.own_splits;
-  return 1;
-}
-
-extern "C" int q3_matmul(const void* x, const void* w, void* out, int M, int N, int K, int out_dtype, void* stream_) {
-  if (M <= 0 || N <= 0 || K <= 0 || !x || !w || !out) return Q3_ERR_BAD_ARGUMENT;
-  if (out_dtype != Q3_F32 && out_dtype != Q3_BF16) return Q3_ERR_BAD_ARGUMENT;
-  hipStream_t stream = (hipStream_t)stream_;
-  std::lock_guard<std::mutex> hold(g_lock);
-  int device = 0;
-  HIP_TRY(hipGetDevice(&device));
-  Device& d = g_devices[device];
+// out = x @ w^T by whichever kernel the contest chose for the size (the lock is held).
+int product(Device& d, const void* x, const void* w, void* out, int M, int N, int K, int out_dtype, hipStream_t stream) {
   hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
   HIP_TRY(hipStreamIsCapturing(stream, &capture));
   const bool capturing = capture != hipStreamCaptureStatusNone;
@@ -541,4 +331,267 @@ extern "C" int q3_matmul(const void* x, const void* w, void* out, int M, int N, 
     }
   }
   return run_plan(d, p, x, w, out, M, N, K, out_dtype, stream);
+}
+
+// Tile shape and shares of K for a product of some tens of rows that carries a norm. `kind` tells the
+// variants apart (0 plain, 1 SwiGLU, 2 residual); `launch(config, splits)` runs one without side effects and
+// returns its status; `other()` does the same work around the contest's product (the vendor library's, mostly)
+// and wins where the tiled kernel's tiles fit the size badly: `config` is then LIBRARY. Timed once per size
+// with cold caches outside a graph capture; a capture that meets a new size takes the rule of thumb and leaves
+// the timing to the next eager call.
+constexpr int LIBRARY = -1;
+template <typename Launch, typename Other>
+int choose_fused(Device& d, int kind, int M, int N, int K, hipStream_t stream, Launch launch, Other other, int& config,
+                 int& splits) {
+  // rows that differ within a step of eight share a choice: a serving loop meets most of them
+  const auto key = std::make_tuple(kind + 4 * g_kernels, (M + 7) / 8 * 8, N, K);
+  auto known = d.fused.find(key);
+  if (known != d.fused.end()) {
+    config = known->second.first;
+    splits = known->second.second;
+    return 0;
+  }
+  // 64 x 128 tiles also with five stages: with K shared out they need fewer shares to fill the chip (q/k/v at
+  // 64 rows 17.7 us in 5 shares against 21.9 in 8). The 64 x 256 tiles lose here too (gate/up 67 us against 51).
+  constexpr int FUSED_SHAPES[] = {1, 5, 8};
+  int configs[6], shares[6], n = 0;
+  for (int shape : FUSED_SHAPES) {
+    const int fill = tiles::splits_that_fill(shape, M, N, K);   // the same for all rows that share the choice
+    if (fill > 1 && (size_t)fill * ((M + 7) / 8 * 8) * N * sizeof(float) <= PARTIALS_BYTES) {
+      configs[n] = shape;
+      shares[n++] = fill;
+    }
+    configs[n] = shape;
+    shares[n++] = 1;
+  }
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  HIP_TRY(hipStreamIsCapturing(stream, &capture));
+  if (!d.partials) {
+    if (capture != hipStreamCaptureStatusNone) return (int)hipErrorStreamCaptureUnsupported;
+    HIP_TRY(hipMalloc((void**)&d.partials, PARTIALS_BYTES));
+  }
+  config = configs[0];
+  splits = shares[0];
+  if (capture != hipStreamCaptureStatusNone) return 0;
+  if (!d.begin) {
+    HIP_TRY(hipEventCreate(&d.begin));
+    HIP_TRY(hipEventCreate(&d.end));
+  }
+  if (!d.evict) {
+    HIP_TRY(hipMalloc(&d.evict, EVICT_BYTES));
+    HIP_TRY(hipMemsetAsync(d.evict, 0, EVICT_BYTES, stream));
+  }
+  float best = -1.f;
+  // the first call of the other way holds that product's own contest: not inside a timed run, whose events it uses
+  const bool other_works = g_kernels != KERNELS_OWN && other() == 0;
+  for (int i = 0; i < n && !(other_works && g_kernels == KERNELS_LIBRARY); ++i) {
+    auto one = [&] { return launch(configs[i], shares[i]) == 0; };
+    if (time_runs(d, stream, 1, one) < 0.f) continue;   // the first run also loads the code
+    const float us = time_runs(d, stream, 4, one);
+    if (us > 0.f && (best < 0.f || us < best)) {
+      best = us;
+      config = configs[i];
+      splits = shares[i];
+    }
+  }
+  if (other_works) {
+    const float us = time_runs(d, stream, 4, [&] { return other() == 0; });
+    if (us > 0.f && (best < 0.f || us < best)) {
+      best = us;
+      config = LIBRARY;
+      splits = 1;
+    }
+  }
+  if (best < 0.f) return Q3_ERR_UNSUPPORTED;
+  d.fused[key] = std::make_pair(config, splits);
+  return 0;
+}
+
+}  // namespace
+
+// Products of up to 256 rows that carry a norm, by the hand-written tiled kernel (the few-row kernel of
+// gemm.hip does the same for up to 16 rows and is faster there; the callers' policy decides which rows come
+// here). x (M, K) and w (N, K) bfloat16, K a multiple of 64, N of 4.
+//
+// q3_tiles_scaled: the rows of x hold stream * norm_weight and still lack the norm's division; `sums`
+// (chunks, M) float32 holds the rows' sums of squares of the stream in partial sums, `width` the stream's
+// width (= K). out = (x @ w^T) * rsqrt(sum / width + eps) row by row: epilogue 0 gives (M, N) in `out_dtype`,
+// 1 (rows of w interleave gate and up) gives (M, N / 2) bfloat16 = silu(gate) * up.
+extern "C" int q3_tiles_scaled(const void* x, const void* w, void* out, int M, int N, int K, int out_dtype,
+                               int epilogue, const float* sums, int chunks, float eps, int width, void* stream_) {
+  if (!x || !w || !out || !sums || M < 1 || M > 256 || N % 4 || !tiles::takes(M, N, K)) return Q3_ERR_BAD_ARGUMENT;
+  if (chunks < 1 || width != K) return Q3_ERR_BAD_ARGUMENT;
+  const bool swiglu = epilogue == tiles::EPI_SWIGLU;
+  if (!swiglu && epilogue != tiles::EPI_PLAIN) return Q3_ERR_BAD_ARGUMENT;
+  if (swiglu ? out_dtype != Q3_BF16 : (out_dtype != Q3_BF16 && out_dtype != Q3_F32)) return Q3_ERR_BAD_ARGUMENT;
+  hipStream_t stream = (hipStream_t)stream_;
+  std::lock_guard<std::mutex> hold(g_lock);
+  int device = 0;
+  HIP_TRY(hipGetDevice(&device));
+  Device& d = g_devices[device];
+  tiles::RowScale scale;
+  scale.sums = sums;
+  scale.chunks = chunks;
+  scale.rows = M;
+  scale.eps = eps;
+  scale.inv_width = 1.f / (float)width;
+  auto launch = [&](int config, int splits) {
+    if (swiglu)
+      return tiles::launch<bf16_t, tiles::EPI_SWIGLU>(config, x, w, out, M, N, K, stream, splits, d.partials, scale);
+    if (out_dtype == Q3_F32)
+      return tiles::launch<float, tiles::EPI_PLAIN>(config, x, w, out, M, N, K, stream, splits, d.partials, scale);
+    return tiles::launch<bf16_t, tiles::EPI_PLAIN>(config, x, w, out, M, N, K, stream, splits, d.partials, scale);
+  };
+  // the other way: the contest's product in float32, then the kernel that otherwise adds partial products
+  // divides (and activates) its rows
+  auto other = [&]() {
+    if ((size_t)M * N * sizeof(float) > STAGING_BYTES) return Q3_ERR_UNSUPPORTED;
+    if (!d.staging) {
+      hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+      HIP_TRY(hipStreamIsCapturing(stream, &capture));
+      if (capture != hipStreamCaptureStatusNone) return (int)hipErrorStreamCaptureUnsupported;
+      HIP_TRY(hipMalloc((void**)&d.staging, STAGING_BYTES));
+    }
+    const int status = product(d, x, w, d.staging, M, N, K, Q3_F32, stream);
+    if (status) return status;
+    const size_t quads = (size_t)M * N / 4;
+    const dim3 grid((unsigned)((quads + 255) / 256));
+    if (swiglu)
+      hipLaunchKernelGGL((tiles::gemm_tiles_reduce_kernel<bf16_t, true>), grid, dim3(256), 0, stream, d.staging,
+                         (bf16_t*)out, quads, N / 4, 1, scale);
+    else if (out_dtype == Q3_F32)
+      hipLaunchKernelGGL((tiles::gemm_tiles_reduce_kernel<float, false>), grid, dim3(256), 0, stream, d.staging,
+                         (float*)out, quads, N / 4, 1, scale);
+    else
+      hipLaunchKernelGGL((tiles::gemm_tiles_reduce_kernel<bf16_t, false>), grid, dim3(256), 0, stream, d.staging,
+                         (bf16_t*)out, quads, N / 4, 1, scale);
+    return q3_launch_status();
+  };
+  int config = 0, splits = 1;
+  const int status = choose_fused(d, swiglu ? 1 : 0, M, N, K, stream, launch, other, config, splits);
+  if (status) return status;
+  return config == LIBRARY ? other() : launch(config, splits);
+}
+
+// q3_tiles_residual: residual (M, N) float32 += bfloat16(x @ w^T) in place; values (M, N) bfloat16 =
+// residual * norm_weight; sums (ceil(N / 1024), M) float32 = the rows' sums of squares of the new residual over
+// chunks of 1,024 columns: what q3_tiles_scaled takes for the next product. Returns Q3_DECLINED, and has done
+// nothing, where the contest's plain product followed by the norm's own kernel is the faster way for this size.
+extern "C" int q3_tiles_residual_chunks(int N) { return (N + tiles::CHUNK_COLUMNS - 1) / tiles::CHUNK_COLUMNS; }
+
+extern "C" int q3_tiles_residual(const void* x, const void* w, int M, int N, int K, float* residual,
+                                 const void* norm_weight, int norm_weight_dtype, void* values, float* sums,
+                                 void* stream_) {
+  if (!x || !w || !residual || !norm_weight || !values || !sums) return Q3_ERR_BAD_ARGUMENT;
+  if (M < 1 || M > 256 || N % 4 || !tiles::takes(M, N, K)) return Q3_ERR_BAD_ARGUMENT;
+  if (norm_weight_dtype != Q3_BF16 && norm_weight_dtype != Q3_F32) return Q3_ERR_BAD_ARGUMENT;
+  hipStream_t stream = (hipStream_t)stream_;
+  std::lock_guard<std::mutex> hold(g_lock);
+  int device = 0;
+  HIP_TRY(hipGetDevice(&device));
+  Device& d = g_devices[device];
+  int config = 0, splits = 1;
+  // timed by the products alone (the tiled kernel's partial products; the contest's product into `values`,
+  // which the real run overwrites): each way has one small kernel more, and the residual is not touched
+  int status = choose_fused(
+      d, 2, M, N, K, stream,
+      [&](int c, int s) {
+        if ((size_t)s * M * N * sizeof(float) > PARTIALS_BYTES) return Q3_ERR_UNSUPPORTED;
+        return tiles::launch<bf16_t, tiles::EPI_PLAIN>(c, x, w, values, M, N, K, stream, s, d.partials,
+                                                       tiles::RowScale(), true);
+      },
+      [&]() { return product(d, x, w, values, M, N, K, Q3_BF16, stream); }, config, splits);
+  if (status) return status;
+  if (config == LIBRARY) return Q3_DECLINED;
+  if ((size_t)splits * M * N * sizeof(float) > PARTIALS_BYTES) return Q3_ERR_UNSUPPORTED;   // also a single share
+  int used = 1;
+  status = tiles::launch<bf16_t, tiles::EPI_PLAIN>(config, x, w, values, M, N, K, stream, splits, d.partials,
+                                                   tiles::RowScale(), true, &used);
+  if (status) return status;
+  const dim3 grid(q3_tiles_residual_chunks(N), M);
+  if (norm_weight_dtype == Q3_F32)
+    hipLaunchKernelGGL(tiles::tiles_residual_kernel<float>, grid, dim3(256), 0, stream, d.partials, used, residual,
+                       (const float*)norm_weight, (bf16_t*)values, sums, M, N);
+  else
+    hipLaunchKernelGGL(tiles::tiles_residual_kernel<bf16_t>, grid, dim3(256), 0, stream, d.partials, used, residual,
+                       (const bf16_t*)norm_weight, (bf16_t*)values, sums, M, N);
+  return q3_launch_status();
+}
+
+// The hand-written tiled kernel alone (gemm_tiles.h), tile shape `config` (0 .. q3_gemm_tiles_configs() - 1):
+// x (M, K) and w (N, K) bfloat16, K a multiple of 64; `epilogue` 0: out (M, N) in `out_dtype`; 1: rows of w
+// interleave gate and up, out (M, N / 2) bfloat16 = silu(gate) * up.
+extern "C" int q3_gemm_tiles_configs() { return tiles::NUM_CONFIGS; }
+
+// `splits` > 1 (plain epilogue, N a multiple of 4): K is shared out over that many blocks per tile and
+// `partials` (splits * M * N floats) takes their partial products; q3_gemm_tiles_splits says how many fill the
+// chip once.
+extern "C" int q3_gemm_tiles_splits(int config, int M, int N, int K) {
+  return tiles::takes(M, N, K) && config >= 0 && config < tiles::NUM_CONFIGS ? tiles::splits_that_fill(config, M, N, K)
+                                                                            : 1;
+}
+
+extern "C" int q3_gemm_tiles(const void* x, const void* w, void* out, int M, int N, int K, int out_dtype,
+                             int epilogue, int config, int splits, float* partials, void* stream_) {
+  if (!x || !w || !out || !tiles::takes(M, N, K)) return Q3_ERR_BAD_ARGUMENT;
+  hipStream_t stream = (hipStream_t)stream_;
+  std::lock_guard<std::mutex> hold(g_lock);   // the launchers keep a per-device flag
+  if (epilogue == tiles::EPI_SWIGLU) {
+    if (out_dtype != Q3_BF16 || N % 2) return Q3_ERR_BAD_ARGUMENT;
+    return tiles::launch<bf16_t, tiles::EPI_SWIGLU>(config, x, w, out, M, N, K, stream, splits, partials);
+  }
+  if (epilogue != tiles::EPI_PLAIN) return Q3_ERR_BAD_ARGUMENT;
+  if (out_dtype == Q3_F32)
+    return tiles::launch<float, tiles::EPI_PLAIN>(config, x, w, out, M, N, K, stream, splits, partials);
+  if (out_dtype == Q3_BF16)
+    return tiles::launch<bf16_t, tiles::EPI_PLAIN>(config, x, w, out, M, N, K, stream, splits, partials);
+  return Q3_ERR_BAD_ARGUMENT;
+}
+
+// How many of the library's candidates are timed for a new problem size (1: take its first choice).
+extern "C" int q3_matmul_set_candidates(int n) {
+  if (n < 1 || n > MAX_CANDIDATES) return Q3_ERR_BAD_ARGUMENT;
+  std::lock_guard<std::mutex> hold(g_lock);
+  g_candidates = n;
+  return 0;
+}
+
+// Which kernels enter the contest for a new size: 0 the library's and the hand-written one's (the default),
+// 1 the library's alone, 2 the hand-written ones alone where they take the size. Sizes already met keep their
+// choice. The products that carry a norm (q3_tiles_*) keep a choice for each of the three.
+extern "C" int q3_matmul_set_kernels(int mode) {
+  if (mode < KERNELS_BOTH || mode > KERNELS_OWN) return Q3_ERR_BAD_ARGUMENT;
+  std::lock_guard<std::mutex> hold(g_lock);
+  g_kernels = mode;
+  return 0;
+}
+
+// What was chosen for a size on the current device: info[0] candidates timed, info[1] index chosen,
+// info[2] microseconds of the first candidate, info[3] of the chosen one, info[4] the hand-written kernel's
+// tile shape if that was chosen, else -1, info[5] over how many blocks it shares K out. Returns 1 if the size
+// is known.
+extern "C" int q3_matmul_plan(int M, int N, int K, int out_dtype, float* info) {
+  std::lock_guard<std::mutex> hold(g_lock);
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) return 0;
+  auto d = g_devices.find(device);
+  if (d == g_devices.end()) return 0;
+  auto p = d->second.plans.find(std::make_tuple(M, N, K, out_dtype));
+  if (p == d->second.plans.end()) return 0;
+  info[0] = (float)p->second.candidates;
+  info[1] = (float)p->second.chosen;
+  info[2] = p->second.first_us;
+  info[3] = p->second.best_us;
+  info[4] = (float)p->second.own;
+  info[5] = (float)p->second.own_splits;
+  return 1;
+}
+
+extern "C" int q3_matmul(const void* x, const void* w, void* out, int M, int N, int K, int out_dtype, void* stream_) {
+  if (M <= 0 || N <= 0 || K <= 0 || !x || !w || !out) return Q3_ERR_BAD_ARGUMENT;
+  if (out_dtype != Q3_F32 && out_dtype != Q3_BF16) return Q3_ERR_BAD_ARGUMENT;
+  std::lock_guard<std::mutex> hold(g_lock);
+  int device = 0;
+  HIP_TRY(hipGetDevice(&device));
+  return product(g_devices[device], x, w, out, M, N, K, out_dtype, (hipStream_t)stream_);
 }

@@ -43,6 +43,7 @@ __all__ = [
 
 _DT = {torch.float32: 0, torch.bfloat16: 1}
 _UNSUPPORTED = 10002          # a launcher's refusal of a size it has no kernel for
+_DECLINED = 1                 # the fused product of 17 to 128 rows did nothing: the plain product is faster here
 
 
 class OperandError(ValueError):
@@ -575,7 +576,9 @@ def linear_residual_norm(x, weight, tiled, residual, norm_weight):
 
     With 17 to 128 rows (`fused_rows_take`; `tiled` is not used) the tiled kernel's partial
     products are added by a second kernel that does the same; sums is then (ceil(N / 1024), M),
-    partial sums over 1,024 columns, row m of the stream in column m."""
+    partial sums over 1,024 columns, row m of the stream in column m. There the result is None,
+    and nothing was done, for a size at which timing found the plain product (`linear`) followed
+    by the norm's own kernel faster."""
     _dev(x, weight, tiled, residual, norm_weight)
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1], "x (M, K) and weight (N, K)")
     M, K = x.shape
@@ -588,9 +591,12 @@ def linear_residual_norm(x, weight, tiled, residual, norm_weight):
         _need(x.is_contiguous(), "x must be contiguous")
         lib = library("matmul")
         sums = torch.empty((lib.q3_tiles_residual_chunks(N), M), dtype=torch.float32, device=x.device)
-        _check(lib.q3_tiles_residual(
+        status = lib.q3_tiles_residual(
             _ptr(x), _ptr(weight), M, N, K, _ptr(residual), _ptr(norm_weight), _DT[norm_weight.dtype], _ptr(values),
-            _ptr(sums), _stream()), "linear_residual_norm")
+            _ptr(sums), _stream())
+        if status == _DECLINED:
+            return None
+        _check(status, "linear_residual_norm")
         return values, sums
     _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and _tiled_ok(tiled, weight, M) and N % 16 == 0,
           "bfloat16, 1 to 16 rows, a tiled weight and a width that is a multiple of 16")

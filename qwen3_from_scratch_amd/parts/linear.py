@@ -46,5 +46,7 @@ class LinearWeight:
         if self.tiled is None or not (ops.fused_rows_take(self.weight, rows) if rows > ops.FUSED_ROWS_FEW
                                       else self.weight.shape[0] % 16 == 0):
             return self.forward(x)
-        values, sums = ops.linear_residual_norm(x, self.weight, self.tiled, sink.residual, norm.weight)
-        return UnscaledRows(values, sums, norm.eps, norm.size)
+        fused = ops.linear_residual_norm(x, self.weight, self.tiled, sink.residual, norm.weight)
+        if fused is None:                       # the kernel leaves this size to the plain product
+            return self.forward(x)
+        return UnscaledRows(fused[0], fused[1], norm.eps, norm.size)

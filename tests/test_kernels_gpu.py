@@ -666,40 +666,59 @@ def test_linear_residual_norm_and_unscaled_rows_beyond_sixteen(M, H, K, N2, norm
     assert ops.fused_rows_take(w1, M) and ops.fused_rows_take(w2, M)
 
     exact_delta = (x.double() @ w1.double().T)
-    fused_stream = residual.clone()
-    values, sums = ops.linear_residual_norm(x, w1, None, fused_stream, nw)
-    # the stream: the product rounded to bfloat16 once, then added in float32
-    stream = residual + exact_delta.float().bfloat16().float()
-    differs = fused_stream != stream
-    assert float(differs.float().mean()) < 0.02                   # roundings at a bfloat16 tie aside
-    torch.testing.assert_close(fused_stream, stream, rtol=0, atol=2 ** -7 * float(exact_delta.abs().max()))
-    stream = fused_stream
-    assert sums.shape == (-(-H // 1024), M)
-    torch.testing.assert_close(sums.double().sum(dim=0), (stream.double() ** 2).sum(dim=1), rtol=1e-5, atol=1e-6)
-    assert torch.equal(values, (stream * nw.float()).bfloat16())
+    ops.linear(_rand((20, 64), torch.bfloat16, 1), _rand((64, 64), torch.bfloat16, 2))   # the device's set-up
+    try:
+        # with the hand-written kernel alone in the contest the fusion is never declined
+        ops.matmul_kernels("own")
+        fused_stream = residual.clone()
+        values, sums = ops.linear_residual_norm(x, w1, None, fused_stream, nw)
+        # the stream: the product rounded to bfloat16 once, then added in float32
+        stream = residual + exact_delta.float().bfloat16().float()
+        differs = fused_stream != stream
+        assert float(differs.float().mean()) < 0.02               # roundings at a bfloat16 tie aside
+        torch.testing.assert_close(fused_stream, stream, rtol=0, atol=2 ** -7 * float(exact_delta.abs().max()))
+        stream = fused_stream
+        assert sums.shape == (-(-H // 1024), M)
+        torch.testing.assert_close(sums.double().sum(dim=0), (stream.double() ** 2).sum(dim=1), rtol=1e-5, atol=1e-6)
+        assert torch.equal(values, (stream * nw.float()).bfloat16())
+        # a second call gives the same bits (the choice of tile shape is kept, the additions are ordered)
+        again_stream = residual.clone()
+        v2, s2 = ops.linear_residual_norm(x, w1, None, again_stream, nw)
+        assert torch.equal(again_stream, fused_stream) and torch.equal(v2, values) and torch.equal(s2, sums)
 
-    h = ops.rmsnorm(stream.clone(), nw, eps, torch.bfloat16)
-    want = ops.linear(h, w2, out_dtype=torch.float32)
-    got = ops.linear(values, w2, out_dtype=torch.float32, unscaled=(sums, eps, H))
-    exact = (stream.double() * torch.rsqrt((stream.double() ** 2).mean(dim=1, keepdim=True) + eps) * nw.double()) @ w2.double().T
-    for m in range(M):                                             # row by row: their sizes differ
-        scale = float(exact[m].abs().max())
-        assert float((got[m] - want[m]).abs().max()) <= 6e-3 * scale
-        assert float((got[m].double() - exact[m]).abs().max()) <= 6e-3 * scale
-    got_bf16 = ops.linear(values, w2, unscaled=(sums, eps, H))
-    torch.testing.assert_close(got_bf16.float(), got, rtol=8e-3, atol=1e-3)
-    if N2 % 2 == 0:
-        want_act = torch_ops.swiglu(exact.float().bfloat16().float())
-        got_act = ops.linear_swiglu(values, w2, unscaled=(sums, eps, H))
-        assert got_act.shape == (M, N2 // 2)
-        assert float((got_act.float() - want_act).abs().max()) <= 2e-2 * max(1.0, float(want_act.abs().max()))
-    # a second call gives the same bits (the choice of tile shape is kept, the additions are ordered)
-    again_stream = residual.clone()
-    v2, s2 = ops.linear_residual_norm(x, w1, None, again_stream, nw)
-    assert torch.equal(again_stream, fused_stream) and torch.equal(v2, values) and torch.equal(s2, sums)
-    assert torch.equal(ops.linear(values, w2, out_dtype=torch.float32, unscaled=(sums, eps, H)), got)
-    with pytest.raises(ops.OperandError):                          # sums of another number of rows
-        ops.linear(values, w2, unscaled=(sums[:, :-1].contiguous(), eps, H))
+        h = ops.rmsnorm(stream.clone(), nw, eps, torch.bfloat16)
+        want = ops.linear(h, w2, out_dtype=torch.float32)
+        exact = (stream.double() * torch.rsqrt((stream.double() ** 2).mean(dim=1, keepdim=True) + eps)
+                 * nw.double()) @ w2.double().T
+        # the reader by the tiled kernel, by the contest's product with the division behind it, and by
+        # whichever of the two was faster; there the writer may leave the size to the plain product
+        for which in ("own", "library", "both"):
+            ops.matmul_kernels(which)
+            got = ops.linear(values, w2, out_dtype=torch.float32, unscaled=(sums, eps, H))
+            for m in range(M):                                     # row by row: their sizes differ
+                scale = float(exact[m].abs().max())
+                assert float((got[m] - want[m]).abs().max()) <= 6e-3 * scale, (which, m)
+                assert float((got[m].double() - exact[m]).abs().max()) <= 6e-3 * scale, (which, m)
+            assert torch.equal(ops.linear(values, w2, out_dtype=torch.float32, unscaled=(sums, eps, H)), got)
+            got_bf16 = ops.linear(values, w2, unscaled=(sums, eps, H))
+            torch.testing.assert_close(got_bf16.float(), got, rtol=8e-3, atol=1e-3)
+            if N2 % 2 == 0:
+                want_act = torch_ops.swiglu(exact.float().bfloat16().float())
+                got_act = ops.linear_swiglu(values, w2, unscaled=(sums, eps, H))
+                assert got_act.shape == (M, N2 // 2)
+                assert float((got_act.float() - want_act).abs().max()) <= 2e-2 * max(1.0, float(want_act.abs().max()))
+            other_stream = residual.clone()
+            fused = ops.linear_residual_norm(x, w1, None, other_stream, nw)
+            if fused is None:
+                assert which != "own" and torch.equal(other_stream, residual)      # declined: nothing was done
+            else:
+                # another tile shape may have won this time: other shares of K, other roundings
+                torch.testing.assert_close(other_stream, fused_stream, rtol=0, atol=2 ** -7 * float(exact_delta.abs().max()))
+                assert float((other_stream != fused_stream).float().mean()) < 0.02
+        with pytest.raises(ops.OperandError):                      # sums of another number of rows
+            ops.linear(values, w2, unscaled=(sums[:, :-1].contiguous(), eps, H))
+    finally:
+        ops.matmul_kernels("both")
 
 
 def test_linear_float32_is_true_float32():

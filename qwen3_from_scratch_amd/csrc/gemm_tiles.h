@@ -85,23 +85,53 @@ struct RowScale {
   const float* sums = nullptr;
   int chunks = 0, rows = 0;
   float eps = 0.f, inv_width = 0.f;
+  // the partial sums are asked for eight at a time (a chain of loads otherwise) and added in the chunks' order
   __device__ float of(int m) const {
     float total = 0.f;
-    for (int c = 0; c < chunks; ++c) total += sums[(size_t)c * rows + m];   // in the chunks' order
+    for (int c0 = 0; c0 < chunks; c0 += 8) {
+      float part[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) part[k] = c0 + k < chunks ? sums[(size_t)(c0 + k) * rows + m] : 0.f;
+#pragma unroll
+      for (int k = 0; k < 8; ++k)
+        if (c0 + k < chunks) total += part[k];
+    }
     return rsqrtf(total * inv_width + eps);
   }
 };
+
+// The sum of `splits` partial products' quads at `at` (`stride` floats apart), added in the splits' order; the
+// loads go out eight at a time.
+__device__ inline float4 sum_of_shares(const float* __restrict__ partials, size_t at, size_t stride, int splits) {
+  float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int s0 = 0; s0 < splits; s0 += 8) {
+    float4 part[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+      if (s0 + k < splits) part[k] = *reinterpret_cast<const float4*>(partials + (size_t)(s0 + k) * stride + at);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      if (s0 + k >= splits) continue;
+      if (s0 + k == 0) {
+        sum = part[k];
+      } else {
+        sum.x += part[k].x; sum.y += part[k].y; sum.z += part[k].z; sum.w += part[k].w;
+      }
+    }
+  }
+  return sum;
+}
 
 // A wavefront's outputs to memory: lane (col, grp) of block (i, j) holds out[m][n .. n + 3] with
 // m = m_base + 16 i + col, n = n_base + 16 j + 4 grp.
 template <typename OUT, int EPI, int MI, int NJ>
 __device__ inline void store_tile(const f32x4_t (&acc)[MI][NJ], OUT* __restrict__ out, int M, int N, int m_base,
-                                  int n_base, int col, int grp, const RowScale& scale = RowScale()) {
+                                  int n_base, int col, int grp, const float (&factor)[MI]) {
 #pragma unroll
   for (int i = 0; i < MI; ++i) {
     const int m = m_base + 16 * i + col;
     if (m >= M) continue;
-    const float r = scale.sums ? scale.of(m) : 1.f;
+    const float r = factor[i];
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
       const int n = n_base + 16 * j + 4 * grp;
@@ -225,10 +255,17 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiles_kernel(const bf16_t* 
           acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j].v, xf[i].v, acc[i][j], 0, 0, 0);
     }
   };
+  float factor[S::MI];
   {
 #pragma unroll
     for (int ahead = 0; ahead < STAGES - 1; ++ahead)
       if (ahead < steps) copy_step(first + ahead, ahead);
+    // the rows' factors while the first copies are on their way (the wait for them is one for those copies too)
+#pragma unroll
+    for (int i = 0; i < S::MI; ++i) {
+      const int m = m0 + wm * (BM / WM) + 16 * i + col;
+      factor[i] = scale.sums && m < M ? scale.of(m) : 1.f;
+    }
     for (int kt = 0; kt < steps; ++kt) {
       // step kt has landed in every thread's view, and nobody still reads the stage that the
       // next copy overwrites (step kt - 1's)
@@ -240,9 +277,9 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiles_kernel(const bf16_t* 
   }
   if (partials)   // a share of K: float32 sums for gemm_tiles_reduce_kernel
     store_tile<float, EPI_PLAIN, S::MI, S::NJ>(acc, partials + (size_t)blockIdx.y * M * N, M, N, m0 + wm * (BM / WM),
-                                               n0 + wn * (BN / WN), col, grp);
+                                               n0 + wn * (BN / WN), col, grp, factor);
   else
-    store_tile<OUT, EPI, S::MI, S::NJ>(acc, out, M, N, m0 + wm * (BM / WM), n0 + wn * (BN / WN), col, grp, scale);
+    store_tile<OUT, EPI, S::MI, S::NJ>(acc, out, M, N, m0 + wm * (BM / WM), n0 + wn * (BN / WN), col, grp, factor);
 }
 
 // out = the sum of `splits` float32 partial products (each M x N, N a multiple of 4), added in the
@@ -254,15 +291,9 @@ __global__ __launch_bounds__(256) void gemm_tiles_reduce_kernel(const float* __r
                                                                 RowScale scale) {
   const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= quads) return;
-  float4 sum = reinterpret_cast<const float4*>(partials)[i];
-  for (int s = 1; s < splits; ++s) {
-    const float4 v = reinterpret_cast<const float4*>(partials)[(size_t)s * quads + i];
-    sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
-  }
-  if (scale.sums) {
-    const float r = scale.of((int)(i / quads_per_row));
-    sum.x *= r; sum.y *= r; sum.z *= r; sum.w *= r;
-  }
+  const float r = scale.sums ? scale.of((int)(i / quads_per_row)) : 1.f;
+  float4 sum = sum_of_shares(partials, 4 * i, 4 * quads, splits);
+  sum.x *= r; sum.y *= r; sum.z *= r; sum.w *= r;
   if constexpr (SWIGLU) {
     // both rounded to the activation type first, as a separate activation kernel would have read them
     const float g0 = to_float(from_float<OUT>(sum.x)), u0 = to_float(from_float<OUT>(sum.y));
@@ -294,12 +325,8 @@ __global__ __launch_bounds__(256) void tiles_residual_kernel(const float* __rest
   float ss = 0.f;
   if (n < N) {
     const size_t at = (size_t)m * N + n;
-    float4 sum = *reinterpret_cast<const float4*>(partials + at);
-    for (int s = 1; s < splits; ++s) {
-      const float4 v = *reinterpret_cast<const float4*>(partials + (size_t)s * M * N + at);
-      sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
-    }
     float4 r = *reinterpret_cast<const float4*>(residual + at);
+    const float4 sum = sum_of_shares(partials, at, (size_t)M * N, splits);
     r.x += bf16_to_float(float_to_bf16(sum.x)); r.y += bf16_to_float(float_to_bf16(sum.y));
     r.z += bf16_to_float(float_to_bf16(sum.z)); r.w += bf16_to_float(float_to_bf16(sum.w));
     *reinterpret_cast<float4*>(residual + at) = r;

@@ -30,6 +30,12 @@
 // out over several blocks per tile, whose float32 partial products a second kernel adds in a
 // fixed order.
 //
+// For steps of some tens of rows it carries what the few-row kernel of gemm.hip carries for up
+// to sixteen: the division by the rows' root mean square that the norm before the product
+// left out (RowScale: in the epilogue, also before SwiGLU, or in the kernel that adds the
+// shares of K), and the residual addition with the next norm's preparation
+// (tiles_residual_kernel, which takes the float32 partial products, a single share too).
+//
 // K must be a multiple of 64. Rows of x beyond M and of w beyond N are read from the last
 // valid row and never written. Blocks are numbered so that the eight XCDs each take a
 // contiguous run of tiles, M fastest: the blocks that share a slice of w run on one XCD at

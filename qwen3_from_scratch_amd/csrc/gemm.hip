@@ -322,6 +322,8 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
 // 42.6 and 44.3 us at 8, 12 and 16 rows (one slab a block: 40.7, 46.1, 51.1) and the q/k/v
 // product 13.1, 14.8, 15.8 (13.5, 15.7, 17.7): used with more than eight rows, where the pairs
 // still give most CUs a block (384 slabs or more). Epilogues: plain and SwiGLU.
+// (Four slabs a block, with four or with eight k-steps a turn, were slower: a decode step at batch 16 went from
+// 4.91 to 5.32 and 5.40 ms.)
 #define PAIR_PRE 2  // fewer partial sums in flight than the one-slab kernel: the registers go to the second slab
 template <typename OUT, int EPI, bool SCALED>
 __global__ __launch_bounds__(512, 4) void gemm_skinny_pair_kernel(const bf16_t* __restrict__ x,

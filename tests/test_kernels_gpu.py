@@ -556,12 +556,12 @@ def test_linear_many_rows_by_the_hand_written_kernel_alone():
 
 @pytest.mark.parametrize("M,N,K", [(1, 6144, 4096), (8, 4096, 12288), (16, 1000, 96), (3, 331, 64), (9, 24, 2048),
                                    (5, 151936, 256), (12, 6144, 4096), (16, 24576, 512), (9, 6168, 160),
-                                   (13, 6150, 4096)])
+                                   (13, 6150, 4096), (9, 12312, 160), (11, 151936, 256), (16, 24576, 4096)])
 def test_linear_from_the_tiled_copy(M, N, K):
     """The tile-ordered copy gives the very sums of the row-major kernel: the same numbers
     are added in the same order, only their addresses differ. That holds for the kernel that
     gives two slabs to a block too (more than eight rows, 384 slabs or more; also with an odd
-    number of slabs and a last slab that is not whole)."""
+    number of slabs and a last slab that is not whole; the vocabulary's 9,496 slabs)."""
     ops = _ops()
     x = _rand((M, K), torch.bfloat16, 23)
     w = _rand((N, K), torch.bfloat16, 24, scale=0.05)

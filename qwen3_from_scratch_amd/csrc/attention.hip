@@ -536,8 +536,25 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   const int q0 = cu_q[b];
   const int q_len = cu_q[b + 1] - q0;
   if (q_len <= 0 || q_len * G > 16) return;  // the other kernel's sequence
-  if (PREP && q_len != 1) return;            // the host sends single tokens only
   const int kv_len = kv_lens[b];
+  if (PREP && (q_len != 1 || kv_len < 1)) {
+    // not a step of single tokens (the host sends no such row): the row's output is zero, and
+    // the merge finds an empty share in this block's place, not whatever the workspace held
+    for (int i = threadIdx.x; i < q_len * G * D; i += blockDim.x) {
+      const int r = i / D, d = i - r * D;
+      if (splits == 1) {
+        out[(size_t)(q0 + r / G) * Hq * D + (size_t)(g_kv * G + r % G) * D + d] = float_to_bf16(0.f);
+      } else {
+        const size_t slot = (((size_t)b * Hkv + g_kv) * splits + split) * 16 + r;
+        ws_acc[slot * D + d] = 0.f;
+        if (d == 0) {
+          ws_ml[slot * 2] = -INFINITY;
+          ws_ml[slot * 2 + 1] = 0.f;
+        }
+      }
+    }
+    return;
+  }
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, grp = lane >> 4;
   const int rows = q_len * G;
@@ -548,7 +565,6 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   const bool brings_new = fresh && split == splits - 1;  // uniform in the block
   const float* table_row = nullptr;
   if constexpr (PREP) {
-    if (first_pos < 0) return;
     if (prep.table != nullptr && first_pos < prep.max_pos) table_row = prep.table + (size_t)first_pos * D;
   }
   __shared__ float sh_k[PREP ? D : 1], sh_v[PREP ? D : 1];
@@ -586,13 +602,14 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     if (brings_new) {
       // the last two wavefronts, which have the fewest tiles, lend a few lanes: the key and the
       // value into the cache for later steps, and into shared memory for this one (the value
-      // is read after the barriers of the merge, the key by the wavefront that wrote it)
+      // is read after the barriers of the merge, the key after the barrier below)
       const int blk = first_pos / page;
       int pg = blk < bt_stride ? bt_row[blk] : -1;
       if (pg >= num_pages) pg = -1;
       store_new_key_value<D, W>(q + (size_t)q0 * q_stride, Hq, Hkv, g_kv, static_cast<const W*>(prep.k_weight),
                                 prep.eps, table_row, prep.k_cache, prep.v_cache, pg, page, first_pos % page, sh_k,
                                 sh_v);
+      __syncthreads();  // the key is in shared memory for all lanes that read it (brings_new is the block's)
       if (wave == 3) {
         float dot = 0.f;
 #pragma unroll
@@ -720,7 +737,7 @@ __global__ __launch_bounds__(256) void attn_decode_reduce_kernel(
       const float m_all = wave_max(ml.x);
       const float e = ml.x > -INFINITY ? exp2f(ml.x - m_all) : 0.f;
       const float l_all = wave_sum(ml.y * e);
-      if (lane < splits) sh_w[r][lane] = e / l_all;
+      if (lane < splits) sh_w[r][lane] = l_all > 0.f ? e / l_all : 0.f;   // a row that saw no key at all: zeros
     }
   }
   __syncthreads();

@@ -42,8 +42,40 @@ class StepBatch:
     kv_lens_host: list
 
 
+@dataclass
+class PackedLayout:
+    """Where each part of a step's description lies in its one int32 buffer, in
+    words: `pack_step` writes by it and whoever patches a packed buffer in place
+    (a graph's fixed buffer between replays) finds the parts by it."""
+
+    tokens: slice
+    positions: slice
+    seq_index: slice
+    cu_seqlens_q: slice
+    kv_lens: slice
+    state_slots: slice
+    logits_rows: slice
+    tables: list              # per group (slice, width)
+    total: int
+
+
+def packed_layout(B, T, R, widths):
+    """The layout of a step of B entries, T tokens and R wanted rows whose
+    block tables are `widths[g]` entries wide in group g."""
+    at = 0
+    parts = []
+    for n in (T, T, T, B + 1, B, B, R):
+        parts.append(slice(at, at + n))
+        at += n
+    tables = []
+    for w in widths:
+        tables.append((slice(at, at + B * w), w))
+        at += B * w
+    return PackedLayout(*parts, tables=tables, total=at)
+
+
 def packed_size(B, T, R, widths):
-    return 3 * T + (B + 1) + 2 * B + R + sum(B * w for w in widths)
+    return packed_layout(B, T, R, widths).total
 
 
 def pack_step(entries, lengths, slots, tables_per_group, device, min_table_width=1, fixed_widths=None,
@@ -54,7 +86,8 @@ def pack_step(entries, lengths, slots, tables_per_group, device, min_table_width
     `tables_per_group[g][i]`: the request's page list in group g (-1 = given back).
     `fixed_widths`: block-table widths to use instead of the longest list's.
     `buffers`: (pinned host int32 tensor, device int32 tensor) to pack into, so
-    that the batch lives at the same addresses every step (for graph replay).
+    that the batch lives at the same addresses every step (for graph replay);
+    with None for the device tensor the batch stays in the host tensor.
     `all_rows`: ask for logits at every packed row, whatever `want` says.
     Returns (StepBatch, [block table per group]).
     """
@@ -80,7 +113,8 @@ def pack_step(entries, lengths, slots, tables_per_group, device, min_table_width
                 raise ValueError("a block table is wider than the fixed width %d" % w)
     else:
         widths = [max([min_table_width] + [len(t) for t in tables]) for tables in tables_per_group]
-    total = packed_size(B, T, R, widths)
+    lay = packed_layout(B, T, R, widths)
+    total = lay.total
     if buffers is not None:
         host_t, dev_t = buffers
         if host_t.numel() < total:
@@ -88,38 +122,29 @@ def pack_step(entries, lengths, slots, tables_per_group, device, min_table_width
         host = host_t.numpy()
     else:
         host = np.empty(total, dtype=np.int32)
-    o = 0
-
-    def put(values, n):
-        nonlocal o
-        host[o:o + n] = values
-        sl = slice(o, o + n)
-        o += n
-        return sl
-
-    tok = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries]) if T else np.zeros(0, np.int64)
-    pos = np.concatenate([np.arange(lengths[i], kv[i]) for i in range(B)]) if T else np.zeros(0, np.int64)
-    seq = np.repeat(np.arange(B), q_lens) if T else np.zeros(0, np.int64)
-    s_tok = put(tok, T)
-    s_pos = put(pos, T)
-    s_seq = put(seq, T)
-    s_cu = put(np.concatenate([[0], np.cumsum(q_lens)]), B + 1)
-    s_kv = put(kv, B)
-    s_slot = put(slots, B)
-    s_rows = put(rows, R)
-    s_tables = []
-    for tables, w in zip(tables_per_group, widths):
-        flat = np.full((B, w), -1, dtype=np.int32)
+    host[lay.tokens] = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries]) if T else 0
+    host[lay.positions] = np.concatenate([np.arange(lengths[i], kv[i]) for i in range(B)]) if T else 0
+    host[lay.seq_index] = np.repeat(np.arange(B), q_lens) if T else 0
+    host[lay.cu_seqlens_q] = np.concatenate([[0], np.cumsum(q_lens)])
+    host[lay.kv_lens] = kv
+    host[lay.state_slots] = slots
+    host[lay.logits_rows] = rows
+    for tables, (sl, w) in zip(tables_per_group, lay.tables):
+        flat = host[sl].reshape(B, w)
+        flat[:] = -1
         for i, t in enumerate(tables):
             flat[i, :len(t)] = t
-        s_tables.append((put(flat.reshape(-1), B * w), w))
     if buffers is not None:
-        dev_t[:total].copy_(host_t[:total], non_blocking=True)
-        dev = dev_t
+        if dev_t is not None:
+            dev_t[:total].copy_(host_t[:total], non_blocking=True)
+        dev = dev_t if dev_t is not None else host_t
     else:
         dev = torch.from_numpy(host)
         if torch.device(device).type == "cuda":
             dev = dev.pin_memory().to(device, non_blocking=True)
+    s_tok, s_pos, s_seq, s_cu, s_kv, s_slot, s_rows, s_tables = (
+        lay.tokens, lay.positions, lay.seq_index, lay.cu_seqlens_q, lay.kv_lens, lay.state_slots, lay.logits_rows,
+        lay.tables)
     batch = StepBatch(
         num_tokens=T, num_seqs=B,
         token_ids=dev[s_tok], positions=dev[s_pos], seq_index=dev[s_seq],

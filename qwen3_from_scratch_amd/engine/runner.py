@@ -1,9 +1,12 @@
 """The step function: run a batch of (request, its next tokens) from the cache."""
 
+import contextlib
+import gc
+
 import torch
 
 from ..cache import CacheManager, CacheStorage
-from .batch import StepEntry, pack_step, packed_size
+from .batch import StepEntry, pack_step, packed_layout, packed_size
 
 
 def padded_batch(n):
@@ -21,6 +24,85 @@ def padded_batch(n):
     return size
 
 
+@contextlib.contextmanager
+def collector_paused():
+    """No object is finalized by the cyclic collector inside this block: what
+    is already dead is collected on entry, and the automatic collector is off
+    until the block ends.
+
+    A stream capture must not be interrupted by a finalizer that talks to the
+    device. The collector runs whenever enough containers have been allocated,
+    in the middle of any Python code, and finalizes whatever dead cycles it
+    finds: an engine that a caller dropped while something still pointed back
+    at it (a closure over one of its own methods is enough), and with it its
+    captured graphs. Destroying a captured graph synchronizes the device, which
+    is an error while a capture is open, and an error in a destructor ends the
+    process (SIGABRT). The same engine dropped without a cycle is freed at once
+    by its reference count, outside any capture."""
+    gc.collect()
+    was_enabled = gc.isenabled()
+    gc.disable()
+    try:
+        yield
+    finally:
+        if was_enabled:
+            gc.enable()
+
+
+class DecodeDescription:
+    """The packed description of a step of `B` rows of one token each, kept in
+    one host buffer between steps (host memory only: a graph's device twin is
+    the caller's). The first rows are the step's requests, the rest fill the
+    batch up (see `padded_batch`): token 0 at position 0 on the spare page and
+    slot. While the same requests decode on, each one token further, the buffer
+    is patched in place: tokens, positions and lengths by one, block tables in
+    their new entries; anything else packs it afresh."""
+
+    def __init__(self, B, widths, host, spare_pages, spare_slot, windowed):
+        self.B = B
+        self.widths = list(widths)
+        self.layout = packed_layout(B, B, B, self.widths)
+        self.host = host                     # int32 tensor of at least layout.total words
+        self.spare_pages = list(spare_pages)
+        self.spare_slot = spare_slot
+        self.windowed = list(windowed)       # per group: entries may turn -1 anywhere in a table
+        self.last_ids = self.last_lengths = self.last_slots = self.last_table_lens = None
+
+    def fill(self, entries, ids, lengths, slots, tables, device=None, dev=None):
+        """Bring the buffer to this step. `ids[i]` tells requests (and admissions of one request) apart.
+        Returns the StepBatch and block tables if the buffer was packed afresh, else None."""
+        fresh = None
+        if (self.last_ids is not None and ids == self.last_ids and slots == self.last_slots
+                and all(n == m + 1 for n, m in zip(lengths, self.last_lengths))):
+            self._advance(entries, tables)
+        else:
+            fill = self.B - len(entries)
+            fresh = pack_step(
+                list(entries) + [StepEntry(None, [0])] * fill, list(lengths) + [0] * fill,
+                list(slots) + [self.spare_slot] * fill,
+                [list(group) + [[self.spare_pages[g]]] * fill for g, group in enumerate(tables)],
+                device, fixed_widths=self.widths, buffers=(self.host, dev), all_rows=True)
+        self.last_ids, self.last_lengths, self.last_slots = list(ids), list(lengths), list(slots)
+        self.last_table_lens = [[len(t) for t in group] for group in tables]
+        return fresh
+
+    def _advance(self, entries, tables):
+        lay, n, host = self.layout, len(entries), self.host.numpy()
+        first = lay.tokens.start
+        host[first:first + n] = [e.tokens[0] for e in entries]
+        first = lay.positions.start
+        host[first:first + n] += 1              # the rows that fill up stay where they are
+        first = lay.kv_lens.start
+        host[first:first + n] += 1              # keys visible after the step
+        for g, (group_tables, (sl, w)) in enumerate(zip(tables, lay.tables)):
+            for i, t in enumerate(group_tables):
+                had = 0 if self.windowed[g] else self.last_table_lens[g][i]
+                if len(t) > w:
+                    raise ValueError("a block table is wider than the fixed width %d" % w)
+                if len(t) > had:
+                    host[sl.start + i * w + had: sl.start + i * w + len(t)] = t[had:]
+
+
 class _DecodeGraph:
     """A captured HIP graph of the model's forward pass for `B` rows of one
     token each, none longer than `max_kv_len`; the first rows are the step's
@@ -34,60 +116,41 @@ class _DecodeGraph:
         m = runner.manager
         self.B = B
         self.max_kv_len = max_kv_len
-        self.widths = [-(-runner.max_request_tokens // m.page_size)] * len(m.groups)
-        n = packed_size(B, B, B, self.widths)
+        widths = [-(-runner.max_request_tokens // m.page_size)] * len(m.groups)
+        n = packed_size(B, B, B, widths)
         self.host = torch.empty(n, dtype=torch.int32).pin_memory()
         self.dev = torch.zeros(n, dtype=torch.int32, device=runner.device)
+        storage = runner.storage
+        self.description = DecodeDescription(
+            B, widths, self.host, [storage.spare_page(g) for g in range(len(m.groups))], storage.spare_slot,
+            [grp.window > 0 for grp in m.groups])
         self.graph = None
         self.logits = None
         self.copied = torch.cuda.Event()
-        self.last_ids = self.last_lengths = self.last_slots = self.last_table_lens = None
 
     def run(self, runner, entries, lengths, slots, tables, device_tokens=None):
         self.copied.synchronize()          # the last step's copy has left the host buffer
         ids = [(e.request_id, runner.manager.admission(e.request_id)) for e in entries]
-        if (self.graph is not None and ids == self.last_ids and slots == self.last_slots
-                and all(n == m + 1 for n, m in zip(lengths, self.last_lengths))):
-            self._advance(runner, entries, tables)
-        else:
-            fill = self.B - len(entries)
-            storage = runner.storage
-            batch, block_tables = pack_step(
-                list(entries) + [StepEntry(None, [0])] * fill, list(lengths) + [0] * fill,
-                list(slots) + [storage.spare_slot] * fill,
-                [list(group) + [[storage.spare_page(g)]] * fill for g, group in enumerate(tables)],
-                runner.device, fixed_widths=self.widths, buffers=(self.host, self.dev), all_rows=True)
+        if self.graph is None:
+            self.description.last_ids = None
+        fresh = self.description.fill(entries, ids, lengths, slots, tables, runner.device, self.dev)
+        if fresh is None:
+            self.dev.copy_(self.host, non_blocking=True)
+        elif self.graph is None:
+            batch, block_tables = fresh
             batch.max_kv_len = self.max_kv_len
-            if self.graph is None:
-                self._capture(runner, batch, block_tables)
+            self._capture(runner, batch, block_tables)
         self.copied.record()
         if device_tokens is not None:      # the tokens are still on the device: they replace the placeholders
             self.dev[0:len(entries)].copy_(device_tokens)
-        self.last_ids, self.last_lengths, self.last_slots = ids, list(lengths), list(slots)
-        self.last_table_lens = [[len(t) for t in group] for group in tables]
         self.graph.replay()
         return self.logits
 
-    def _advance(self, runner, entries, tables):
-        """The same requests (and admissions of them) as in the last step, each one token further: the
-        packed description changes in its tokens, by one in positions and
-        lengths, and in the block tables' new entries (all entries where a
-        window gives pages back)."""
-        B, n, host = self.B, len(entries), self.host.numpy()
-        host[0:n] = [e.tokens[0] for e in entries]
-        host[B:B + n] += 1                        # positions (the rows that fill up stay where they are)
-        host[4 * B + 1:4 * B + 1 + n] += 1        # keys visible after the step
-        base = 7 * B + 1
-        for g, (group_tables, w) in enumerate(zip(tables, self.widths)):
-            windowed = runner.manager.groups[g].window > 0
-            for i, t in enumerate(group_tables):
-                had = 0 if windowed else self.last_table_lens[g][i]
-                if len(t) > w:
-                    raise ValueError("a block table is wider than the fixed width %d" % w)
-                if len(t) > had:
-                    host[base + i * w + had: base + i * w + len(t)] = t[had:]
-            base += B * w
-        self.dev.copy_(self.host, non_blocking=True)
+    def retire(self, device):
+        """Before the graph and its buffers are let go: its last replay has ended, and so has
+        whatever was queued behind it to read its logits (the sampler of a step that is still
+        on its way)."""
+        torch.cuda.synchronize(device)
 
     def _capture(self, runner, batch, block_tables):
         runner.storage.bind(block_tables)
@@ -99,8 +162,9 @@ class _DecodeGraph:
         torch.cuda.current_stream(runner.device).wait_stream(side)
         torch.cuda.synchronize(runner.device)
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            self.logits = runner.model.forward(batch, runner.storage)
+        with collector_paused():
+            with torch.cuda.graph(graph):
+                self.logits = runner.model.forward(batch, runner.storage)
         self.graph = graph
 
 
@@ -198,8 +262,8 @@ class ModelRunner:
         bucket = min(bucket, self.max_request_tokens)
         graph = self._graphs.pop((rows, bucket), None)
         if graph is None:
-            if len(self._graphs) >= self.max_graphs:       # drop the one used longest ago
-                self._graphs.pop(next(iter(self._graphs)))
+            if len(self._graphs) >= self.max_graphs:       # drop the one used longest ago, once it is idle
+                self._graphs.pop(next(iter(self._graphs))).retire(self.device)
             graph = _DecodeGraph(self, rows, bucket)
         self._graphs[(rows, bucket)] = graph                # most recently used last
         logits = graph.run(self, entries, lengths, slots, tables, device_tokens)

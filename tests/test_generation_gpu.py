@@ -100,6 +100,56 @@ def test_a_step_ahead_changes_no_token(model_folders, name, dtype, block_size, n
         assert sum(preempted) > 0
 
 
+def test_a_dropped_engine_in_a_cycle_is_freed_before_the_next_capture(model_folders):
+    """An engine that is dropped while something points back at it is only found by the cyclic
+    collector, which must not finalize its captured graphs while another capture is open
+    (destroying a graph synchronizes the device): the capture collects what is dead first and
+    keeps the collector off until it ends."""
+    import gc
+    import weakref
+
+    kw = dict(path=model_folders["D"], dtype="bfloat16", block_size=16, num_blocks=12, max_num_seqs=2)
+
+    def first():
+        engine = SyncEngine(**kw)
+        engine.myself = engine                       # the cycle
+        tokens = engine.generate_ids([[1, 2, 3]], 6, temperature=0.0, ignore_eos=True)
+        assert engine.runner._graphs
+        return weakref.ref(engine.runner), tokens
+
+    gc.collect()
+    gc.disable()                                     # only the capture's own collection can find it
+    try:
+        gone, tokens = first()
+        assert gone() is not None
+        second = SyncEngine(**kw)
+        assert second.generate_ids([[1, 2, 3]], 6, temperature=0.0, ignore_eos=True) == tokens
+        assert gone() is None
+        assert not gc.isenabled()
+    finally:
+        gc.enable()
+
+
+def test_more_graphs_than_are_kept(model_folders):
+    """With room for two graphs, batches of one to four requests and a step ahead: the graph used
+    longest ago goes each time a new one comes, after the work that still reads it has ended;
+    tokens are those of an engine that keeps them all."""
+    vocab = TINY["D"]["config"]["vocab_size"]
+    prompts = [random_tokens(n, vocab, 70 + n) for n in (5, 9, 13, 17)]
+    kw = dict(path=model_folders["D"], dtype="bfloat16", block_size=16, num_blocks=40, max_num_seqs=4)
+
+    def run(max_graphs):
+        engine = SyncEngine(**kw)
+        engine.runner.max_graphs = max_graphs
+        out = []
+        for count in (1, 2, 3, 4, 2, 1, 4, 3):
+            out.append(engine.generate_ids(prompts[:count], 5, temperature=0.7, top_k=8, seed=5, ignore_eos=True))
+            assert len(engine.runner._graphs) <= max_graphs
+        return out
+
+    assert run(2) == run(32)
+
+
 def _replay(folder, dtype, steps, out, max_tokens):
     lines = []
     for i, (entries, ends) in enumerate(steps):

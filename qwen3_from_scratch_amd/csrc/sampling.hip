@@ -2,8 +2,11 @@
 // temperature, optionally among the k best, as the arg-max of
 // logit / temperature + Gumbel noise.
 #include "common.h"
+#include "sampling.h"
 
 #include <math.h>
+
+#include <mutex>
 
 // Philox-4x32 with 10 rounds (Salmon et al., "Parallel random numbers: as easy
 // as 1, 2, 3"): a counter-based generator, so the noise of (seed, counter,
@@ -181,13 +184,9 @@ extern "C" long q3_sample_workspace(int R, int V) {
   return (long)R * q3_sample_chunks(V) * (long)sizeof(Best) + (long)R * (long)sizeof(uint32_t);
 }
 
-// `with_top_k`: 0 if the caller knows that no row restricts its draw (the select is skipped).
-// `workspace`: q3_sample_workspace(R, V) bytes, 8-byte aligned.
-extern "C" int q3_sample(const float* logits, const float* temperature, const int* top_k,
-                         const long long* seed, const int* counter, int* out, int R, int V,
-                         int with_top_k, void* workspace, hipStream_t stream) {
-  if (R <= 0 || V <= 0 || workspace == nullptr) return Q3_ERR_BAD_ARGUMENT;
-  if (R > 65535) return Q3_ERR_UNSUPPORTED;
+static int launch_sample(const float* logits, const float* temperature, const int* top_k, const long long* seed,
+                         const int* counter, int* out, int R, int V, int with_top_k, void* workspace,
+                         hipStream_t stream) {
   const int chunks = q3_sample_chunks(V);
   const int chunk = ((V + chunks - 1) / chunks + 3) / 4 * 4;
   Best* partial = static_cast<Best*>(workspace);
@@ -202,4 +201,50 @@ extern "C" int q3_sample(const float* logits, const float* temperature, const in
                      with_top_k ? threshold : nullptr, partial, V, chunk);
   hipLaunchKernelGGL(sample_final_kernel, dim3(R), dim3(64), 0, stream, partial, chunks, out, V);
   return q3_launch_status();
+}
+
+// `with_top_k`: 0 if the caller knows that no row restricts its draw (the select is skipped).
+// `workspace`: q3_sample_workspace(R, V) bytes, 8-byte aligned.
+extern "C" int q3_sample(const float* logits, const float* temperature, const int* top_k,
+                         const long long* seed, const int* counter, int* out, int R, int V,
+                         int with_top_k, void* workspace, hipStream_t stream) {
+  if (R <= 0 || V <= 0 || workspace == nullptr) return Q3_ERR_BAD_ARGUMENT;
+  if (R > 65535) return Q3_ERR_UNSUPPORTED;
+  return launch_sample(logits, temperature, top_k, seed, counter, out, R, V, with_top_k, workspace, stream);
+}
+
+// ---- the same without a workspace from the caller (see sampling.h) ------------------------
+// The chunks' candidates and the rows' thresholds live in this array, one copy on every GPU that
+// loads the library, held until the process ends. Host code never uses the array's name as an
+// address: it asks each device for its copy's address once and passes that to the kernels.
+static __device__ __align__(256) unsigned char scratch[Q3_SAMPLE_STATIC_BYTES];
+
+#define Q3_MAX_DEVICES 64
+static std::mutex scratch_lock;
+static void* scratch_of_device[Q3_MAX_DEVICES];   // null until the device's first call
+
+extern "C" int q3_sample_static(const float* logits, const float* temperature, const int* top_k,
+                                const long long* seed, const int* counter, int* out, int R, int V,
+                                int with_top_k, hipStream_t stream) {
+  if (R <= 0 || V <= 0 || !logits || !temperature || !top_k || !seed || !counter || !out) return Q3_ERR_BAD_ARGUMENT;
+  if (R > 65535 || q3_sample_workspace(R, V) > (long)Q3_SAMPLE_STATIC_BYTES) return Q3_ERR_UNSUPPORTED;
+  int device = 0;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return (int)e;
+  if (device < 0 || device >= Q3_MAX_DEVICES) return Q3_ERR_UNSUPPORTED;
+  void* workspace = nullptr;
+  {
+    std::lock_guard<std::mutex> hold(scratch_lock);
+    if (scratch_of_device[device] == nullptr) {   // this device's copy of the array, asked for with it current
+      void* ptr = nullptr;
+      e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+      if (e != hipSuccess) return (int)e;
+      if (ptr == nullptr) return Q3_ERR_UNSUPPORTED;
+      scratch_of_device[device] = ptr;
+    }
+    workspace = scratch_of_device[device];
+  }
+  // every word the kernels read from the array they have written in this call (a candidate per
+  // row and chunk, a threshold per row where a selection is asked for): nothing needs clearing
+  return launch_sample(logits, temperature, top_k, seed, counter, out, R, V, with_top_k, workspace, stream);
 }

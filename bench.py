@@ -54,6 +54,29 @@ def prefill_flops(c, tokens):
     return gemm + attn
 
 
+def _model_tensors(model):
+    """Every tensor a loaded model keeps on the device, each once."""
+    import torch
+
+    seen, found, stack = set(), [], [model]
+    while stack:
+        obj = stack.pop()
+        if id(obj) in seen:
+            continue
+        seen.add(id(obj))
+        if isinstance(obj, torch.Tensor):
+            if obj.is_cuda and obj.untyped_storage().data_ptr() not in seen:
+                seen.add(obj.untyped_storage().data_ptr())
+                found.append(obj)
+        elif isinstance(obj, (list, tuple)):
+            stack.extend(obj)
+        elif isinstance(obj, dict):
+            stack.extend(obj.values())
+        elif hasattr(obj, "__dict__") and type(obj).__module__.startswith("qwen3_from_scratch_amd"):
+            stack.extend(vars(obj).values())
+    return found
+
+
 def continuous(args, config, model, shape_name, gen, sync):
     """64 requests admitted at once and served by continuous batching: prompt lengths uniform in
     [128, 4096], generated tokens uniform in [64, 512], prompts cut into portions of 512 beside
@@ -327,14 +350,17 @@ def main():
     need = decode_bytes(config, contexts, itemsize)
     roofline = {"bound": "hbm", "achieved": round(need / step_s / 1e9, 1), "peak": PEAK_HBM / 1e9,
                 "unit": "GB/s", "frac": round(need / step_s / PEAK_HBM, 4)}
-    points = {}
+    points, points_roofline = {}, {}
     if not args.no_points:
         for b in (1, 64):
             if b == args.batch:
                 points["decode_b%d" % b] = round(tps, 1)
+                points_roofline["decode_b%d" % b] = roofline["frac"]
                 continue
-            p_tps, _, _ = decode(b, max(16, args.steps // 4), max(4, args.warmup // 2))
+            p_tps, p_step_s, p_contexts = decode(b, max(16, args.steps // 4), max(4, args.warmup // 2))
             points["decode_b%d" % b] = round(p_tps, 1)
+            points_roofline["decode_b%d" % b] = round(decode_bytes(config, p_contexts, itemsize) / p_step_s / PEAK_HBM, 4)
+    resident = sum(t.untyped_storage().nbytes() for t in _model_tensors(model))
 
     line = {
         "metric": "decode tok/s at batch 1/8/64 + prefill tok/s at 2048 tokens, %s %s"
@@ -352,6 +378,10 @@ def main():
             "tie_word_embeddings": config.tie_word_embeddings, "kv_block_size": BLOCK, "sampling": "greedy",
         },
         "prefill": prefill, "roofline": roofline, "points": points,
+        # the same fraction of the HBM peak for the other batch sizes; what the weights hold on the GPU (bfloat16
+        # matrices are kept twice, row-major and in the few-row kernel's order); how many-row products get their kernels
+        "points_roofline": points_roofline, "resident_weight_gb": round(resident / 1e9, 2),
+        "matmul_choice": "table and rule, no timing",
     }
     print(json.dumps(line))
     return 0

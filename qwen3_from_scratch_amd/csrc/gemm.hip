@@ -5,15 +5,17 @@
 // float32: plain fused multiply-adds, no matrix-core mode of reduced precision.
 // A block of 256 threads computes a 64 x 64 tile of out; each thread a 4 x 4
 // patch, summing over k in ascending order, so an output element's value does
-// not depend on which rows share its batch.
+// not depend on which rows share its batch. The same kernel with bfloat16
+// operands (read one by one, summed in float32) serves bfloat16 products of any
+// size that no matrix-core kernel takes: an inner size that is no multiple of 8.
 // ---------------------------------------------------------------------------
 #define F32_BM 64
 #define F32_BN 64
 #define F32_BK 16
 
-__global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__ a,
-                                                       const float* __restrict__ w,
-                                                       float* __restrict__ out, int M, int N, int K) {
+template <typename IN, typename OUT>
+__global__ __launch_bounds__(256) void gemm_f32_kernel(const IN* __restrict__ a, const IN* __restrict__ w,
+                                                       OUT* __restrict__ out, int M, int N, int K) {
   __shared__ float as[F32_BK][F32_BM + 4];
   __shared__ float ws[F32_BK][F32_BN + 4];
   const int t = threadIdx.x;
@@ -24,7 +26,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
   // loader coordinates: 64 rows x 16 k per tile, 4 elements per thread
   const int lr = t / 4;          // row 0..63
   const int lk = (t % 4) * 4;    // k offset 0, 4, 8, 12
-  const bool vec = (K % 4) == 0;
+  const bool vec = sizeof(IN) == 4 && (K % 4) == 0;
   float acc[4][4];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
@@ -35,25 +37,25 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
     float av[4] = {0.f, 0.f, 0.f, 0.f}, wv[4] = {0.f, 0.f, 0.f, 0.f};
     const int gm = m0 + lr, gn = n0 + lr, gk = k0 + lk;
     if (gm < M) {
-      const float* p = a + (size_t)gm * K + gk;
+      const IN* p = a + (size_t)gm * K + gk;
       if (vec && gk + 3 < K) {
         const float4 v = *reinterpret_cast<const float4*>(p);
         av[0] = v.x; av[1] = v.y; av[2] = v.z; av[3] = v.w;
       } else {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          if (gk + i < K) av[i] = p[i];
+          if (gk + i < K) av[i] = to_float(p[i]);
       }
     }
     if (gn < N) {
-      const float* p = w + (size_t)gn * K + gk;
+      const IN* p = w + (size_t)gn * K + gk;
       if (vec && gk + 3 < K) {
         const float4 v = *reinterpret_cast<const float4*>(p);
         wv[0] = v.x; wv[1] = v.y; wv[2] = v.z; wv[3] = v.w;
       } else {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          if (gk + i < K) wv[i] = p[i];
+          if (gk + i < K) wv[i] = to_float(p[i]);
       }
     }
     __syncthreads();
@@ -83,7 +85,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int gn = n0 + tn + j;
-      if (gn < N) out[(size_t)gm * N + gn] = acc[i][j];
+      if (gn < N) out[(size_t)gm * N + gn] = from_float<OUT>(acc[i][j]);
     }
   }
 }
@@ -563,11 +565,22 @@ extern "C" int q3_linear(const void* x, const void* weight, void* out, int M, in
     }
     const dim3 grid((N + F32_BN - 1) / F32_BN, (M + F32_BM - 1) / F32_BM);
     if (grid.y > 65535) return Q3_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL(gemm_f32_kernel, grid, dim3(256), 0, stream, (const float*)x, (const float*)weight,
-                       (float*)out, M, N, K);
+    hipLaunchKernelGGL((gemm_f32_kernel<float, float>), grid, dim3(256), 0, stream, (const float*)x,
+                       (const float*)weight, (float*)out, M, N, K);
     return q3_launch_status();
   }
-  if (!q3_linear_is_skinny(M, N, K, in_dtype)) return Q3_ERR_UNSUPPORTED;
+  if (in_dtype != Q3_BF16 || (out_dtype != Q3_F32 && out_dtype != Q3_BF16)) return Q3_ERR_BAD_ARGUMENT;
+  if (!q3_linear_is_skinny(M, N, K, in_dtype)) {   // any size, by plain multiply-adds
+    const dim3 grid((N + F32_BN - 1) / F32_BN, (M + F32_BM - 1) / F32_BM);
+    if (grid.y > 65535) return Q3_ERR_UNSUPPORTED;
+    if (out_dtype == Q3_F32)
+      hipLaunchKernelGGL((gemm_f32_kernel<bf16_t, float>), grid, dim3(256), 0, stream, (const bf16_t*)x,
+                         (const bf16_t*)weight, (float*)out, M, N, K);
+    else
+      hipLaunchKernelGGL((gemm_f32_kernel<bf16_t, bf16_t>), grid, dim3(256), 0, stream, (const bf16_t*)x,
+                         (const bf16_t*)weight, (bf16_t*)out, M, N, K);
+    return q3_launch_status();
+  }
   return out_dtype == Q3_F32 ? launch_skinny<float, EPI_PLAIN>(x, weight, out, M, N, K, stream)
                              : launch_skinny<bf16_t, EPI_PLAIN>(x, weight, out, M, N, K, stream);
 }

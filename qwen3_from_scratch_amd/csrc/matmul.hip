@@ -1,30 +1,38 @@
 // Matrix products with many rows, out[M, N] = x[M, K] . w[N, K]^T in bfloat16
-// with float32 accumulation, through the vendor library (hipBLASLt), as the
+// with float32 accumulation, by the vendor library (hipBLASLt), as the
 // reference's engine uses its vendor library for them
-// (src/qwen3_from_scratch/models/linear.py:24-31 calls F.linear).
+// (src/qwen3_from_scratch/models/linear.py:24-31 calls F.linear), or by the
+// hand-written tiled kernel (gemm_tiles.h).
 //
-// The library's heuristic returns a ranked list of kernels for a problem; its
-// first choice is often not its fastest (for 576 x 5120 x 17408 the first took
-// 108 us and the fourth 92; for 2048 x 4096 x 4096, 101 against 55). The first
-// time a problem size is seen outside a graph capture, the leading candidates
-// are timed on the caller's own operands and the fastest is kept for the life
-// of the process. A size first seen during a capture runs the first candidate
-// and is tuned at its next eager call. In the model every weight is read once
-// a step, with gigabytes of other traffic in between, so a candidate is timed
-// with cold caches: a kernel that reads a buffer larger than the last-level
-// cache runs before each timed run. Timed warm, products of few rows pick
-// kernels that are the fastest only while the weight sits in that cache.
+// Which kernel serves a size is decided without a stopwatch: the same size gets
+// the same kernel in every process and on every box, so a product's bits are
+// reproducible. The decision is, in this order,
+//   1. an entry of the table that the caller loaded (q3_matmul_table_add): a
+//      place in the library's ranked list of candidates for the size, or a tile
+//      shape of the hand-written kernel with a number of shares of K; the table is
+//      data made beforehand by the tuner below, keyed by (kind of product, rows
+//      rounded up, N, K, output type);
+//   2. a rule of thumb: the library's first candidate for a plain product; for
+//      the products of 17 to 128 rows that carry a norm the 64 x 128 tiles with
+//      K shared out until the chip is full, unless those tiles fit the chip badly.
+// The library's list is asked for the exact size every time, so a kernel is
+// never run on a size the library has not offered it for.
 //
-// The hand-written tiled kernel (gemm_tiles.h) stands in the same contest: where it takes a
-// size (K a multiple of 64) two or three of its tile shapes, chosen by the rows, are timed after
-// the library's candidates, each also with K shared out over several blocks per tile where its
-// tiles alone would not fill the chip, and a size goes to whichever kernel was the fastest. q3_matmul_set_kernels narrows the
-// contest to the library's kernels alone, or to the hand-written ones where they take the size.
+// The tuner (q3_matmul_set_mode(1), off unless asked for) is what the table is
+// made with: a size first met outside a graph capture has its candidates timed
+// on the caller's own operands, the library's leading ones and the tile shapes
+// that fit the rows, each also with K shared out where its tiles alone would not
+// fill the chip, and the fastest is kept for the life of the process
+// (q3_matmul_plan and q3_matmul_fused_plan tell what it was). In the model every
+// weight is read once a step, with gigabytes of other traffic in between, so a
+// candidate is timed with cold caches: a kernel that reads a buffer larger than
+// the last-level cache runs before each timed run.
 //
-// One workspace, one such buffer and one buffer for the hand-written kernel's partial products
-// per device, allocated at first need and kept. Calls on one
-// device share it and the plans: they are serialised by a lock and are meant
-// to come from one stream at a time.
+// One workspace, one buffer for the tiled kernel's partial products and one
+// staging buffer per device, allocated by q3_matmul_init (the engine calls it
+// when a model is built) or at the first product outside a capture. Calls on one
+// device share them and the plans: they are serialised by a lock and are meant to
+// come from one stream at a time.
 
 #include "common.h"
 #include "gemm_tiles.h"
@@ -37,16 +45,17 @@
 #include <vector>
 
 #define Q3_ERR_LIBRARY 20000   // + the library's status
-#define Q3_DECLINED 1          // q3_tiles_residual: nothing was done, the caller's other way is faster
+#define Q3_DECLINED 1          // q3_tiles_residual: nothing was done, the caller's other way is the one for this size
 
 namespace {
 
 constexpr size_t WORKSPACE_BYTES = 128u << 20;
-constexpr size_t EVICT_BYTES = 512u << 20;     // twice the 256 MB last-level cache
+constexpr size_t EVICT_BYTES = 512u << 20;     // twice the 256 MB last-level cache (the tuner's)
 constexpr size_t PARTIALS_BYTES = 128u << 20;  // float32 partial products of the hand-written kernel's K shares
 constexpr size_t STAGING_BYTES = 64u << 20;
 constexpr int EVICT_BLOCKS = 2048, EVICT_THREADS = 256;
 constexpr int MAX_CANDIDATES = 64;
+constexpr int LIBRARY = -1;                    // a Choice's `own` when the library serves the size
 
 // Reads the whole buffer; the store never happens (the buffer holds zeros) but keeps the loads alive.
 __global__ void evict_kernel(float4* buffer, size_t count) {
@@ -58,16 +67,29 @@ __global__ void evict_kernel(float4* buffer, size_t count) {
   if (sum == 12345.f) buffer[0].x = sum;
 }
 
+// The kinds of product a choice is made for.
+enum { KIND_PLAIN = 0, KIND_SCALED = 1, KIND_SCALED_SWIGLU = 2, KIND_RESIDUAL = 3 };
+
+// Who serves a size: the library's candidate number `library` (own == LIBRARY), or the hand-written kernel's
+// tile shape `own` with K shared out over `splits` blocks per tile.
+struct Choice {
+  int library = 0;
+  int own = LIBRARY;
+  int splits = 1;
+};
+
 struct Plan {
   hipblasLtMatmulDesc_t desc = nullptr;
   hipblasLtMatrixLayout_t w = nullptr, x = nullptr, out = nullptr;
   hipblasLtMatmulAlgo_t algo;
-  bool tuned = false;
-  int own = -1;            // the hand-written kernel's tile shape, if that was chosen; else `algo`
-  int own_splits = 1;      // and over how many blocks it shares K out
+  bool ready = false;      // the choice is made (and, for the library, its kernel found)
+  bool timed = false;      // by the tuner
+  Choice choice;
   int candidates = 0, chosen = 0;
   float first_us = 0.f, best_us = 0.f;
 };
+
+typedef std::tuple<int, int, int, int, int> Key;   // kind (+ 4 * which kernels, for the tuner's notes), rows, N, K, output type
 
 struct Device {
   hipblasLtHandle_t handle = nullptr;
@@ -76,35 +98,25 @@ struct Device {
   float* partials = nullptr;
   float* staging = nullptr;   // a float32 product on its way to the kernel that divides its rows (q3_tiles_scaled)
   hipEvent_t begin = nullptr, end = nullptr;
-  std::map<std::tuple<int, int, int, int>, Plan> plans;
-  // what was chosen for a size, by its rows rounded up to a multiple of 32: sizes beyond 64
-  // rows that differ only within such a step take the choice of the first one that was timed
-  // (a serving loop meets dozens of them, a prompt's portion plus however many requests decode)
-  std::map<std::tuple<int, int, int, int>, Plan> chosen_near;
-  // (kind, M, N, K) -> (tile shape, shares of K) of the products that carry a norm (q3_tiles_*)
-  std::map<std::tuple<int, int, int, int>, std::pair<int, int>> fused;
+  std::map<std::tuple<int, int, int, int>, Plan> plans;   // by the exact size
+  std::map<Key, Choice> noted;                            // what the tuner found, by rounded rows
 };
-
-int rows_class(int M) { return M <= 64 ? M : (M + 31) / 32 * 32; }
 
 std::mutex g_lock;
 std::map<int, Device> g_devices;
+std::map<Key, Choice> g_table;
 int g_candidates = 16;
 enum { KERNELS_BOTH = 0, KERNELS_LIBRARY = 1, KERNELS_OWN = 2 };
 int g_kernels = KERNELS_BOTH;
-// The tile shapes that enter the contest, by the product's rows (the others never won a size of the 8B, 14B
-// and 32B models there): small tiles with three stages where the weights' passage bounds the product, the
-// largest where the matrix units do. Each enters a second time with K shared out where its tiles alone would
-// not fill the chip.
-constexpr int OWN_FEW_ROWS[] = {1, 5}, OWN_SOME_ROWS[] = {0, 1, 2}, OWN_MANY_ROWS[] = {0, 2, 4};
-constexpr int MAX_OWN = 6;
-inline const int* own_shapes(int M, int& count) {
-  if (M <= 256) {
-    count = 2;
-    return OWN_FEW_ROWS;
-  }
-  count = 3;
-  return M <= 1024 ? OWN_SOME_ROWS : OWN_MANY_ROWS;
+enum { MODE_RULE = 0, MODE_TUNE = 1 };
+int g_mode = MODE_RULE;
+
+// Sizes that differ only within a step of rows share a table entry (a serving loop meets dozens of them, a
+// prompt's portion plus however many requests decode): plain products up to 64 rows by their own count, beyond
+// in steps of 32; the products that carry a norm in steps of 8.
+int rows_key(int kind, int M) {
+  if (kind != KIND_PLAIN) return (M + 7) / 8 * 8;
+  return M <= 64 ? M : (M + 31) / 32 * 32;
 }
 
 #define HIP_TRY(call)                    \
@@ -117,6 +129,42 @@ inline const int* own_shapes(int M, int& count) {
     hipblasStatus_t s_ = (call);                                  \
     if (s_ != HIPBLAS_STATUS_SUCCESS) return Q3_ERR_LIBRARY + (int)s_; \
   } while (0)
+
+bool capturing(hipStream_t stream, int& status) {
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  status = (int)hipStreamIsCapturing(stream, &capture);
+  return capture != hipStreamCaptureStatusNone;
+}
+
+// The device's handle and buffers. Not inside a capture: it allocates.
+int set_up(Device& d) {
+  if (!d.workspace) HIP_TRY(hipMalloc(&d.workspace, WORKSPACE_BYTES));
+  if (!d.partials) HIP_TRY(hipMalloc((void**)&d.partials, PARTIALS_BYTES));
+  if (!d.staging) HIP_TRY(hipMalloc((void**)&d.staging, STAGING_BYTES));
+  if (!d.handle) LT_TRY(hipblasLtCreate(&d.handle));
+  return 0;
+}
+
+int ready_device(Device& d, hipStream_t stream) {
+  if (d.handle && d.workspace && d.partials && d.staging) return 0;
+  int status = 0;
+  if (capturing(stream, status)) return (int)hipErrorStreamCaptureUnsupported;   // set-up allocates
+  if (status) return status;
+  return set_up(d);
+}
+
+// The tuner's own: events and the buffer that empties the caches.
+int set_up_tuner(Device& d, hipStream_t stream) {
+  if (!d.begin) {
+    HIP_TRY(hipEventCreate(&d.begin));
+    HIP_TRY(hipEventCreate(&d.end));
+  }
+  if (!d.evict) {
+    HIP_TRY(hipMalloc(&d.evict, EVICT_BYTES));
+    HIP_TRY(hipMemsetAsync(d.evict, 0, EVICT_BYTES, stream));
+  }
+  return 0;
+}
 
 int describe(Plan& p, int M, int N, int K, int out_dtype) {
   // Row-major x (M, K), w (N, K), out (M, N) are column-major (K, M), (K, N), (N, M):
@@ -140,9 +188,26 @@ void forget(Plan& p) {
   p = Plan();
 }
 
+// The library's ranked candidates for the plan's exact size, at most `want` of them.
+int candidates_of(Device& d, const Plan& p, int want, std::vector<hipblasLtMatmulHeuristicResult_t>& found) {
+  hipblasLtMatmulPreference_t pref = nullptr;
+  LT_TRY(hipblasLtMatmulPreferenceCreate(&pref));
+  size_t bytes = WORKSPACE_BYTES;
+  hipblasStatus_t s = hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &bytes,
+                                                            sizeof(bytes));
+  found.assign(want, hipblasLtMatmulHeuristicResult_t());
+  int got = 0;
+  if (s == HIPBLAS_STATUS_SUCCESS)
+    s = hipblasLtMatmulAlgoGetHeuristic(d.handle, p.desc, p.w, p.x, p.out, p.out, pref, want, found.data(), &got);
+  (void)hipblasLtMatmulPreferenceDestroy(pref);
+  if (s != HIPBLAS_STATUS_SUCCESS) return Q3_ERR_LIBRARY + (int)s;
+  found.resize(got);
+  return got == 0 ? Q3_ERR_UNSUPPORTED : 0;
+}
+
 int run_own(Device& d, int config, int splits, const void* x, const void* w, void* out, int M, int N, int K,
             int out_dtype, hipStream_t stream) {
-  if (splits > 1 && (!d.partials || (size_t)splits * M * N * sizeof(float) > PARTIALS_BYTES)) return Q3_ERR_UNSUPPORTED;
+  if (splits > 1 && (size_t)splits * M * N * sizeof(float) > PARTIALS_BYTES) return Q3_ERR_UNSUPPORTED;
   return out_dtype == Q3_F32
              ? tiles::launch<float, tiles::EPI_PLAIN>(config, x, w, out, M, N, K, stream, splits, d.partials)
              : tiles::launch<bf16_t, tiles::EPI_PLAIN>(config, x, w, out, M, N, K, stream, splits, d.partials);
@@ -153,6 +218,84 @@ hipblasStatus_t run(Device& d, const Plan& p, const hipblasLtMatmulAlgo_t& algo,
   const float one = 1.f, zero = 0.f;
   return hipblasLtMatmul(d.handle, p.desc, &one, w, p.w, x, p.x, &zero, out, p.out, out, p.out, &algo, d.workspace,
                          WORKSPACE_BYTES, stream);
+}
+
+// ---- the rules of thumb ----------------------------------------------------------------------
+
+// The hand-written kernel's shape for a plain product, by its rows: small tiles with three stages where the
+// weights' passage bounds the product, the largest where the matrix units do; K shared out where the tiles
+// alone would not fill the chip.
+Choice own_by_rule(int M, int N, int K) {
+  Choice c;
+  c.own = M <= 256 ? 5 : (M <= 1024 ? 1 : 4);
+  c.splits = M <= 1024 ? tiles::splits_that_fill(c.own, M, N, K) : 1;
+  if ((size_t)c.splits * M * N * sizeof(float) > PARTIALS_BYTES) c.splits = 1;
+  return c;
+}
+
+Choice plain_by_rule(int M, int N, int K) {
+  if (g_kernels == KERNELS_OWN && tiles::takes(M, N, K)) return own_by_rule(M, N, K);
+  if (g_kernels == KERNELS_BOTH && tiles::takes(M, N, K) && M >= 32 && M <= 640 && K >= 2 * N && N % 4 == 0) {
+    // few output tiles and a long inner size (a feed-forward's way down with some hundreds of rows): the
+    // library's kernels leave most of the chip idle there, the tiled kernel shares K out over the idle CUs
+    // (4,096 x 12,288 at 64, 256 and 576 rows: 29, 47 and 81 us against the library's best 38, 58 and 99)
+    Choice c;
+    c.own = M <= 256 ? 1 : 0;
+    c.splits = tiles::splits_that_fill(c.own, M, N, K);
+    if (c.splits > 1 && (size_t)c.splits * M * N * sizeof(float) <= PARTIALS_BYTES) return c;
+  }
+  return Choice();   // the library's first candidate
+}
+
+// The products of 17 to 128 rows that carry a norm: 64 x 128 tiles in five stages (with K shared out they need
+// the fewest shares to fill the chip), unless the tiles come to a little more than a whole number of rounds over
+// the 256 CUs and leave most of them idle in the last one: then the library's product with the norm's work in a
+// kernel behind it (for KIND_RESIDUAL: declined, the caller's plain product and the norm's own kernel).
+Choice fused_by_rule(int kind, int M, int N, int K) {
+  (void)kind;
+  Choice c;
+  if (g_kernels == KERNELS_LIBRARY) return c;
+  c.own = 8;
+  c.splits = tiles::splits_that_fill(8, M, N, K);
+  if ((size_t)c.splits * ((M + 7) / 8 * 8) * N * sizeof(float) > PARTIALS_BYTES) c.splits = 1;
+  if (g_kernels == KERNELS_BOTH && c.splits == 1) {
+    const long tiles_n = (long)((M + 63) / 64) * ((N + 127) / 128);
+    const long rounds = (tiles_n + 255) / 256;
+    if (tiles_n < rounds * 256 * 7 / 10) return Choice();
+  }
+  return c;
+}
+
+// What the table or the rule says for a size.
+Choice choice_for(int kind, int M, int N, int K, int out_dtype) {
+  if (g_kernels == KERNELS_BOTH) {
+    auto entry = g_table.find(Key(kind, rows_key(kind, M), N, K, out_dtype));
+    if (entry != g_table.end()) {
+      Choice c = entry->second;
+      const bool fits = c.own == LIBRARY ||
+                        (tiles::takes(M, N, K) && c.own < tiles::NUM_CONFIGS && c.splits >= 1 && c.splits <= K / tiles::BK &&
+                         c.splits <= 64 && (c.splits == 1 || N % 4 == 0) &&
+                         (size_t)c.splits * ((M + 7) / 8 * 8) * N * sizeof(float) <= PARTIALS_BYTES);
+      if (fits) return c;
+    }
+  }
+  return kind == KIND_PLAIN ? plain_by_rule(M, N, K) : fused_by_rule(kind, M, N, K);
+}
+
+// ---- the tuner ---------------------------------------------------------------------------------
+
+// The tile shapes that enter the contest, by the product's rows (the others never won a size of the 8B, 14B
+// and 32B models there). Each enters a second time with K shared out where its tiles alone would not fill the
+// chip.
+constexpr int OWN_FEW_ROWS[] = {1, 5}, OWN_SOME_ROWS[] = {0, 1, 2}, OWN_MANY_ROWS[] = {0, 2, 4};
+constexpr int MAX_OWN = 6;
+inline const int* own_shapes(int M, int& count) {
+  if (M <= 256) {
+    count = 2;
+    return OWN_FEW_ROWS;
+  }
+  count = 3;
+  return M <= 1024 ? OWN_SOME_ROWS : OWN_MANY_ROWS;
 }
 
 // The shortest of `reps` runs of `launch`, each with cold caches, in microseconds; negative if it fails.
@@ -171,49 +314,19 @@ float time_runs(Device& d, hipStream_t stream, int reps, Launch launch) {
   return best;
 }
 
-float time_candidate(Device& d, const Plan& p, const hipblasLtMatmulAlgo_t& algo, const void* x, const void* w,
-                     void* out, hipStream_t stream, int reps) {
-  return time_runs(d, stream, reps, [&] { return run(d, p, algo, x, w, out, stream) == HIPBLAS_STATUS_SUCCESS; });
-}
-
-int choose(Device& d, Plan& p, const void* x, const void* w, void* out, int M, int N, int K, int out_dtype,
-           hipStream_t stream, bool capturing) {
+// Times the candidates for the plan's size on the caller's operands and leaves the fastest in the plan.
+int tune_plain(Device& d, Plan& p, const void* x, const void* w, void* out, int M, int N, int K, int out_dtype,
+               hipStream_t stream) {
+  const int set = set_up_tuner(d, stream);
+  if (set) return set;
   const bool own_takes = tiles::takes(M, N, K) && g_kernels != KERNELS_LIBRARY;
-  if (own_takes && g_kernels == KERNELS_OWN && capturing) {   // untimed: the first shape, timed at the next eager call
-    p.candidates = 1;
-    p.chosen = 0;
-    int count = 0;
-    p.own = own_shapes(M, count)[0];
-    p.own_splits = 1;
-    p.tuned = false;
-    return 0;
-  }
-  hipblasLtMatmulPreference_t pref = nullptr;
-  LT_TRY(hipblasLtMatmulPreferenceCreate(&pref));
-  size_t bytes = WORKSPACE_BYTES;
-  hipblasStatus_t s = hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &bytes,
-                                                            sizeof(bytes));
-  const int want = capturing ? 1 : g_candidates;
-  std::vector<hipblasLtMatmulHeuristicResult_t> found(want);
+  std::vector<hipblasLtMatmulHeuristicResult_t> found;
   int got = 0;
-  if (s == HIPBLAS_STATUS_SUCCESS)
-    s = hipblasLtMatmulAlgoGetHeuristic(d.handle, p.desc, p.w, p.x, p.out, p.out, pref, want, found.data(), &got);
-  (void)hipblasLtMatmulPreferenceDestroy(pref);
-  if (s != HIPBLAS_STATUS_SUCCESS) return Q3_ERR_LIBRARY + (int)s;
-  if (got == 0) return Q3_ERR_UNSUPPORTED;
-  p.candidates = got;
-  p.chosen = 0;
-  p.own = -1;
-  p.own_splits = 1;
-  p.algo = found[0].algo;
-  p.tuned = !capturing;
-  if (capturing || (got == 1 && !own_takes)) return 0;
-  if (!d.evict) {
-    HIP_TRY(hipMalloc(&d.evict, EVICT_BYTES));
-    HIP_TRY(hipMemsetAsync(d.evict, 0, EVICT_BYTES, stream));
+  if (!(own_takes && g_kernels == KERNELS_OWN)) {
+    const int status = candidates_of(d, p, g_candidates, found);
+    if (status && !(status == Q3_ERR_UNSUPPORTED && own_takes)) return status;
+    got = (int)found.size();
   }
-  // two passes: all candidates briefly (the first run of each also loads its code), then those
-  // near the front again and longer
   // candidates from `got` on are the hand-written kernel's: (tile shape, shares of K)
   int own_config[MAX_OWN], own_splits[MAX_OWN], owns = 0;
   if (own_takes) {
@@ -224,133 +337,148 @@ int choose(Device& d, Plan& p, const void* x, const void* w, void* out, int M, i
       own_splits[owns++] = 1;
       const int splits = tiles::splits_that_fill(shapes[i], M, N, K);
       if (splits < 2 || (size_t)splits * M * N * sizeof(float) > PARTIALS_BYTES) continue;
-      if (!d.partials) HIP_TRY(hipMalloc((void**)&d.partials, PARTIALS_BYTES));
       own_config[owns] = shapes[i];
       own_splits[owns++] = splits;
     }
   }
   const int all = got + owns;
-  const int first = g_kernels == KERNELS_OWN && own_takes ? got : 0;
+  if (all == 0) return Q3_ERR_UNSUPPORTED;
   auto time_one = [&](int i, int reps) {
-    if (i < got) return time_candidate(d, p, found[i].algo, x, w, out, stream, reps);
+    if (i < got)
+      return time_runs(d, stream, reps, [&] { return run(d, p, found[i].algo, x, w, out, stream) == HIPBLAS_STATUS_SUCCESS; });
     return time_runs(d, stream, reps, [&] {
       return run_own(d, own_config[i - got], own_splits[i - got], x, w, out, M, N, K, out_dtype, stream) == 0;
     });
   };
+  // two passes: all candidates briefly (the first run of each also loads its code), then those
+  // near the front again and longer
   std::vector<float> us(all, -1.f);
   float best = -1.f;
-  for (int i = first; i < all; ++i) {
-    if (time_one(i, 1) < 0.f) continue;     // the first run of a kernel also loads its code
+  for (int i = 0; i < all; ++i) {
+    if (time_one(i, 1) < 0.f) continue;
     us[i] = time_one(i, 2);
     if (us[i] > 0.f && (best < 0.f || us[i] < best)) best = us[i];
   }
   if (best < 0.f) return Q3_ERR_UNSUPPORTED;
-  for (int i = first; i < all; ++i) {
+  for (int i = 0; i < all; ++i) {
     if (us[i] < 0.f || us[i] > 1.2f * best) continue;
     const float again = time_one(i, 5);
     if (again > 0.f && again < us[i]) us[i] = again;
   }
   int chosen = -1;
-  for (int i = first; i < all; ++i)
+  for (int i = 0; i < all; ++i)
     if (us[i] > 0.f && (chosen < 0 || us[i] < us[chosen])) chosen = i;
-  p.candidates = all - first;
-  p.chosen = chosen - first;
+  p.candidates = all;
+  p.chosen = chosen;
+  p.choice = Choice();
   if (chosen < got) {
+    p.choice.library = chosen;
     p.algo = found[chosen].algo;
   } else {
-    p.own = own_config[chosen - got];
-    p.own_splits = own_splits[chosen - got];
+    p.choice.own = own_config[chosen - got];
+    p.choice.splits = own_splits[chosen - got];
   }
-  p.first_us = us[first];
+  p.first_us = us[0] > 0.f ? us[0] : us[chosen];
   p.best_us = us[chosen];
+  p.ready = true;
+  p.timed = true;
   return 0;
 }
 
 // The product by the plan's kernel.
 int run_plan(Device& d, const Plan& p, const void* x, const void* w, void* out, int M, int N, int K, int out_dtype,
              hipStream_t stream) {
-  if (p.own >= 0) return run_own(d, p.own, p.own_splits, x, w, out, M, N, K, out_dtype, stream);
+  if (p.choice.own >= 0) return run_own(d, p.choice.own, p.choice.splits, x, w, out, M, N, K, out_dtype, stream);
   const hipblasStatus_t s = run(d, p, p.algo, x, w, out, stream);
   return s == HIPBLAS_STATUS_SUCCESS ? 0 : Q3_ERR_LIBRARY + (int)s;
 }
 
-// out = x @ w^T by whichever kernel the contest chose for the size (the lock is held).
-int product(Device& d, const void* x, const void* w, void* out, int M, int N, int K, int out_dtype, hipStream_t stream) {
-  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
-  HIP_TRY(hipStreamIsCapturing(stream, &capture));
-  const bool capturing = capture != hipStreamCaptureStatusNone;
-  if (!d.handle) {
-    if (capturing) return (int)hipErrorStreamCaptureUnsupported;   // the first call on a device allocates
-    HIP_TRY(hipMalloc(&d.workspace, WORKSPACE_BYTES));
-    if (!d.begin) {
-      HIP_TRY(hipEventCreate(&d.begin));
-      HIP_TRY(hipEventCreate(&d.end));
+// Makes the plan ready by `c`: for the library, its candidate number c.library for this exact size (its last
+// one if it offers fewer; the hand-written kernel if it offers none and that takes the size).
+int settle(Device& d, Plan& p, Choice c, int M, int N, int K) {
+  p.choice = c;
+  p.candidates = 1;
+  p.chosen = 0;
+  if (c.own < 0) {
+    std::vector<hipblasLtMatmulHeuristicResult_t> found;
+    const int status = candidates_of(d, p, c.library + 1, found);
+    if (status == Q3_ERR_UNSUPPORTED && tiles::takes(M, N, K)) {
+      p.choice = own_by_rule(M, N, K);
+    } else if (status) {
+      return status;
+    } else {
+      p.choice.library = c.library < (int)found.size() ? c.library : (int)found.size() - 1;
+      p.algo = found[p.choice.library].algo;
     }
-    LT_TRY(hipblasLtCreate(&d.handle));
   }
+  p.ready = true;
+  return 0;
+}
+
+// out = x @ w^T by the kernel chosen for the size (the lock is held).
+int product(Device& d, const void* x, const void* w, void* out, int M, int N, int K, int out_dtype, hipStream_t stream) {
+  int status = ready_device(d, stream);
+  if (status) return status;
   Plan& p = d.plans[std::make_tuple(M, N, K, out_dtype)];
   if (!p.desc) {
-    const int status = describe(p, M, N, K, out_dtype);
+    status = describe(p, M, N, K, out_dtype);
     if (status) {
       forget(p);
       return status;
     }
   }
-  const auto near_key = std::make_tuple(rows_class(M), N, K, out_dtype);
-  if (!p.tuned) {
-    auto near = d.chosen_near.find(near_key);
-    if (near != d.chosen_near.end()) {   // a neighbour's choice, if the library takes it for this size
-      p.own = near->second.own;
-      p.own_splits = near->second.own_splits;
-      p.algo = near->second.algo;
-      if (run_plan(d, p, x, w, out, M, N, K, out_dtype, stream) == 0) {
-        p.candidates = near->second.candidates;
-        p.chosen = near->second.chosen;
-        p.first_us = near->second.first_us;
-        p.best_us = near->second.best_us;
-        p.tuned = true;
-        return 0;
+  if (g_mode == MODE_TUNE && !p.timed) {
+    const bool in_capture = capturing(stream, status);
+    if (status) return status;
+    if (!in_capture) {
+      const Key near(KIND_PLAIN + 4 * g_kernels, rows_key(KIND_PLAIN, M), N, K, out_dtype);
+      auto noted = d.noted.find(near);
+      if (noted != d.noted.end()) {   // a neighbour's choice, asked of the library anew for this size
+        status = settle(d, p, noted->second, M, N, K);
+        if (status == 0) p.timed = true;
+      } else {
+        status = tune_plain(d, p, x, w, out, M, N, K, out_dtype, stream);
+        if (status == 0) d.noted[near] = p.choice;
+      }
+      if (status) {
+        forget(p);
+        return status;
       }
     }
   }
-  if (!p.candidates || (!p.tuned && !capturing)) {
-    const int status = choose(d, p, x, w, out, M, N, K, out_dtype, stream, capturing);
+  if (!p.ready) {
+    status = settle(d, p, choice_for(KIND_PLAIN, M, N, K, out_dtype), M, N, K);
     if (status) {
       forget(p);
       return status;
-    }
-    if (p.tuned) {
-      Plan& kept = d.chosen_near[near_key];   // the choice only: the descriptors stay with their size
-      kept.algo = p.algo;
-      kept.own = p.own;
-      kept.own_splits = p.own_splits;
-      kept.candidates = p.candidates;
-      kept.chosen = p.chosen;
-      kept.first_us = p.first_us;
-      kept.best_us = p.best_us;
     }
   }
   return run_plan(d, p, x, w, out, M, N, K, out_dtype, stream);
 }
 
-// Tile shape and shares of K for a product of some tens of rows that carries a norm. `kind` tells the
-// variants apart (0 plain, 1 SwiGLU, 2 residual); `launch(config, splits)` runs one without side effects and
-// returns its status; `other()` does the same work around the contest's product (the vendor library's, mostly)
-// and wins where the tiled kernel's tiles fit the size badly: `config` is then LIBRARY. Timed once per size
-// with cold caches outside a graph capture; a capture that meets a new size takes the rule of thumb and leaves
-// the timing to the next eager call.
-constexpr int LIBRARY = -1;
+// Tile shape and shares of K for a product of some tens of rows that carries a norm, or LIBRARY: `other()`
+// then does the same work around the library's product. `launch(config, splits)` runs the tiled kernel
+// without side effects and returns its status. By the table or the rule; with the tuner on, timed once per
+// size with cold caches outside a graph capture.
 template <typename Launch, typename Other>
-int choose_fused(Device& d, int kind, int M, int N, int K, hipStream_t stream, Launch launch, Other other, int& config,
-                 int& splits) {
-  // rows that differ within a step of eight share a choice: a serving loop meets most of them
-  const auto key = std::make_tuple(kind + 4 * g_kernels, (M + 7) / 8 * 8, N, K);
-  auto known = d.fused.find(key);
-  if (known != d.fused.end()) {
-    config = known->second.first;
-    splits = known->second.second;
+int choose_fused(Device& d, int kind, int M, int N, int K, hipStream_t stream, Launch launch, Other other, Choice& c) {
+  if (g_mode != MODE_TUNE) {
+    c = choice_for(kind, M, N, K, Q3_BF16);
     return 0;
   }
+  const Key key(kind + 4 * g_kernels, rows_key(kind, M), N, K, Q3_BF16);
+  auto known = d.noted.find(key);
+  if (known != d.noted.end()) {
+    c = known->second;
+    return 0;
+  }
+  int status = 0;
+  if (capturing(stream, status) || status) {
+    c = fused_by_rule(kind, M, N, K);
+    return status;
+  }
+  status = set_up_tuner(d, stream);
+  if (status) return status;
   // 64 x 128 tiles also with five stages: with K shared out they need fewer shares to fill the chip (q/k/v at
   // 64 rows 17.7 us in 5 shares against 21.9 in 8). The 64 x 256 tiles lose here too (gate/up 67 us against 51).
   constexpr int FUSED_SHAPES[] = {1, 5, 8};
@@ -364,24 +492,8 @@ int choose_fused(Device& d, int kind, int M, int N, int K, hipStream_t stream, L
     configs[n] = shape;
     shares[n++] = 1;
   }
-  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
-  HIP_TRY(hipStreamIsCapturing(stream, &capture));
-  if (!d.partials) {
-    if (capture != hipStreamCaptureStatusNone) return (int)hipErrorStreamCaptureUnsupported;
-    HIP_TRY(hipMalloc((void**)&d.partials, PARTIALS_BYTES));
-  }
-  config = configs[0];
-  splits = shares[0];
-  if (capture != hipStreamCaptureStatusNone) return 0;
-  if (!d.begin) {
-    HIP_TRY(hipEventCreate(&d.begin));
-    HIP_TRY(hipEventCreate(&d.end));
-  }
-  if (!d.evict) {
-    HIP_TRY(hipMalloc(&d.evict, EVICT_BYTES));
-    HIP_TRY(hipMemsetAsync(d.evict, 0, EVICT_BYTES, stream));
-  }
   float best = -1.f;
+  c = Choice();
   // the first call of the other way holds that product's own contest: not inside a timed run, whose events it uses
   const bool other_works = g_kernels != KERNELS_OWN && other() == 0;
   for (int i = 0; i < n && !(other_works && g_kernels == KERNELS_LIBRARY); ++i) {
@@ -390,24 +502,32 @@ int choose_fused(Device& d, int kind, int M, int N, int K, hipStream_t stream, L
     const float us = time_runs(d, stream, 4, one);
     if (us > 0.f && (best < 0.f || us < best)) {
       best = us;
-      config = configs[i];
-      splits = shares[i];
+      c.own = configs[i];
+      c.splits = shares[i];
     }
   }
   if (other_works) {
     const float us = time_runs(d, stream, 4, [&] { return other() == 0; });
     if (us > 0.f && (best < 0.f || us < best)) {
       best = us;
-      config = LIBRARY;
-      splits = 1;
+      c = Choice();
     }
   }
   if (best < 0.f) return Q3_ERR_UNSUPPORTED;
-  d.fused[key] = std::make_pair(config, splits);
+  d.noted[key] = c;
   return 0;
 }
 
 }  // namespace
+
+// The device's buffers and the library's handle, once per device; the engine calls this when a bfloat16 model is
+// built, so that no product in a step allocates.
+extern "C" int q3_matmul_init() {
+  std::lock_guard<std::mutex> hold(g_lock);
+  int device = 0;
+  HIP_TRY(hipGetDevice(&device));
+  return set_up(g_devices[device]);
+}
 
 // Products of up to 256 rows that carry a norm, by the hand-written tiled kernel (the few-row kernel of
 // gemm.hip does the same for up to 16 rows and is faster there; the callers' policy decides which rows come
@@ -429,6 +549,8 @@ extern "C" int q3_tiles_scaled(const void* x, const void* w, void* out, int M, i
   int device = 0;
   HIP_TRY(hipGetDevice(&device));
   Device& d = g_devices[device];
+  int status = ready_device(d, stream);
+  if (status) return status;
   tiles::RowScale scale;
   scale.sums = sums;
   scale.chunks = chunks;
@@ -442,18 +564,12 @@ extern "C" int q3_tiles_scaled(const void* x, const void* w, void* out, int M, i
       return tiles::launch<float, tiles::EPI_PLAIN>(config, x, w, out, M, N, K, stream, splits, d.partials, scale);
     return tiles::launch<bf16_t, tiles::EPI_PLAIN>(config, x, w, out, M, N, K, stream, splits, d.partials, scale);
   };
-  // the other way: the contest's product in float32, then the kernel that otherwise adds partial products
+  // the other way: the library's product in float32, then the kernel that otherwise adds partial products
   // divides (and activates) its rows
   auto other = [&]() {
     if ((size_t)M * N * sizeof(float) > STAGING_BYTES) return Q3_ERR_UNSUPPORTED;
-    if (!d.staging) {
-      hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
-      HIP_TRY(hipStreamIsCapturing(stream, &capture));
-      if (capture != hipStreamCaptureStatusNone) return (int)hipErrorStreamCaptureUnsupported;
-      HIP_TRY(hipMalloc((void**)&d.staging, STAGING_BYTES));
-    }
-    const int status = product(d, x, w, d.staging, M, N, K, Q3_F32, stream);
-    if (status) return status;
+    const int product_status = product(d, x, w, d.staging, M, N, K, Q3_F32, stream);
+    if (product_status) return product_status;
     const size_t quads = (size_t)M * N / 4;
     const dim3 grid((unsigned)((quads + 255) / 256));
     if (swiglu)
@@ -467,16 +583,25 @@ extern "C" int q3_tiles_scaled(const void* x, const void* w, void* out, int M, i
                          (bf16_t*)out, quads, N / 4, 1, scale);
     return q3_launch_status();
   };
-  int config = 0, splits = 1;
-  const int status = choose_fused(d, swiglu ? 1 : 0, M, N, K, stream, launch, other, config, splits);
+  Choice c;
+  status = choose_fused(d, swiglu ? KIND_SCALED_SWIGLU : KIND_SCALED, M, N, K, stream, launch, other, c);
   if (status) return status;
-  return config == LIBRARY ? other() : launch(config, splits);
+  if (c.own == LIBRARY) {
+    status = other();
+    if (status != Q3_ERR_UNSUPPORTED) return status;
+    c = fused_by_rule(KIND_SCALED, M, N, K);      // the library has nothing for the size: the tiled kernel
+    if (c.own == LIBRARY) {
+      c.own = 8;
+      c.splits = 1;
+    }
+  }
+  return launch(c.own, c.splits);
 }
 
 // q3_tiles_residual: residual (M, N) float32 += bfloat16(x @ w^T) in place; values (M, N) bfloat16 =
 // residual * norm_weight; sums (ceil(N / 1024), M) float32 = the rows' sums of squares of the new residual over
 // chunks of 1,024 columns: what q3_tiles_scaled takes for the next product. Returns Q3_DECLINED, and has done
-// nothing, where the contest's plain product followed by the norm's own kernel is the faster way for this size.
+// nothing, where the plain product followed by the norm's own kernel is the way for this size.
 extern "C" int q3_tiles_residual_chunks(int N) { return (N + tiles::CHUNK_COLUMNS - 1) / tiles::CHUNK_COLUMNS; }
 
 extern "C" int q3_tiles_residual(const void* x, const void* w, int M, int N, int K, float* residual,
@@ -490,22 +615,24 @@ extern "C" int q3_tiles_residual(const void* x, const void* w, int M, int N, int
   int device = 0;
   HIP_TRY(hipGetDevice(&device));
   Device& d = g_devices[device];
-  int config = 0, splits = 1;
-  // timed by the products alone (the tiled kernel's partial products; the contest's product into `values`,
+  int status = ready_device(d, stream);
+  if (status) return status;
+  Choice c;
+  // the tuner times the products alone (the tiled kernel's partial products; the other product into `values`,
   // which the real run overwrites): each way has one small kernel more, and the residual is not touched
-  int status = choose_fused(
-      d, 2, M, N, K, stream,
-      [&](int c, int s) {
-        if ((size_t)s * M * N * sizeof(float) > PARTIALS_BYTES) return Q3_ERR_UNSUPPORTED;
-        return tiles::launch<bf16_t, tiles::EPI_PLAIN>(c, x, w, values, M, N, K, stream, s, d.partials,
+  status = choose_fused(
+      d, KIND_RESIDUAL, M, N, K, stream,
+      [&](int config, int splits) {
+        if ((size_t)splits * M * N * sizeof(float) > PARTIALS_BYTES) return Q3_ERR_UNSUPPORTED;
+        return tiles::launch<bf16_t, tiles::EPI_PLAIN>(config, x, w, values, M, N, K, stream, splits, d.partials,
                                                        tiles::RowScale(), true);
       },
-      [&]() { return product(d, x, w, values, M, N, K, Q3_BF16, stream); }, config, splits);
+      [&]() { return product(d, x, w, values, M, N, K, Q3_BF16, stream); }, c);
   if (status) return status;
-  if (config == LIBRARY) return Q3_DECLINED;
-  if ((size_t)splits * M * N * sizeof(float) > PARTIALS_BYTES) return Q3_ERR_UNSUPPORTED;   // also a single share
+  if (c.own == LIBRARY) return Q3_DECLINED;
+  if ((size_t)c.splits * M * N * sizeof(float) > PARTIALS_BYTES) return Q3_ERR_UNSUPPORTED;   // also a single share
   int used = 1;
-  status = tiles::launch<bf16_t, tiles::EPI_PLAIN>(config, x, w, values, M, N, K, stream, splits, d.partials,
+  status = tiles::launch<bf16_t, tiles::EPI_PLAIN>(c.own, x, w, values, M, N, K, stream, c.splits, d.partials,
                                                    tiles::RowScale(), true, &used);
   if (status) return status;
   const dim3 grid(q3_tiles_residual_chunks(N), M);
@@ -548,7 +675,16 @@ extern "C" int q3_gemm_tiles(const void* x, const void* w, void* out, int M, int
   return Q3_ERR_BAD_ARGUMENT;
 }
 
-// How many of the library's candidates are timed for a new problem size (1: take its first choice).
+// 0: sizes get their kernels by the table and the rules (the default); 1: the tuner times the candidates of
+// every size it first meets outside a capture. Sizes already settled keep their kernel.
+extern "C" int q3_matmul_set_mode(int mode) {
+  if (mode != MODE_RULE && mode != MODE_TUNE) return Q3_ERR_BAD_ARGUMENT;
+  std::lock_guard<std::mutex> hold(g_lock);
+  g_mode = mode;
+  return 0;
+}
+
+// How many of the library's candidates the tuner times for a new size.
 extern "C" int q3_matmul_set_candidates(int n) {
   if (n < 1 || n > MAX_CANDIDATES) return Q3_ERR_BAD_ARGUMENT;
   std::lock_guard<std::mutex> hold(g_lock);
@@ -556,20 +692,53 @@ extern "C" int q3_matmul_set_candidates(int n) {
   return 0;
 }
 
-// Which kernels enter the contest for a new size: 0 the library's and the hand-written one's (the default),
-// 1 the library's alone, 2 the hand-written ones alone where they take the size. Sizes already met keep their
-// choice. The products that carry a norm (q3_tiles_*) keep a choice for each of the three.
+// Which kernels a new size may go to: 0 the library's and the hand-written one's, by the table and the rules
+// (the default), 1 the library's alone (its first candidate), 2 the hand-written ones alone where they take
+// the size. The table speaks for mode 0 only. Sizes already settled are forgotten, so that the next product
+// of every size follows the new setting.
 extern "C" int q3_matmul_set_kernels(int mode) {
   if (mode < KERNELS_BOTH || mode > KERNELS_OWN) return Q3_ERR_BAD_ARGUMENT;
   std::lock_guard<std::mutex> hold(g_lock);
+  if (mode != g_kernels) {
+    for (auto& d : g_devices) {
+      for (auto& p : d.second.plans) forget(p.second);
+      d.second.plans.clear();
+    }
+  }
   g_kernels = mode;
   return 0;
 }
 
-// What was chosen for a size on the current device: info[0] candidates timed, info[1] index chosen,
-// info[2] microseconds of the first candidate, info[3] of the chosen one, info[4] the hand-written kernel's
-// tile shape if that was chosen, else -1, info[5] over how many blocks it shares K out. Returns 1 if the size
-// is known.
+// The table: `kind` 0 a plain product, 1 a product whose rows still lack their norm's division, 2 the same with
+// the SwiGLU activation, 3 a product that is added into the residual stream; `rows` as q3_matmul_rows_key
+// rounds them; `own` >= 0: the hand-written kernel's tile shape with `splits` shares of K; own < 0: the
+// library's candidate number `library` (for kind 3: the caller's plain product and separate norm).
+extern "C" int q3_matmul_rows_key(int kind, int M) { return rows_key(kind, M); }
+
+extern "C" int q3_matmul_table_add(int kind, int rows, int N, int K, int out_dtype, int library, int own, int splits) {
+  if (kind < KIND_PLAIN || kind > KIND_RESIDUAL || rows < 1 || N < 1 || K < 1) return Q3_ERR_BAD_ARGUMENT;
+  if (library < 0 || library >= MAX_CANDIDATES || own >= tiles::NUM_CONFIGS || splits < 1 || splits > 64)
+    return Q3_ERR_BAD_ARGUMENT;
+  std::lock_guard<std::mutex> hold(g_lock);
+  Choice c;
+  c.library = library;
+  c.own = own < 0 ? LIBRARY : own;
+  c.splits = splits;
+  g_table[Key(kind, rows, N, K, out_dtype)] = c;
+  return 0;
+}
+
+extern "C" int q3_matmul_table_clear() {
+  std::lock_guard<std::mutex> hold(g_lock);
+  g_table.clear();
+  return 0;
+}
+
+// What serves a plain product of this size on the current device: info[0] candidates timed (1 if none were),
+// info[1] the one chosen among them, info[2] microseconds of the first candidate, info[3] of the chosen one
+// (zero if untimed), info[4] the hand-written kernel's tile shape if that serves it, else -1, info[5] over how
+// many blocks it shares K out, info[6] the library's candidate number if the library serves it. Returns 1 if
+// the size has been met.
 extern "C" int q3_matmul_plan(int M, int N, int K, int out_dtype, float* info) {
   std::lock_guard<std::mutex> hold(g_lock);
   int device = 0;
@@ -577,13 +746,38 @@ extern "C" int q3_matmul_plan(int M, int N, int K, int out_dtype, float* info) {
   auto d = g_devices.find(device);
   if (d == g_devices.end()) return 0;
   auto p = d->second.plans.find(std::make_tuple(M, N, K, out_dtype));
-  if (p == d->second.plans.end()) return 0;
+  if (p == d->second.plans.end() || !p->second.ready) return 0;
   info[0] = (float)p->second.candidates;
   info[1] = (float)p->second.chosen;
   info[2] = p->second.first_us;
   info[3] = p->second.best_us;
-  info[4] = (float)p->second.own;
-  info[5] = (float)p->second.own_splits;
+  info[4] = (float)p->second.choice.own;
+  info[5] = (float)p->second.choice.splits;
+  info[6] = (float)p->second.choice.library;
+  return 1;
+}
+
+// What serves a product of 17 to 128 rows that carries a norm (`kind` 1, 2 or 3 as in the table) under the
+// current settings: info[0] the tile shape or -1 (the library's product with the norm's work behind it, or
+// declined), info[1] the shares of K. With the tuner on: what it found, and 0 is returned for a size it has
+// not met.
+extern "C" int q3_matmul_fused_plan(int kind, int M, int N, int K, int* info) {
+  if (kind < KIND_SCALED || kind > KIND_RESIDUAL) return 0;
+  std::lock_guard<std::mutex> hold(g_lock);
+  Choice c;
+  if (g_mode == MODE_TUNE) {
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess) return 0;
+    auto d = g_devices.find(device);
+    if (d == g_devices.end()) return 0;
+    auto known = d->second.noted.find(Key(kind + 4 * g_kernels, rows_key(kind, M), N, K, Q3_BF16));
+    if (known == d->second.noted.end()) return 0;
+    c = known->second;
+  } else {
+    c = choice_for(kind, M, N, K, Q3_BF16);
+  }
+  info[0] = c.own;
+  info[1] = c.splits;
   return 1;
 }
 

@@ -11,6 +11,8 @@ statistics and logits are float32 in both modes.
 """
 
 import ctypes
+import json
+import os
 
 import torch
 
@@ -29,10 +31,16 @@ __all__ = [
     "decode_attention_takes",
     "swiglu",
     "linear",
+    "linear_plain",
     "linear_swiglu",
     "linear_residual_norm",
     "matmul_candidates",
     "matmul_kernels",
+    "matmul_init",
+    "matmul_table",
+    "matmul_tuner",
+    "matmul_rows_key",
+    "matmul_fused_plan",
     "gemm_tiles",
     "gemm_tiles_configs",
     "gemm_tiles_splits",
@@ -78,31 +86,91 @@ def _check(status, what):
         raise RuntimeError("%s failed: HIP error %d" % (what, status))
 
 
+_KINDS = {"plain": 0, "scaled": 1, "scaled_swiglu": 2, "residual": 3}
+TABLE_FILE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "matmul_table.json")
+_table_loaded = False
+
+
+def _matmul():
+    """The many-row product library, with the table of kernel choices loaded at its first use."""
+    global _table_loaded
+    lib = library("matmul")
+    if not _table_loaded:
+        _table_loaded = True
+        if os.path.isfile(TABLE_FILE):
+            with open(TABLE_FILE, encoding="utf-8") as fh:
+                matmul_table(json.load(fh)["entries"])
+    return lib
+
+
+def matmul_init():
+    """Allocate the many-row products' workspace and buffers on the current device now (a model
+    being built calls this), so that no product inside a step allocates."""
+    _check(_matmul().q3_matmul_init(), "matmul_init")
+
+
+def matmul_table(entries, clear=False):
+    """Load kernel choices: each entry {"kind": "plain" | "scaled" | "scaled_swiglu" | "residual",
+    "rows": rounded rows (`matmul_rows_key`), "N", "K", "out": "bfloat16" | "float32",
+    "library": the library's candidate number, or "own": tile shape and "splits": shares of K}.
+    Sizes without an entry follow the rules of thumb. Sizes already met keep their kernel."""
+    lib = library("matmul")
+    if clear:
+        _check(lib.q3_matmul_table_clear(), "matmul_table")
+    for e in entries:
+        out = _DT[getattr(torch, e.get("out", "bfloat16"))]
+        _check(lib.q3_matmul_table_add(_KINDS[e["kind"]], int(e["rows"]), int(e["N"]), int(e["K"]), out,
+                                       int(e.get("library", 0)), int(e.get("own", -1)), int(e.get("splits", 1))),
+               "matmul_table")
+
+
+def matmul_rows_key(kind, M):
+    """The rows a table entry for `M` rows is filed under (sizes within a step of rows share one)."""
+    return int(library("matmul").q3_matmul_rows_key(_KINDS[kind], int(M)))
+
+
+def matmul_tuner(on):
+    """With the tuner on, a product size first met outside a graph capture has its candidate
+    kernels timed on the caller's operands and keeps the fastest for the life of the process
+    (`matmul_plan`, `matmul_fused_plan` tell which): the way the table is made. Off (the
+    default), kernels are chosen by the table and the rules alone, the same in every process."""
+    _check(_matmul().q3_matmul_set_mode(1 if on else 0), "matmul_tuner")
+
+
 def matmul_candidates(n):
-    """How many of the vendor library's candidate kernels are timed when a product with many rows
-    meets a new size (1: its first choice is taken untimed)."""
-    _check(library("matmul").q3_matmul_set_candidates(int(n)), "matmul_candidates")
+    """How many of the vendor library's candidate kernels the tuner times for a new size."""
+    _check(_matmul().q3_matmul_set_candidates(int(n)), "matmul_candidates")
 
 
 def matmul_kernels(which):
-    """Which kernels a product with many rows may go to when it meets a new size: "both" (the
-    vendor library's candidates and the hand-written tiled kernel's shapes are timed and the
-    fastest is kept; the default), "library", or "own" (the hand-written kernel wherever it
-    takes the size: an inner size that is a multiple of 64). Sizes already met keep their choice."""
+    """Which kernels a product with many rows may go to: "both" (the table and the rules decide
+    between the vendor library and the hand-written tiled kernel; the default), "library" (the
+    library's first candidate), or "own" (the hand-written kernel wherever it takes the size: an
+    inner size that is a multiple of 64). A change makes every size choose anew."""
     modes = {"both": 0, "library": 1, "own": 2}
     _need(which in modes, "which is one of %s" % ", ".join(sorted(modes)))
-    _check(library("matmul").q3_matmul_set_kernels(modes[which]), "matmul_kernels")
+    _check(_matmul().q3_matmul_set_kernels(modes[which]), "matmul_kernels")
 
 
 def matmul_plan(M, N, K, out_dtype=torch.bfloat16):
-    """What was chosen for a size on the current device, or None if it has not been met:
-    (candidates timed, index chosen, microseconds of the first candidate, of the chosen one,
-    the hand-written kernel's tile shape if that was chosen, else -1, and over how many blocks
-    it shares K out)."""
-    info = (ctypes.c_float * 6)()
-    if not library("matmul").q3_matmul_plan(int(M), int(N), int(K), _DT[out_dtype], info):
+    """What serves a plain product of this size on the current device, or None if it has not
+    been met: (candidates timed (1 without the tuner), index chosen, microseconds of the first
+    candidate, of the chosen one, the hand-written kernel's tile shape if that serves it, else
+    -1, over how many blocks it shares K out, the library's candidate number)."""
+    info = (ctypes.c_float * 7)()
+    if not _matmul().q3_matmul_plan(int(M), int(N), int(K), _DT[out_dtype], info):
         return None
-    return int(info[0]), int(info[1]), float(info[2]), float(info[3]), int(info[4]), int(info[5])
+    return int(info[0]), int(info[1]), float(info[2]), float(info[3]), int(info[4]), int(info[5]), int(info[6])
+
+
+def matmul_fused_plan(kind, M, N, K):
+    """What serves a product of 17 to 128 rows that carries a norm (`kind` "scaled",
+    "scaled_swiglu" or "residual"): (tile shape or -1 for the library's product with the norm's
+    work behind it, shares of K); None with the tuner on for a size it has not met."""
+    info = (ctypes.c_int * 2)()
+    if not _matmul().q3_matmul_fused_plan(_KINDS[kind], int(M), int(N), int(K), info):
+        return None
+    return int(info[0]), int(info[1])
 
 
 def gemm_tiles_configs():
@@ -472,7 +540,7 @@ def _tiles_scaled(x, weight, out, unscaled, swiglu, what):
           and sums.is_contiguous(), "row sums must be float32 (chunks, M)")
     _need(width == K, "the rows' width must be the product's inner size")
     _need(x.is_contiguous() and out.is_contiguous(), "operands must be contiguous")
-    _check(library("matmul").q3_tiles_scaled(
+    _check(_matmul().q3_tiles_scaled(
         _ptr(x), _ptr(weight), _ptr(out), M, weight.shape[0], K, _DT[out.dtype], 1 if swiglu else 0, _ptr(sums),
         sums.shape[0], ctypes.c_float(eps), int(width), _stream()), what)
     return out
@@ -511,23 +579,40 @@ def linear(x, weight, out_dtype=None, out=None, tiled=None, unscaled=None):
           "with an inner size that is a multiple of 64")
     if M and x.dtype == torch.bfloat16 and not library("gemm").q3_linear_is_skinny(M, N, K, 1):
         # bfloat16 products with many rows go to the vendor library (hipBLASLt), as the
-        # reference's engine uses its vendor library for them; accumulation is float32.
-        # The module picks the library's kernel for each size by timing its candidates
-        # once. Few rows take the weight-streaming kernel below.
+        # reference's engine uses its vendor library for them, or to the hand-written tiled
+        # kernel, as a table of sizes and a rule of thumb say; accumulation is float32.
+        # Few rows take the weight-streaming kernel below.
         _need(x.is_contiguous() and weight.is_contiguous() and out.is_contiguous(), "operands must be contiguous")
-        status = library("matmul").q3_matmul(_ptr(x), _ptr(weight), _ptr(out), M, N, K, _DT[out_dtype], _stream())
+        status = _matmul().q3_matmul(_ptr(x), _ptr(weight), _ptr(out), M, N, K, _DT[out_dtype], _stream())
         if status == _UNSUPPORTED:
-            # a size hipBLASLt offers no kernel for (an odd inner size, say): the vendor's other
-            # library, through torch
-            if out_dtype == torch.bfloat16:
-                torch.mm(x, weight.t(), out=out)
-            else:
-                torch.mm(x, weight.t(), out_dtype=torch.float32, out=out)
+            # a size neither hipBLASLt nor the tiled kernel has a kernel for (an odd inner size,
+            # say): plain multiply-adds with float32 sums
+            linear_plain(x, weight, out)
         else:
             _check(status, "matmul")
     elif M:
         _check(library("gemm").q3_linear(
             _ptr(x), _ptr(weight), _ptr(out), M, N, K, _DT[x.dtype], _DT[out_dtype], _stream()), "linear")
+    return out
+
+
+def linear_plain(x, weight, out):
+    """out = x @ weight^T by plain multiply-adds with float32 sums, for any size: what serves a
+    bfloat16 product with more than 16 rows that neither the vendor library nor the tiled
+    kernel takes, and every float32 product."""
+    _dev(x, weight, out)
+    _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1] and x.dtype in _DT
+          and weight.dtype == x.dtype, "x (M, K) and weight (N, K) of one dtype")
+    M, K = x.shape
+    N = weight.shape[0]
+    _need(out.shape == (M, N) and out.dtype in _DT and not (x.dtype == torch.float32 and out.dtype != torch.float32),
+          "out must be (M, N); float32 inputs give float32 output")
+    lib = library("gemm")
+    _need(M > 16 or x.dtype == torch.float32 or not lib.q3_linear_is_skinny(M, N, K, 1),
+          "bfloat16 products of up to 16 rows are the weight-streaming kernel's")
+    if M:
+        _check(lib.q3_linear(_ptr(x), _ptr(weight), _ptr(out), M, N, K, _DT[x.dtype], _DT[out.dtype], _stream()),
+               "linear_plain")
     return out
 
 
@@ -589,7 +674,7 @@ def linear_residual_norm(x, weight, tiled, residual, norm_weight):
     values = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
     if x.dtype == torch.bfloat16 and fused_rows_take(weight, M):
         _need(x.is_contiguous(), "x must be contiguous")
-        lib = library("matmul")
+        lib = _matmul()
         sums = torch.empty((lib.q3_tiles_residual_chunks(N), M), dtype=torch.float32, device=x.device)
         status = lib.q3_tiles_residual(
             _ptr(x), _ptr(weight), M, N, K, _ptr(residual), _ptr(norm_weight), _DT[norm_weight.dtype], _ptr(values),

@@ -90,13 +90,17 @@ class Part:
 @dataclass
 class NormSink:
     """Where a part's last product may go instead of being returned: added into
-    `residual` (float32 (T, width), in place) and prepared for `norm`, the norm
-    that reads the residual next. A part whose class sets `feeds_sink` takes it
-    as `forward(..., sink=...)` and then returns `UnscaledRows`; it may also
-    ignore the sink and return its result as always."""
+    `residual` (float32 (T, width), in place) and prepared for the root-mean-square
+    norm that reads the residual next, which is given by its numbers alone:
+    `weight` (width,), `eps`, `width`. A part whose class sets `feeds_sink` takes
+    it as `forward(..., sink=...)` and then returns `UnscaledRows`; it may also
+    ignore the sink and return its result as always. A norm of another form (a
+    bias, a mean taken out) offers no sink and is applied by its own kernel."""
 
     residual: torch.Tensor
-    norm: object
+    weight: torch.Tensor
+    eps: float
+    width: int
 
 
 @dataclass

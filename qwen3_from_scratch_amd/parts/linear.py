@@ -17,6 +17,8 @@ class LinearWeight:
     def __init__(self, weight, precision):
         self.weight = weight
         self.tiled = ops.tile_weight(weight) if precision.tiled else None
+        if weight.is_cuda and weight.dtype == torch.bfloat16:
+            ops.matmul_init()          # the many-row products' buffers: now, not inside a step
 
     def forward(self, x, out_dtype=None):
         """x @ W^T; x may be UnscaledRows (see `fuses`)."""
@@ -41,12 +43,11 @@ class LinearWeight:
     def forward_into(self, x, sink):
         """x @ W^T added into the sink's residual and prepared for its norm, as
         UnscaledRows; or, where the kernels do not take the case, returned."""
-        norm = sink.norm
         rows = x.shape[0]
         if self.tiled is None or not (ops.fused_rows_take(self.weight, rows) if rows > ops.FUSED_ROWS_FEW
                                       else self.weight.shape[0] % 16 == 0):
             return self.forward(x)
-        fused = ops.linear_residual_norm(x, self.weight, self.tiled, sink.residual, norm.weight)
+        fused = ops.linear_residual_norm(x, self.weight, self.tiled, sink.residual, sink.weight)
         if fused is None:                       # the kernel leaves this size to the plain product
             return self.forward(x)
-        return UnscaledRows(fused[0], fused[1], norm.eps, norm.size)
+        return UnscaledRows(fused[0], fused[1], sink.eps, sink.width)

@@ -45,4 +45,4 @@ class RMSNorm(Part):
             return None
         if not 1 <= rows <= ops.FUSED_ROWS_MOST or self.size % (16 if rows <= ops.FUSED_ROWS_FEW else 64):
             return None
-        return NormSink(x, self)
+        return NormSink(x, self.weight, self.eps, self.size)

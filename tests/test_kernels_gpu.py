@@ -403,12 +403,31 @@ def test_linear_few_rows_streams_weights(M, N, K):
         assert torch.equal(alone[0], got[0])
 
 
+def _forget_choices(ops):
+    ops.matmul_kernels("library")          # a change of setting makes every size choose anew
+    ops.matmul_kernels("both")
+
+
+@pytest.fixture
+def rules_alone():
+    """The table of kernel choices emptied for a test, and the package's own loaded again after it."""
+    import json
+
+    ops = _ops()
+    ops.matmul_table([], clear=True)
+    _forget_choices(ops)
+    yield ops
+    with open(ops.TABLE_FILE) as fh:
+        ops.matmul_table(json.load(fh)["entries"], clear=True)
+    _forget_choices(ops)
+
+
 @pytest.mark.parametrize("M,N,K", [(17, 4096, 4096), (64, 6144, 4096), (200, 1000, 2056), (576, 5120, 1024),
-                                   (2048, 768, 512), (33, 331, 72), (40, 129, 515)])
-def test_linear_many_rows_is_the_library_kernel_that_was_fastest(M, N, K):
-    """More than 16 bfloat16 rows go to the vendor library, which times its candidates once
-    for a size; the choice holds from then on, also inside a graph, and a size it has no
-    kernel for takes the other route."""
+                                   (2048, 768, 512), (33, 331, 72), (40, 129, 515), (300, 77, 100)])
+def test_linear_many_rows_takes_its_kernel_by_rule(rules_alone, M, N, K):
+    """More than 16 bfloat16 rows go to the vendor library's first candidate for the exact size
+    (no stopwatch: the same kernel in every process), also inside a graph; a size it has no
+    kernel for goes to the hand-written kernels."""
     ops = _ops()
     x = _rand((M, K), torch.bfloat16, 41)
     w = _rand((N, K), torch.bfloat16, 42, scale=0.05)
@@ -418,49 +437,109 @@ def test_linear_many_rows_is_the_library_kernel_that_was_fastest(M, N, K):
     got16 = ops.linear(x, w)
     torch.testing.assert_close(got16.double(), want, rtol=1.6e-2, atol=1e-2)
     plan = ops.matmul_plan(M, N, K)
-    if K % 8 == 0:
-        assert plan is not None and plan[0] >= 1 and 0 <= plan[1] < plan[0]
-        assert plan[3] <= plan[2] or plan[0] == 1          # the chosen one was no slower than the first
-    assert torch.equal(ops.linear(x, w), got16)            # and stays chosen
+    assert plan is not None and plan[0] == 1 and plan[2] == 0.0            # nothing was timed
+    assert plan[4] == -1 and plan[6] == 0                                  # the library's first candidate
+    assert torch.equal(ops.linear(x, w), got16)
+    # the kernel for sizes that nothing else takes: plain multiply-adds, float32 sums
+    plain = ops.linear_plain(x, w, torch.empty((M, N), dtype=torch.float32, device=x.device))
+    torch.testing.assert_close(plain.double(), want, rtol=1e-4, atol=1e-4)
+    plain16 = ops.linear_plain(x, w, torch.empty((M, N), dtype=torch.bfloat16, device=x.device))
+    assert torch.equal(plain16, plain.bfloat16())
     # rows do not mix: a row's result is the same whatever its neighbours hold
     other = x.clone()
     other[1:] = _rand((M - 1, K), torch.bfloat16, 43)
     assert torch.equal(ops.linear(other, w)[0], got16[0])
-    if M > 64 and K % 8 == 0:
-        # a few rows fewer (the same multiple of 32 rounded up): the same kernel, not timed again
-        fewer = ops.linear(x[:M - 7].contiguous(), w, out_dtype=torch.float32)
-        torch.testing.assert_close(fewer.double(), want[:M - 7], rtol=2e-3, atol=2e-3)
-        assert ops.matmul_plan(M - 7, N, K, torch.float32)[:2] == ops.matmul_plan(M, N, K, torch.float32)[:2]
+
+
+def test_the_rule_for_few_tiles_and_a_long_inner_size(rules_alone):
+    """A product with some hundreds of rows whose inner size is twice its width or more goes to
+    the tiled kernel with K shared out; the same bits from two runs of the choice."""
+    ops = rules_alone
+    M, N, K = 200, 256, 1024
+    x = _rand((M, K), torch.bfloat16, 61)
+    w = _rand((N, K), torch.bfloat16, 62, scale=0.05)
+    got = ops.linear(x, w)
+    plan = ops.matmul_plan(M, N, K)
+    assert plan[4] == 1 and plan[5] == ops.gemm_tiles_splits(1, M, N, K) > 1
+    torch.testing.assert_close(got.double(), x.double() @ w.double().T, rtol=1.6e-2, atol=1e-2)
+    _forget_choices(ops)
+    assert torch.equal(ops.linear(x, w), got) and ops.matmul_plan(M, N, K) == plan
+
+
+def test_the_table_decides_a_size():
+    """A table entry sends a size to the library's second candidate or to a tile shape of the
+    hand-written kernel with K shared out; sizes within the same step of rows follow it, others
+    keep the rule; an entry the size cannot take (K no multiple of 64) is passed over."""
+    ops = _ops()
+    N, K = 1184, 640
+    w = _rand((N, K), torch.bfloat16, 45, scale=0.05)
+    rows = ops.matmul_rows_key("plain", 200)
+    assert rows == 224 and ops.matmul_rows_key("plain", 50) == 50 and ops.matmul_rows_key("scaled", 50) == 56
+    try:
+        ops.matmul_table([{"kind": "plain", "rows": rows, "N": N, "K": K, "own": 1, "splits": 2},
+                          {"kind": "plain", "rows": rows, "N": N, "K": K, "out": "float32", "library": 1},
+                          {"kind": "plain", "rows": 64, "N": 96, "K": 72, "own": 0, "splits": 1}], clear=True)
+        _forget_choices(ops)
+        for M in (200, 195):
+            x = _rand((M, K), torch.bfloat16, 46)
+            got = ops.linear(x, w)
+            assert ops.matmul_plan(M, N, K)[4:6] == (1, 2)
+            assert torch.equal(got, ops.gemm_tiles(x, w, 1, splits=2))
+            ops.linear(x, w, out_dtype=torch.float32)
+            assert ops.matmul_plan(M, N, K, torch.float32)[4] == -1 and ops.matmul_plan(M, N, K, torch.float32)[6] in (0, 1)
+        x = _rand((150, K), torch.bfloat16, 47)
+        ops.linear(x, w)
+        assert ops.matmul_plan(150, N, K)[4] == -1 and ops.matmul_plan(150, N, K)[6] == 0
+        x3, w3 = _rand((64, 72), torch.bfloat16, 57), _rand((96, 72), torch.bfloat16, 58, scale=0.05)
+        torch.testing.assert_close(ops.linear(x3, w3, out_dtype=torch.float32).double(), x3.double() @ w3.double().T,
+                                   rtol=2e-3, atol=2e-3)
+    finally:
+        import json
+        with open(ops.TABLE_FILE) as fh:
+            ops.matmul_table(json.load(fh)["entries"], clear=True)
+        _forget_choices(ops)
 
 
 def test_linear_many_rows_first_met_in_a_graph():
-    """A size first met while a graph is captured runs untimed there, is timed at its next
-    eager call, and the graph's replays keep giving the right product."""
+    """A size first met while a graph is captured gets its kernel there as anywhere (the choice
+    needs no run); with the tuner on it runs untimed in the capture and is timed at its next
+    eager call; the graph's replays keep giving the right product."""
     ops = _ops()
     M, N, K = 48, 1184, 608
     x = _rand((M, K), torch.bfloat16, 44)
     w = _rand((N, K), torch.bfloat16, 45, scale=0.05)
-    ops.linear(_rand((20, 64), torch.bfloat16, 1), _rand((64, 64), torch.bfloat16, 2))   # the device's set-up is eager
+    ops.matmul_init()
     out = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
     assert ops.matmul_plan(M, N, K) is None
-    side = torch.cuda.Stream()
-    side.wait_stream(torch.cuda.current_stream())
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.stream(side):
-        with torch.cuda.graph(graph, stream=side):
-            ops.linear(x, w, out=out)
-    torch.cuda.current_stream().wait_stream(side)
-    assert ops.matmul_plan(M, N, K)[0] == 1
-    want = x.double() @ w.double().T
-    for seed in (46, 47, 48):
-        out.zero_()
-        graph.replay()
-        torch.testing.assert_close(out.double(), want, rtol=1.6e-2, atol=1e-2)
-        eager = ops.linear(x, w)                               # timed at the first of these
-        torch.testing.assert_close(eager.double(), want, rtol=1.6e-2, atol=1e-2)
-        x.copy_(_rand((M, K), torch.bfloat16, seed))
+    ops.matmul_tuner(True)
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                ops.linear(x, w, out=out)
+        torch.cuda.current_stream().wait_stream(side)
+        assert ops.matmul_plan(M, N, K)[0] == 1
         want = x.double() @ w.double().T
-    assert ops.matmul_plan(M, N, K)[0] > 1
+        for seed in (46, 47, 48):
+            out.zero_()
+            graph.replay()
+            torch.testing.assert_close(out.double(), want, rtol=1.6e-2, atol=1e-2)
+            eager = ops.linear(x, w)                               # timed at the first of these
+            torch.testing.assert_close(eager.double(), want, rtol=1.6e-2, atol=1e-2)
+            x.copy_(_rand((M, K), torch.bfloat16, seed))
+            want = x.double() @ w.double().T
+        plan = ops.matmul_plan(M, N, K)
+        assert plan[0] > 1 and 0 <= plan[1] < plan[0] and plan[3] <= plan[2]
+        # a few rows fewer (the same step of rows): the same choice, asked of the library for the exact size
+        M2 = 200
+        x2 = _rand((M2, K), torch.bfloat16, 49)
+        ops.linear(x2, w)
+        fewer = ops.linear(x2[:M2 - 7].contiguous(), w, out_dtype=torch.float32)
+        torch.testing.assert_close(fewer.double(), x2[:M2 - 7].double() @ w.double().T, rtol=2e-3, atol=2e-3)
+    finally:
+        ops.matmul_tuner(False)
 
 
 @pytest.mark.parametrize("M,N,K", [(200, 304, 128), (513, 1000, 192), (77, 48, 64), (17, 2, 64), (300, 331, 4096),
@@ -505,10 +584,10 @@ def test_tiled_product_every_shape_and_epilogue(M, N, K):
 
 
 def test_linear_many_rows_by_the_hand_written_kernel_alone():
-    """With the contest narrowed to the hand-written kernel, products with many rows are its:
+    """Narrowed to the hand-written kernel, products with many rows are its:
     a size it takes, also first met inside a graph, and a size it does not take (the library's)."""
     ops = _ops()
-    ops.linear(_rand((20, 64), torch.bfloat16, 1), _rand((64, 64), torch.bfloat16, 2))   # the device's set-up is eager
+    ops.matmul_init()
     ops.matmul_kernels("own")
     try:
         M, N, K = 150, 840, 320
@@ -520,7 +599,7 @@ def test_linear_many_rows_by_the_hand_written_kernel_alone():
         plan = ops.matmul_plan(M, N, K, torch.float32)
         assert plan[4] >= 0 and plan[0] >= 1
         assert torch.equal(got, ops.gemm_tiles(x, w, plan[4], out_dtype=torch.float32))
-        # first met in a capture: runs untimed there, timed at the next eager call
+        # first met in a capture
         M2 = 90
         x2 = _rand((M2, K), torch.bfloat16, 56)
         out = torch.empty((M2, N), dtype=torch.bfloat16, device=x.device)
@@ -537,14 +616,14 @@ def test_linear_many_rows_by_the_hand_written_kernel_alone():
             torch.testing.assert_close(out.double(), x2.double() @ w.double().T, rtol=1.6e-2, atol=1e-2)
             assert torch.equal(ops.linear(x2, w), out)
         assert ops.matmul_plan(M2, N, K)[4] >= 0
-        # few tiles and many steps: the shapes that share K out stand in the contest too
+        # few tiles and many steps: K is shared out
         M4, N4, K4 = 300, 512, 4096
-        assert ops.gemm_tiles_splits(0, M4, N4, K4) > 1
+        assert ops.gemm_tiles_splits(1, M4, N4, K4) > 1
         x4, w4 = _rand((M4, K4), torch.bfloat16, 59), _rand((N4, K4), torch.bfloat16, 60, scale=0.05)
         torch.testing.assert_close(ops.linear(x4, w4, out_dtype=torch.float32).double(), x4.double() @ w4.double().T,
                                    rtol=1e-4, atol=1e-4)
         plan4 = ops.matmul_plan(M4, N4, K4, torch.float32)
-        assert plan4[0] >= 4 and plan4[4] >= 0 and plan4[5] >= 1
+        assert plan4[4] == 1 and plan4[5] == ops.gemm_tiles_splits(1, M4, N4, K4)
         # an inner size it does not take goes to the library
         x3, w3 = _rand((40, 72), torch.bfloat16, 57), _rand((96, 72), torch.bfloat16, 58, scale=0.05)
         torch.testing.assert_close(ops.linear(x3, w3, out_dtype=torch.float32).double(), x3.double() @ w3.double().T,
@@ -666,9 +745,9 @@ def test_linear_residual_norm_and_unscaled_rows_beyond_sixteen(M, H, K, N2, norm
     assert ops.fused_rows_take(w1, M) and ops.fused_rows_take(w2, M)
 
     exact_delta = (x.double() @ w1.double().T)
-    ops.linear(_rand((20, 64), torch.bfloat16, 1), _rand((64, 64), torch.bfloat16, 2))   # the device's set-up
+    ops.matmul_init()
     try:
-        # with the hand-written kernel alone in the contest the fusion is never declined
+        # with the hand-written kernel alone the fusion is never declined
         ops.matmul_kernels("own")
         fused_stream = residual.clone()
         values, sums = ops.linear_residual_norm(x, w1, None, fused_stream, nw)
@@ -690,8 +769,8 @@ def test_linear_residual_norm_and_unscaled_rows_beyond_sixteen(M, H, K, N2, norm
         want = ops.linear(h, w2, out_dtype=torch.float32)
         exact = (stream.double() * torch.rsqrt((stream.double() ** 2).mean(dim=1, keepdim=True) + eps)
                  * nw.double()) @ w2.double().T
-        # the reader by the tiled kernel, by the contest's product with the division behind it, and by
-        # whichever of the two was faster; there the writer may leave the size to the plain product
+        # the reader by the tiled kernel, by the library's product with the division behind it, and by
+        # whichever of the two the table and the rule name; there the writer may leave the size to the plain product
         for which in ("own", "library", "both"):
             ops.matmul_kernels(which)
             got = ops.linear(values, w2, out_dtype=torch.float32, unscaled=(sums, eps, H))
@@ -712,7 +791,7 @@ def test_linear_residual_norm_and_unscaled_rows_beyond_sixteen(M, H, K, N2, norm
             if fused is None:
                 assert which != "own" and torch.equal(other_stream, residual)      # declined: nothing was done
             else:
-                # another tile shape may have won this time: other shares of K, other roundings
+                # another tile shape may serve this setting: other shares of K, other roundings
                 torch.testing.assert_close(other_stream, fused_stream, rtol=0, atol=2 ** -7 * float(exact_delta.abs().max()))
                 assert float((other_stream != fused_stream).float().mean()) < 0.02
         with pytest.raises(ops.OperandError):                      # sums of another number of rows

@@ -52,20 +52,20 @@ def test_linear_part_falls_back_where_the_kernel_declines(cpu_ops, monkeypatch):
         return None
 
     monkeypatch.setattr(ops, "linear_residual_norm", declines, raising=False)
-    out = part.forward_into(x, NormSink(residual, norm))
+    out = part.forward_into(x, NormSink(residual, norm.weight, norm.eps, norm.size))
     assert calls == [40] and torch.equal(out, part.forward(x)) and float(residual.abs().max()) == 0.0
 
     def fuses(x, weight, tiled, residual, norm_weight):
         return torch.ones(x.shape[0], weight.shape[0], dtype=torch.bfloat16), torch.ones(1, x.shape[0])
 
     monkeypatch.setattr(ops, "linear_residual_norm", fuses, raising=False)
-    out = part.forward_into(x, NormSink(residual, norm))
+    out = part.forward_into(x, NormSink(residual, norm.weight, norm.eps, norm.size))
     assert isinstance(out, UnscaledRows) and out.width == 128 and out.sums.shape == (1, 40)
     # rows or sizes outside what the kernels take never reach them
     monkeypatch.setattr(ops, "linear_residual_norm", lambda *a: 1 / 0, raising=False)
     many = torch.randn(200, 64).bfloat16()
-    assert torch.equal(part.forward_into(many, NormSink(torch.zeros(200, 128), norm)), part.forward(many))
+    assert torch.equal(part.forward_into(many, NormSink(torch.zeros(200, 128), norm.weight, norm.eps, norm.size)), part.forward(many))
     odd = LinearWeight((torch.randn(128, 96) * 0.1).bfloat16(), precision)          # inner size 96: not in steps of 64
     odd.tiled = torch.zeros(1)
     x96 = torch.randn(40, 96).bfloat16()
-    assert torch.equal(odd.forward_into(x96, NormSink(torch.zeros(40, 128), norm)), odd.forward(x96))
+    assert torch.equal(odd.forward_into(x96, NormSink(torch.zeros(40, 128), norm.weight, norm.eps, norm.size)), odd.forward(x96))

@@ -306,6 +306,14 @@ class CacheManager:
     def num_pages(self, group=0):
         return self.groups[group].pool.num_pages
 
+    def table_width(self, group, tokens):
+        """Entries a block table of `group` needs for a request of `tokens` tokens. A windowed
+        group's table is as long as any other's: a block keeps its place in the table when its
+        page goes back (the entry turns -1), so kernels find a key's page by its position alone."""
+        if not 0 <= group < len(self.groups):
+            raise IndexError("no group %d" % group)
+        return -(-tokens // self.page_size)
+
     def capacity_tokens(self):
         """Tokens one request can hold at most (bounded by the smallest pool)."""
         if not self.groups:

@@ -116,7 +116,7 @@ class _DecodeGraph:
         m = runner.manager
         self.B = B
         self.max_kv_len = max_kv_len
-        widths = [-(-runner.max_request_tokens // m.page_size)] * len(m.groups)
+        widths = [m.table_width(g, runner.max_request_tokens) for g in range(len(m.groups))]
         n = packed_size(B, B, B, widths)
         self.host = torch.empty(n, dtype=torch.int32).pin_memory()
         self.dev = torch.zeros(n, dtype=torch.int32, device=runner.device)

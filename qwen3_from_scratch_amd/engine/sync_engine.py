@@ -103,20 +103,29 @@ class SyncEngine:
 
     # ---- set-up ----
     def _blocks_from_memory(self):
-        """Pages that fit in `gpu_utilization` of the free memory, halved for
-        keys and values, as the reference sizes its cache
-        (src/qwen3_from_scratch/inference/kv_cache/paged_cache.py:36-49)."""
-        per_token = 0
+        """Pages that fit in `gpu_utilization` of the free memory beside the
+        requests' fixed-size states, halved for keys and values, as the reference
+        sizes its cache (src/qwen3_from_scratch/inference/kv_cache/paged_cache.py:36-49).
+        A page stands for its tokens in every layer of every group."""
+        per_token = per_request = 0
         itemsize = 2 if self.model.precision.act == torch.bfloat16 else 4
         for need in self.model.plane_needs:
-            if need is not None and need.paged:
+            if need is None:
+                continue
+            if need.paged:
                 per_token += 2 * need.kv_heads * need.head_dim * itemsize
+            if need.has_state:           # a slot per request (and a spare one) in every plane that keeps a state
+                size = torch.empty((), dtype=need.state_dtype).element_size()
+                for n in need.state_shape:
+                    size *= n
+                per_request += size
         per_page = max(1, per_token * self.config.block_size)
         if self.model.device.type == "cuda":
             free = torch.cuda.mem_get_info(self.model.device)[0]
         else:
             free = 1 << 30
-        wanted = int(free * self.config.gpu_utilization) // per_page
+        budget = int(free * self.config.gpu_utilization) - per_request * (self.config.max_num_seqs + 1)
+        wanted = max(0, budget) // per_page
         enough = self.config.max_num_seqs * (-(-self.max_len // self.config.block_size))
         return max(1, min(wanted, enough))
 

@@ -32,7 +32,13 @@ class DecoderModel:
         self.device = torch.device(device)
         self.embedding = build_part(spec.embedding, spec.embedding_prefix, precision, device)
         self.position = build_part(spec.position, "", precision, device)
-        self.layers = [_Layer(ls, precision, device, self.position) for ls in spec.layers]
+        self.layer_positions = {}            # position parts that layers name for themselves, one per distinct spec
+        for ls in spec.layers:
+            if ls.position is not None and ls.position not in self.layer_positions:
+                self.layer_positions[ls.position] = build_part(ls.position, "", precision, device)
+        self.layers = [_Layer(ls, precision, device,
+                              self.position if ls.position is None else self.layer_positions[ls.position])
+                       for ls in spec.layers]
         self.final_norm = build_part(spec.final_norm, spec.final_norm_prefix, precision, device)
         self.head = build_part(spec.head, spec.head_prefix, precision, device)
         # each run-order entry that owns a cache gets a plane; readers point at the owner's
@@ -50,6 +56,7 @@ class DecoderModel:
     def parts(self):
         yield self.embedding
         yield self.position
+        yield from self.layer_positions.values()
         for layer in self.layers:
             yield from layer.parts()
         yield self.final_norm
@@ -67,7 +74,8 @@ class DecoderModel:
             for name, shape in part.tensors().items():
                 if name in names and tuple(names[name]) != tuple(shape):
                     raise ValueError("tensor %s is wanted with shapes %s and %s" % (name, names[name], shape))
-                names[name] = tuple(shape)
+                if name not in names or not hasattr(names[name], "kind"):
+                    names[name] = shape if hasattr(shape, "kind") else tuple(shape)
         return names
 
     def load(self, source):

@@ -8,7 +8,10 @@ from ..parts.base import PartSpec
 @dataclass(frozen=True)
 class LayerSpec:
     """One layer's parts. `prefix` is the layer's checkpoint name prefix; the
-    `*_prefix` fields are the sub-prefixes of its parts under it."""
+    `*_prefix` fields are the sub-prefixes of its parts under it. `position`:
+    the position part this layer's mixer asks for its rotation table, if it is
+    not the model's (layers that rotate by another base or over another part of
+    the head, or not at all); layers that name equal parts share one."""
 
     prefix: str
     mixer: PartSpec
@@ -16,6 +19,7 @@ class LayerSpec:
     mixer_norm: PartSpec
     feed_forward_norm: PartSpec
     block: PartSpec = PartSpec("block", "pre_norm")
+    position: PartSpec = None
     mixer_prefix: str = "self_attn"
     feed_forward_prefix: str = "mlp"
     mixer_norm_prefix: str = "input_layernorm"

@@ -4,7 +4,7 @@ import torch
 
 from .. import ops
 from ..config.registry import register_part
-from .base import CacheNeed, Part
+from .base import CacheNeed, Part, TensorShape
 from .linear import LinearWeight
 
 
@@ -61,8 +61,8 @@ class PagedAttention(Part):
             self._name("o_proj.weight"): (H, Hq * D),
         }
         if self.qk_norm:
-            names[self._name("q_norm.weight")] = (D,)
-            names[self._name("k_norm.weight")] = (D,)
+            names[self._name("q_norm.weight")] = TensorShape((D,), "scale")
+            names[self._name("k_norm.weight")] = TensorShape((D,), "scale")
         return names
 
     def load(self, fetch):

@@ -58,6 +58,22 @@ class PartSpec:
         return PartSpec(self.kind, self.name, tuple(sorted(merged.items())))
 
 
+class TensorShape(tuple):
+    """A tensor's shape, with a word on what the tensor is for whoever has to make
+    one up (the random-weights mode): "matrix" (products and tables: small values
+    around zero), "scale" (a norm's multiplier: values around one) or "bias"
+    (an addend: small values around zero). A plain tuple stands for a matrix."""
+
+    kind = "matrix"
+
+    def __new__(cls, shape, kind="matrix"):
+        if kind not in ("matrix", "scale", "bias"):
+            raise ValueError("a tensor is a matrix, a scale or a bias, not %r" % (kind,))
+        self = super().__new__(cls, tuple(shape))
+        self.kind = kind
+        return self
+
+
 class Part:
     """Base class. `prefix` is the checkpoint name prefix of the part's tensors."""
 
@@ -76,7 +92,8 @@ class Part:
         self.device = torch.device(device)
 
     def tensors(self):
-        """{checkpoint tensor name: shape} of everything this part loads."""
+        """{checkpoint tensor name: shape} of everything this part loads; a
+        shape is a tuple, or a `TensorShape` that also says what the tensor is."""
         return {}
 
     def load(self, fetch):

@@ -4,7 +4,7 @@ import torch
 
 from .. import ops
 from ..config.registry import register_part
-from .base import NormSink, Part
+from .base import NormSink, Part, TensorShape
 
 
 @register_part("norm", "rms")
@@ -24,7 +24,7 @@ class RMSNorm(Part):
         self.weight = None
 
     def tensors(self):
-        return {self._name("weight"): (self.size,)}
+        return {self._name("weight"): TensorShape((self.size,), "scale")}
 
     def load(self, fetch):
         self.weight = fetch(self._name("weight"))

@@ -22,8 +22,9 @@ def _tensor_seed(seed, name):
 
 
 class RandomWeights(TensorSource):
-    """Matrices and embeddings N(0, std); one-dimensional tensors (norm
-    weights) 1 + U(-jitter, jitter). All in bfloat16."""
+    """Each tensor by what its part says it is (`TensorShape.kind`): a matrix
+    (also a table, and any tensor whose part says nothing) N(0, std), a scale
+    1 + U(-jitter, jitter), a bias N(0, std). All in bfloat16."""
 
     def __init__(self, expected, seed=0, std=0.02, norm_jitter=0.1, generate_on=None):
         self.where = "<random weights, seed %d>" % seed
@@ -44,7 +45,7 @@ class RandomWeights(TensorSource):
         on = torch.device(self.generate_on) if self.generate_on is not None else torch.device("cpu")
         gen = torch.Generator(device=on)
         gen.manual_seed(_tensor_seed(self.seed, name))
-        if len(shape) == 1:
+        if getattr(self._expected[name], "kind", "matrix") == "scale":
             t = torch.rand(shape, generator=gen, device=on, dtype=torch.float32)
             t = 1.0 + (2.0 * t - 1.0) * self.norm_jitter
         else:

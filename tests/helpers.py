@@ -42,6 +42,14 @@ TINY = {
                     rope_theta=500000.0, tie_word_embeddings=False),
         seed=43, std=0.04, norm_jitter=0.2, page_size=32),
 }
+# D and E with weights so large that logits span ten units or more, where a rounding of bfloat16
+# is small beside a fault; and with query norms twice as large, so that every query's
+# softmax stands on a few keys, most of them far back: a key or a tile left out then shows in
+# the logits of the rows that stood on it
+TINY["DS"] = dict(TINY["D"], seed=45, std=0.2)
+TINY["ES"] = dict(TINY["E"], seed=47, std=0.2)
+TINY["DP"] = dict(TINY["D"], seed=49, std=0.2, peak=2.0)
+TINY["EP"] = dict(TINY["E"], seed=51, std=0.2, peak=2.0)
 
 
 def tiny_config(name):
@@ -51,6 +59,15 @@ def tiny_config(name):
 def make_folder(folder, name):
     t = TINY[name]
     write_random_model(folder, tiny_config(name), seed=t["seed"], std=t["std"], norm_jitter=t["norm_jitter"])
+    if t.get("peak"):
+        from safetensors.torch import load_file, save_file
+
+        path = os.path.join(folder, "model.safetensors")
+        tensors = load_file(path)
+        for key in tensors:
+            if key.endswith("q_norm.weight"):
+                tensors[key] = (tensors[key].float() * t["peak"]).to(tensors[key].dtype)
+        save_file(tensors, path, metadata={"format": "pt"})
     return folder
 
 
@@ -202,3 +219,26 @@ def arrivals_scenario(folder, lookahead, num_blocks, name="B", device="cpu", dty
     assert not engine.scheduler.has_work()
     assert engine.runner.manager.num_free() == num_blocks
     return [list(r.generated) for r in requests], [r.preemptions for r in requests], ahead[0]
+
+
+# ---- how far logits may be off ----
+# float32: rounding order only, 2e-4 of the row's largest magnitude (at least 1). bfloat16: a
+# fiftieth of the row's spread (largest minus smallest logit): a handful of 8-bit roundings, far
+# less than what a key, a tile or a page left out does to a row.
+BF16_SHARE = 2e-2
+
+
+def off_by(got_row, want_row, dtype):
+    """The largest difference between two rows of logits, in units of what `dtype` may be off by
+    (1.0 = at the bound)."""
+    diff = float((got_row.float() - want_row.float()).abs().max())
+    if dtype == "float32":
+        return diff / (2e-4 * max(1.0, float(want_row.abs().max())))
+    return diff / (BF16_SHARE * float(want_row.max() - want_row.min()))
+
+
+def nearly_the_best(logits_row, token, share=BF16_SHARE):
+    """Whether `token` is the row's largest logit or within `share` of the row's spread of it:
+    what a greedy choice made from logits that are off by that much may be."""
+    spread = float(logits_row.max() - logits_row.min())
+    return float(logits_row[token]) >= float(logits_row.max()) - share * spread

@@ -16,9 +16,10 @@ from qwen3_from_scratch_amd.engine import load_runner
 pytestmark = pytest.mark.gpu
 
 # float32: the engine and the plain implementation differ by rounding order only.
-# bfloat16: activations are rounded to 8 bits of mantissa between kernels; the
-# bound is a fraction of the logits' spread, which the weights' scale sets.
-TOL = {"float32": 2e-4, "bfloat16": 6e-2}
+# bfloat16: activations are rounded to 8 bits of mantissa between kernels; a row's logits may
+# be off by a fiftieth of the row's own spread (largest minus smallest logit), which is what a
+# handful of such roundings come to and far less than a key, a tile or a page left out.
+TOL = {"float32": 2e-4, "bfloat16": 2e-2}
 
 _plain_cache = {}
 
@@ -42,20 +43,24 @@ def _plain(folder, name, requests):
 
 
 def _compare(got, want, dtype):
-    worst, scale = 0.0, 0.0
+    worst, where = 0.0, None
     for rid, logits in want.items():
-        scale = max(scale, float(logits.abs().max()))
         for p in range(logits.shape[0]):
             assert (rid, p) in got, "no logits for %s at %d" % (rid, p)
             diff = float((got[(rid, p)] - logits[p]).abs().max())
-            if diff > worst:
-                worst, where = diff, (rid, p)
-    bound = TOL[dtype] * max(1.0, scale)
-    assert worst <= bound, "largest difference %g at %s (bound %g)" % (worst, where, bound)
+            if dtype == "float32":
+                unit = max(1.0, float(logits[p].abs().max()))
+            else:
+                unit = float(logits[p].max() - logits[p].min())
+            if diff / unit > worst:
+                worst, where = diff / unit, (rid, p, diff, unit)
+    assert worst <= TOL[dtype], "largest difference %g of its unit at %s (bound %g)" % (worst, where, TOL[dtype])
+    return worst
 
 
 CASES = [("A", [5, 17, 33, 80]), ("B", [1, 9, 64, 130]), ("C", [40, 70, 3, 201]),
-         ("D", [33, 1, 150, 64, 300]), ("E", [129, 31, 260])]
+         ("D", [33, 1, 150, 64, 300]), ("E", [129, 31, 260]),
+         ("DS", [33, 1, 150, 64, 300]), ("ES", [129, 31, 260]), ("DP", [200, 17, 330, 64]), ("EP", [129, 300, 70])]
 FAMILIES = {"whole": trace_whole, "tail": trace_tail_decoded, "portions": trace_portions, "mixed": trace_mixed}
 
 

@@ -11,7 +11,8 @@ import pytest
 import torch
 
 import plain_qwen3
-from helpers import TINY, arrivals_scenario, max_live_tokens, random_tokens, trace_mixed, trace_portions
+from helpers import (TINY, arrivals_scenario, max_live_tokens, nearly_the_best, off_by, random_tokens, trace_mixed,
+                     trace_portions)
 from qwen3_from_scratch_amd.engine import SyncEngine
 
 pytestmark = pytest.mark.gpu
@@ -75,10 +76,14 @@ def test_bfloat16_generation_and_seeded_sampling(model_folders):
     prompts = [random_tokens(n, vocab, 50 + n) for n in (1, 9, 64, 130)]
     kw = dict(path=model_folders["B"], dtype="bfloat16", block_size=8, num_blocks=64, max_num_tokens=30,
               chunked_prefill_size=24)
-    want = _plain_greedy(model_folders["B"], prompts, 6)
     got = SyncEngine(max_num_seqs=4, **kw).generate_ids(prompts, 6, temperature=0.0, ignore_eos=True)
-    # bfloat16 may flip a near-tie now and then; the first tokens of most requests agree
-    assert sum(g[0] == w[0] for g, w in zip(got, want)) >= 3
+    # bfloat16 may flip a near-tie: every token is the plain implementation's best or within a
+    # fiftieth of the row's spread of it, given the tokens before it
+    cfg, w = plain_qwen3.read_model_folder(model_folders["B"])
+    for prompt, new in zip(prompts, got):
+        logits = plain_qwen3.logits_of_sequence(cfg, w, prompt + new)
+        for i, token in enumerate(new):
+            assert nearly_the_best(logits[len(prompt) + i - 1], token), (len(prompt), i)
     a = SyncEngine(max_num_seqs=4, **kw).generate_ids(prompts, 6, temperature=0.8, top_k=20, seed=3, ignore_eos=True)
     b = SyncEngine(max_num_seqs=1, **kw).generate_ids(prompts[2:3], 6, temperature=0.8, top_k=20, seed=3,
                                                       ignore_eos=True)
@@ -181,14 +186,12 @@ def test_trace_run_program(model_folders, tmp_path, dtype):
     requests = {"q%d" % i: random_tokens(n, vocab, 80 + i) for i, n in enumerate([50, 90, 7, 130, 64, 33])}
     cfg, w = plain_qwen3.read_model_folder(model_folders[name])
     want = {rid: plain_qwen3.logits_of_sequence(cfg, w, toks) for rid, toks in requests.items()}
-    tol = 2e-4 if dtype == "float32" else 6e-2
     for label, steps in (("mixed", trace_mixed(requests, seed=4)), ("portions", trace_portions(requests))):
         got = _replay(model_folders[name], dtype, steps, str(tmp_path / (label + dtype)),
                       max_live_tokens(steps, page=64))
         for rid, logits in want.items():
-            scale = max(1.0, float(logits.abs().max()))
             for p in range(logits.shape[0]):
-                assert float((got[(rid, p)] - logits[p]).abs().max()) <= tol * scale, (label, rid, p)
+                assert off_by(got[(rid, p)], logits[p], dtype) <= 1.0, (label, rid, p)
 
 
 def test_trace_run_answers_step_by_step(model_folders, tmp_path):

@@ -135,3 +135,117 @@ def test_tied_head_is_the_embedding(model_folders):
     assert cfg["tie_word_embeddings"] and "lm_head.weight" not in w
     cfg_b, w_b = plain.read_model_folder(model_folders["B"])
     assert not cfg_b["tie_word_embeddings"] and "lm_head.weight" in w_b
+
+
+def test_head_norms_come_before_the_rotation():
+    """With norm weights that differ between the two elements of a rotated pair, scores depend
+    on the distance alone only if the norm comes first and the rotation last: the other order
+    multiplies the halves of a rotated pair by different numbers and the property is gone."""
+    g = torch.Generator().manual_seed(5)
+    T, H, Hq, Hkv, D = 6, 24, 2, 1, 16
+    cfg = dict(num_attention_heads=Hq, num_key_value_heads=Hkv, head_dim=D, rms_norm_eps=1e-6, rope_theta=100.0)
+    w = {"a.%s_proj.weight" % n: torch.randn(rows, H, generator=g, dtype=torch.float64)
+         for n, rows in (("q", Hq * D), ("k", Hkv * D), ("v", Hkv * D))}
+    w["a.o_proj.weight"] = torch.randn(H, Hq * D, generator=g, dtype=torch.float64)
+    gamma = torch.cat((torch.full((D // 2,), 0.3), torch.full((D // 2,), 2.5))).double()
+    w["a.q_norm.weight"], w["a.k_norm.weight"] = gamma, 1.5 * gamma
+    x = torch.randn(T, H, generator=g, dtype=torch.float64)
+    here = plain.self_attention(x, w, "a", cfg, torch.arange(T))
+    there = plain.self_attention(x, w, "a", cfg, torch.arange(T) + 1000)
+    torch.testing.assert_close(here, there, rtol=1e-9, atol=1e-9)
+
+    def other_order(positions):
+        q = (x @ w["a.q_proj.weight"].T).view(T, Hq, D)
+        k = (x @ w["a.k_proj.weight"].T).view(T, Hkv, D)
+        v = (x @ w["a.v_proj.weight"].T).view(T, Hkv, D)
+        ang = plain.rotary_angles(positions, D, 100.0, torch.float64)
+        q = plain.rms_norm(plain.apply_rotary(q, ang), w["a.q_norm.weight"], 1e-6)
+        k = plain.rms_norm(plain.apply_rotary(k, ang), w["a.k_norm.weight"], 1e-6)
+        return plain.causal_attention(q, k, v, D ** -0.5).reshape(T, Hq * D) @ w["a.o_proj.weight"].T
+
+    assert not torch.allclose(other_order(torch.arange(T)), other_order(torch.arange(T) + 1000), atol=1e-3)
+    assert not torch.allclose(other_order(torch.arange(T)), here, atol=1e-3)
+
+
+def _one_layer(g, zero):
+    V, H, I, Hq, Hkv, D = 50, 24, 40, 2, 1, 16
+    cfg = dict(num_hidden_layers=1, num_attention_heads=Hq, num_key_value_heads=Hkv, head_dim=D, rms_norm_eps=1e-5,
+               rope_theta=1e4, tie_word_embeddings=False, vocab_size=V)
+    shapes = {"model.embed_tokens.weight": (V, H), "lm_head.weight": (V, H),
+              "model.layers.0.self_attn.q_proj.weight": (Hq * D, H), "model.layers.0.self_attn.k_proj.weight": (Hkv * D, H),
+              "model.layers.0.self_attn.v_proj.weight": (Hkv * D, H), "model.layers.0.self_attn.o_proj.weight": (H, Hq * D),
+              "model.layers.0.mlp.gate_proj.weight": (I, H), "model.layers.0.mlp.up_proj.weight": (I, H),
+              "model.layers.0.mlp.down_proj.weight": (H, I)}
+    w = {n: torch.randn(s, generator=g) * 0.3 for n, s in shapes.items()}
+    for n in ("model.layers.0.input_layernorm.weight", "model.layers.0.post_attention_layernorm.weight",
+              "model.norm.weight"):
+        w[n] = 1 + 0.3 * torch.randn(H, generator=g)
+    w["model.layers.0.self_attn.q_norm.weight"] = 1 + 0.3 * torch.randn(D, generator=g)
+    w["model.layers.0.self_attn.k_norm.weight"] = 1 + 0.3 * torch.randn(D, generator=g)
+    for n in zero:
+        w[n] = torch.zeros_like(w[n])
+    return cfg, w
+
+
+def test_a_block_whose_parts_give_nothing_is_the_identity():
+    """The norms sit before the parts and the stream is added outside them: with both output
+    matrices zero a layer changes nothing, whatever the norms' weights; a norm on the stream
+    itself (after the addition) would show."""
+    g = torch.Generator().manual_seed(6)
+    cfg, w = _one_layer(g, ("model.layers.0.self_attn.o_proj.weight", "model.layers.0.mlp.down_proj.weight"))
+    x = torch.randn(7, 24, generator=g) * 5.0
+    assert torch.equal(plain.decoder_layer(x, w, 0, cfg, torch.arange(7)), x)
+
+
+def test_one_layer_without_attention_reduces_to_library_routines():
+    """Embedding rows as they are (no factor), the second norm before the feed-forward, the sum
+    outside it, the final norm, the head: with the attention's output matrix zero the whole
+    model is a few library calls. A scaled embedding would change the balance between the
+    stream and the feed-forward's addend, whose size does not depend on the stream's."""
+    g = torch.Generator().manual_seed(7)
+    cfg, w = _one_layer(g, ("model.layers.0.self_attn.o_proj.weight",))
+    toks = [3, 17, 3, 44, 0, 49]
+    x0 = F.embedding(torch.tensor(toks), w["model.embed_tokens.weight"])
+    h = F.rms_norm(x0, (24,), w["model.layers.0.post_attention_layernorm.weight"], 1e-5)
+    mlp = F.linear(F.silu(F.linear(h, w["model.layers.0.mlp.gate_proj.weight"]))
+                   * F.linear(h, w["model.layers.0.mlp.up_proj.weight"]), w["model.layers.0.mlp.down_proj.weight"])
+    want = F.linear(F.rms_norm(x0 + mlp, (24,), w["model.norm.weight"], 1e-5), w["lm_head.weight"])
+    torch.testing.assert_close(plain.logits_of_sequence(cfg, w, toks), want, rtol=1e-5, atol=1e-5)
+    scaled = F.linear(F.rms_norm(x0 * 24 ** 0.5 + mlp, (24,), w["model.norm.weight"], 1e-5), w["lm_head.weight"])
+    assert not torch.allclose(scaled, want, atol=1e-2)
+
+
+def test_peaked_weights_make_one_missing_key_show(model_folders, monkeypatch):
+    """The tiny configurations with large weights and large query norms are there so that a key
+    left out of the attention shows in the logits beyond the bound of the bfloat16 comparisons
+    (a fiftieth of a row's spread), also for rows that have sixty other keys or more."""
+    from helpers import random_tokens
+
+    def worst_share(name, hidden_key):
+        cfg, w = plain.read_model_folder(model_folders[name])
+        toks = random_tokens(120, cfg["vocab_size"], 13)
+        full = plain.logits_of_sequence(cfg, w, toks)
+        whole = plain.causal_attention
+
+        def without_one_key(q, k, v, scale, window=None):
+            out = whole(q, k, v, scale, window)
+            T = q.shape[0]
+            keep = [j for j in range(T) if j != hidden_key]
+            later = whole(q[keep], k[keep], v[keep], scale, window)     # the sequence as if that token's key were not there
+            out = out.clone()
+            for row, i in enumerate(keep):
+                if i > hidden_key:
+                    out[i] = later[row]
+            return out
+
+        monkeypatch.setattr(plain, "causal_attention", without_one_key)
+        lacking = plain.logits_of_sequence(cfg, w, toks)
+        monkeypatch.setattr(plain, "causal_attention", whole)
+        spread = full.max(dim=1).values - full.min(dim=1).values
+        share = (lacking - full).abs().max(dim=1).values / spread
+        far = share[60:]                                               # rows with sixty keys or more
+        return float(share.max()), float((far > 2e-2).float().mean())
+
+    for name in ("DP", "EP"):
+        worst, far_rows_over = worst_share(name, hidden_key=7)
+        assert worst > 0.2 and far_rows_over > 0.3, (name, worst, far_rows_over)

@@ -8,7 +8,8 @@ import pytest
 import torch
 
 import plain_qwen3
-from helpers import max_live_tokens, random_tokens, run_trace, trace_mixed, trace_tail_decoded
+from helpers import (max_live_tokens, nearly_the_best, off_by, random_tokens, run_trace, trace_mixed,
+                     trace_tail_decoded)
 from qwen3_from_scratch_amd.config import ModelConfig
 from qwen3_from_scratch_amd.engine import StepEntry, load_runner
 from qwen3_from_scratch_amd.weights import write_random_model
@@ -38,19 +39,17 @@ def truth(folder):
     return requests, rows, want
 
 
-@pytest.mark.parametrize("dtype,tol", [("float32", 3e-4), ("bfloat16", 6e-2)])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("family", ["tail", "mixed"])
-def test_real_layer_sizes_match_plain(folder, truth, dtype, tol, family):
+def test_real_layer_sizes_match_plain(folder, truth, dtype, family):
     requests, rows, want = truth
     steps = (trace_tail_decoded(requests, tail=32) if family == "tail" else trace_mixed(requests, seed=2))
     runner = load_runner(folder, dtype=dtype, page_size=16, max_tokens=max_live_tokens(steps, page=16),
                          max_requests=4)
     got = run_trace(runner, steps)
     for rid, logits in want.items():
-        scale = max(1.0, float(logits.abs().max()))
         for i, p in enumerate(rows[rid]):
-            diff = float((got[(rid, p)] - logits[i]).abs().max())
-            assert diff <= tol * scale, (rid, p, diff, scale)
+            assert off_by(got[(rid, p)], logits[i], dtype) <= (1.5 if dtype == "float32" else 1.0), (rid, p)
 
 
 def test_schedules_agree_at_real_sizes(folder):
@@ -107,11 +106,10 @@ def test_long_prompt_in_portions_at_real_sizes(folder):
     for portion in (3000, 512, 300):
         got = run("bfloat16", portion)
         for p in places:
-            scale = max(1.0, float(truth[p].abs().max()))
-            assert float((got[p] - truth[p]).abs().max()) <= 6e-2 * scale, (portion, p)
+            assert off_by(got[p], truth[p], "bfloat16") <= 1.0, (portion, p)
     again = run("float32", 700)
     for p in places:
-        assert float((again[p] - truth[p]).abs().max()) <= 3e-4 * max(1.0, float(truth[p].abs().max())), p
+        assert off_by(again[p], truth[p], "float32") <= 1.5, p
 
 
 def test_some_tens_of_rows_at_real_sizes(folder):
@@ -148,8 +146,7 @@ def test_some_tens_of_rows_at_real_sizes(folder):
             ops.matmul_kernels("both")
         assert set(want) == set(got) and len(got) == count * 7
         for key, logits in want.items():
-            scale = max(1.0, float(logits.abs().max()))
-            assert float((got[key] - logits).abs().max()) <= 6e-2 * scale, (which, key)
+            assert off_by(got[key], logits, "bfloat16") <= 1.0, (which, key)
 
     def generate(max_num_seqs):
         engine = SyncEngine(path=folder, dtype="bfloat16", block_size=16, num_blocks=count * 8,
@@ -158,8 +155,14 @@ def test_some_tens_of_rows_at_real_sizes(folder):
         return engine.generate_ids(prompts, max_new_tokens=12, temperature=0.0, ignore_eos=True)
 
     together, few = generate(count), generate(4)
-    # bfloat16 rounds differently along the two paths: a near tie between two tokens may fall
-    # either way, and the tokens after it then differ too; a fault would leave nothing equal
-    first = sum(a[0] == b[0] for a, b in zip(together, few))
-    all_of_them = sum(x == y for a, b in zip(together, few) for x, y in zip(a, b))
-    assert first >= count - 3 and all_of_them >= 0.6 * count * 12, (first, all_of_them)
+    # bfloat16 rounds differently along the two paths and a near tie between two tokens may fall
+    # either way: every token of either run is the float32 engine's best, or within a fiftieth of
+    # the row's spread of it, given the tokens before it
+    judge = load_runner(folder, dtype="float32", page_size=16, max_tokens=128, max_requests=1)
+    for run_tokens in (together, few):
+        for prompt, new in zip(prompts, run_tokens):
+            places = [len(prompt) - 1 + i for i in range(len(new))]
+            logits = judge.step([StepEntry("judge", prompt + new, places)]).float().cpu()
+            judge.finish("judge")
+            for i, token in enumerate(new):
+                assert nearly_the_best(logits[i], token), (len(prompt), i)

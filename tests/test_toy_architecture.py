@@ -59,6 +59,24 @@ def test_folder_is_read_by_its_architectures_own_keys(folder):
     assert "hybrid.layers.%d.self_attn.mix.weight" % mean_layer in names
     assert "hybrid.layers.%d.self_attn.q_proj.weight" % attention_layer in names
     assert ("hybrid.norm.bias" in names) == (config.norm == "centred")
+    if config.norm == "centred":
+        # the parts say what their tensors are: a scale is drawn around one, a bias around zero
+        tensors = load_file(os.path.join(folder, "model.safetensors"))
+        assert abs(float(tensors["hybrid.norm.weight"].float().mean()) - 1.0) < 0.1
+        assert abs(float(tensors["hybrid.norm.bias"].float().mean())) < 0.05
+        assert float(tensors["hybrid.norm.bias"].float().abs().max()) < 0.5
+
+
+def test_a_layer_with_a_position_part_of_its_own(folder):
+    """Layers `b` name a rotation of their own (half of each head, another base); the model
+    keeps it beside its own, once, however many layers name it."""
+    from qwen3_from_scratch_amd.config import lookup_architecture
+
+    config = load_model_config(folder)
+    spec = lookup_architecture(toy.NAME)[1](config)
+    own = [ls.position for ls in spec.layers if ls.position is not None]
+    assert len(own) == config.pattern.count("b") >= 1 and len(set(own)) == 1
+    assert own[0].get("rotary_dim") == config.head_size // 2 and own[0] != spec.position
 
 
 def test_every_cutting_and_generation_on_the_host(cpu_ops, folder):
@@ -81,6 +99,22 @@ def test_every_cutting_and_generation_on_the_host(cpu_ops, folder):
         for _ in range(6):
             seq.append(int(torch.argmax(toy.plain_logits(config, w, seq)[-1])))
         assert new == seq[len(prompt):]
+
+
+def test_cache_sizing_counts_the_states(cpu_ops, folder):
+    """Sized from memory, the cache leaves room for every request's fixed-size states."""
+    kw = dict(path=folder, dtype="float32", device="cpu", max_len=256, block_size=8, max_num_tokens=24,
+              gpu_utilization=3e-4)                       # of the gigabyte a host engine pretends to have
+    few, many = SyncEngine(max_num_seqs=2, **kw), SyncEngine(max_num_seqs=40, **kw)
+    needs = few.model.plane_needs
+    per_page = sum(2 * n.kv_heads * n.head_dim * 4 for n in needs if n is not None and n.paged) * 8
+    per_request = sum(4 * int(np.prod(n.state_shape)) for n in needs if n is not None and n.has_state)
+    assert per_request > 0
+    budget = int((1 << 30) * 3e-4)
+    whole = -(-min(256, few.model.config.max_position_embeddings) // 8)      # pages of one request of full length
+    assert few.runner.manager.num_pages() == min((budget - 3 * per_request) // per_page, 2 * whole)
+    assert many.runner.manager.num_pages() == (budget - 41 * per_request) // per_page < 40 * whole
+    assert (budget - 41 * per_request) // per_page < (budget - 3 * per_request) // per_page
 
 
 def _replay(folder, dtype, steps, out, max_tokens, plugins):

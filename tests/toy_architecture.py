@@ -1,8 +1,9 @@
 """A whole architecture that lives outside the framework: its own config.json keys, its
 own configuration class, a function from that configuration to a ModelSpec, and one
 `register_architecture` call. Layers follow a pattern string: `a` is the framework's
-attention (with a window), `s` the running-mean mixer of test_toy_parts.py, which keeps a
-state of fixed size per request. Two more keys choose between the framework's RMS norm and a
+attention (with a window), `b` the same attention without a window and with a position part of
+its own (a rotation over the first half of each head only, by another base), `s` the
+running-mean mixer of test_toy_parts.py, which keeps a state of fixed size per request. Two more keys choose between the framework's RMS norm and a
 mean-subtracting norm with a bias defined here, and between the framework's sequential block
 and a block defined here whose mixer and feed-forward read the same stream. It is no model of anyone's; it shows that the loader, the
 random-weights writer, the cache manager, the step function, the engine and the replay
@@ -22,9 +23,10 @@ import test_toy_parts  # registers the mixer "toy_running_mean"  # noqa: F401
 from qwen3_from_scratch_amd.config import register_architecture, register_part
 from qwen3_from_scratch_amd.config.model_config import ConfigError
 from qwen3_from_scratch_amd.models import LayerSpec, ModelSpec, RunStep
-from qwen3_from_scratch_amd.parts import Part, PartSpec
+from qwen3_from_scratch_amd.parts import Part, PartSpec, TensorShape
 
 NAME = "ToyHybridForCausalLM"
+OTHER_BASE = 7.0     # a `b` layer rotates by theta / 7
 KEYS = (("vocab", int), ("width", int), ("inner", int), ("heads", int), ("kv_heads", int), ("head_size", int),
         ("pattern", str), ("window", int), ("eps", float), ("theta", float), ("max_position_embeddings", int),
         ("norm", str), ("arrangement", str))
@@ -42,7 +44,8 @@ class CentredNorm(Part):
         self.weight = self.bias = None
 
     def tensors(self):
-        return {self._name("weight"): (self.size,), self._name("bias"): (self.size,)}
+        return {self._name("weight"): TensorShape((self.size,), "scale"),
+                self._name("bias"): TensorShape((self.size,), "bias")}
 
     def load(self, fetch):
         self.weight = fetch(self._name("weight"), torch.float32)
@@ -105,8 +108,8 @@ class ToyHybridConfig:
         missing = [k for k, _ in KEYS if k not in data]
         if missing:
             raise ConfigError("config.json of %s lacks %s" % (NAME, ", ".join(missing)))
-        if not data["pattern"] or set(data["pattern"]) - set("as"):
-            raise ConfigError("pattern must be a string of 'a' and 's'")
+        if not data["pattern"] or set(data["pattern"]) - set("abs"):
+            raise ConfigError("pattern must be a string of 'a', 'b' and 's'")
         if data["norm"] not in ("rms", "centred") or data["arrangement"] not in ("sequential", "parallel"):
             raise ConfigError("norm is rms or centred, arrangement sequential or parallel")
         return cls(architecture=data["architectures"][0], **{k: kind(data[k]) for k, kind in KEYS})
@@ -123,10 +126,15 @@ def toy_hybrid_spec(c):
     block = PartSpec.of("block", "pre_norm" if c.arrangement == "sequential" else "toy_parallel")
     attention = PartSpec.of("mixer", "attention", hidden_size=c.width, num_heads=c.heads, num_kv_heads=c.kv_heads,
                             head_dim=c.head_size, qk_norm=False, qk_norm_eps=c.eps, window=c.window)
+    everything = attention.with_params(window=0)
+    half_rotation = PartSpec.of("position", "rotary", rotary_dim=c.head_size // 2, theta=c.theta / OTHER_BASE,
+                                max_positions=c.max_position_embeddings)
     mean = PartSpec.of("mixer", "toy_running_mean", hidden_size=c.width)
     ff = PartSpec.of("feed_forward", "swiglu", hidden_size=c.width, intermediate_size=c.inner)
-    layers = tuple(LayerSpec(prefix="hybrid.layers.%d" % i, mixer=attention if kind == "a" else mean, feed_forward=ff,
-                             mixer_norm=norm, feed_forward_norm=norm, block=block) for i, kind in enumerate(c.pattern))
+    mixers = {"a": attention, "b": everything, "s": mean}
+    layers = tuple(LayerSpec(prefix="hybrid.layers.%d" % i, mixer=mixers[kind], feed_forward=ff,
+                             mixer_norm=norm, feed_forward_norm=norm, block=block,
+                             position=half_rotation if kind == "b" else None) for i, kind in enumerate(c.pattern))
     return ModelSpec(
         hidden_size=c.width, vocab_size=c.vocab,
         embedding=PartSpec.of("embedding", "token", vocab_size=c.vocab, hidden_size=c.width),
@@ -140,11 +148,11 @@ def toy_hybrid_spec(c):
 
 register_architecture(NAME, ToyHybridConfig, toy_hybrid_spec)
 
-EXAMPLE = dict(architectures=[NAME], vocab=211, width=40, inner=72, heads=6, kv_heads=2, head_size=16, pattern="asa",
+EXAMPLE = dict(architectures=[NAME], vocab=211, width=40, inner=72, heads=6, kv_heads=2, head_size=16, pattern="asab",
                window=21, eps=1e-5, theta=10000.0, max_position_embeddings=512, norm="rms", arrangement="sequential")
 # every size and option differs; the norm and the block are the ones defined above
 EXAMPLE_PARALLEL = dict(architectures=[NAME], vocab=157, width=56, inner=100, heads=4, kv_heads=4, head_size=32,
-                        pattern="saas", window=0, eps=1e-6, theta=500000.0, max_position_embeddings=300,
+                        pattern="sbas", window=0, eps=1e-6, theta=500000.0, max_position_embeddings=300,
                         norm="centred", arrangement="parallel")
 
 
@@ -169,11 +177,19 @@ def plain_logits(c, w, tokens):
             mixed = mean @ w[p + ".self_attn.mix.weight"].T
         else:
             a = p + ".self_attn"
-            ang = plain.rotary_angles(pos, c.head_size, c.theta, torch.float32)
-            q = plain.apply_rotary((h @ w[a + ".q_proj.weight"].T).view(T, c.heads, c.head_size), ang)
-            k = plain.apply_rotary((h @ w[a + ".k_proj.weight"].T).view(T, c.kv_heads, c.head_size), ang)
+            q = (h @ w[a + ".q_proj.weight"].T).view(T, c.heads, c.head_size)
+            k = (h @ w[a + ".k_proj.weight"].T).view(T, c.kv_heads, c.head_size)
+            if kind == "a":
+                ang = plain.rotary_angles(pos, c.head_size, c.theta, torch.float32)
+                q, k = plain.apply_rotary(q, ang), plain.apply_rotary(k, ang)
+            else:       # the first half of each head rotates, by another base; the second half stays
+                R = c.head_size // 2
+                ang = plain.rotary_angles(pos, R, c.theta / OTHER_BASE, torch.float32)
+                q = torch.cat((plain.apply_rotary(q[..., :R], ang), q[..., R:]), dim=-1)
+                k = torch.cat((plain.apply_rotary(k[..., :R], ang), k[..., R:]), dim=-1)
             v = (h @ w[a + ".v_proj.weight"].T).view(T, c.kv_heads, c.head_size)
-            o = plain.causal_attention(q, k, v, 1.0 / math.sqrt(c.head_size), c.window or None)
+            o = plain.causal_attention(q, k, v, 1.0 / math.sqrt(c.head_size),
+                                       (c.window or None) if kind == "a" else None)
             mixed = o.reshape(T, c.heads * c.head_size) @ w[a + ".o_proj.weight"].T
         if c.arrangement == "parallel":
             x = x + mixed + plain.swiglu_mlp(_norm(c, x, w, p + ".post_attention_layernorm"), w, p + ".mlp")

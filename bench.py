@@ -8,7 +8,8 @@ through the engine's own step loop (scheduler, step function, sampling). A
 "step" is one decode step of the whole batch. One JSON line is printed:
 `value` is decoded tokens per second at the default batch; `prefill` is one
 2,048-token prompt in one step (the median of three); `roofline` prices the decode step against HBM
-bandwidth; `points` holds decoding at batch 1 and 64. The default run is the
+bandwidth, the published peak and the rate a plain read kernel reaches on this GPU (`measured_peak`);
+`points` holds decoding at batch 1 and 64, `points_roofline` their fractions of the published peak. The default run is the
 8B shape with prompts of 2,048 in a context of 8,192; `--shape`, `--prompt` and
 `--context` move the decode measurement to the larger shapes and to longer
 contexts (the prefill measurement stays at 2,048 tokens).
@@ -361,6 +362,14 @@ def main():
             points["decode_b%d" % b] = round(p_tps, 1)
             points_roofline["decode_b%d" % b] = round(decode_bytes(config, p_contexts, itemsize) / p_step_s / PEAK_HBM, 4)
     resident = sum(t.untyped_storage().nbytes() for t in _model_tensors(model))
+    # what this GPU delivers, measured here: a plain read of 4 GB, the matrix instruction from registers
+    from qwen3_from_scratch_amd import ops
+    read_rate, matrix_rate = ops.measured_read_rate(), ops.measured_matrix_rate()
+    roofline["measured_peak"] = round(read_rate / 1e9, 1)
+    roofline["frac_of_measured"] = round(need / step_s / read_rate, 4)
+    if prefill is not None and args.dtype == "bfloat16":
+        prefill["measured_peak_tflops"] = round(matrix_rate / 1e12, 1)
+        prefill["frac_of_measured"] = round(prefill_flops(config, PREFILL) / prefill_s / matrix_rate, 4)
 
     line = {
         "metric": "decode tok/s at batch 1/8/64 + prefill tok/s at 2048 tokens, %s %s"

@@ -1,6 +1,6 @@
 """Command line: generate from a model folder, or make one with random weights.
 
-    python -m qwen3_from_scratch_amd --config_path engine.yaml --model qwen3-0.6b --prompt "..."
+    python -m qwen3_from_scratch_amd --config_path engine.yaml --model qwen3-0.6b --prompt "..." [--chat]
     python -m qwen3_from_scratch_amd --path DIR --prompt_ids 5,17,3 --max_new_tokens 16 --temperature 0
     python -m qwen3_from_scratch_amd --write_random DIR --from_config config.json --seed 1
 
@@ -24,6 +24,9 @@ def main(argv=None):
     p.add_argument("--max_len", type=int, default=None)
     p.add_argument("--prompt", action="append", default=[], help="text prompt (needs a tokenizer); repeatable")
     p.add_argument("--prompt_ids", action="append", default=[], help="comma-separated token ids; repeatable")
+    p.add_argument("--chat", action="store_true",
+                   help="each --prompt is a user's message: the tokenizer's chat template is applied, with the "
+                        "opening of the assistant's turn (as the reference's examples send their prompts)")
     p.add_argument("--max_new_tokens", type=int, default=None)
     p.add_argument("--temperature", type=float, default=None)
     p.add_argument("--top_k", type=int, default=None)
@@ -72,7 +75,8 @@ def main(argv=None):
         engine = SyncEngine(path=args.path, log_interval=args.log_interval, **overrides)
     else:
         p.error("give --config_path and --model, or --path")
-    prompts = list(args.prompt) + [[int(t) for t in s.split(",") if t.strip()] for s in args.prompt_ids]
+    texts = [[{"role": "user", "content": t}] for t in args.prompt] if args.chat else list(args.prompt)
+    prompts = texts + [[int(t) for t in s.split(",") if t.strip()] for s in args.prompt_ids]
     if not prompts:
         p.error("give --prompt or --prompt_ids")
     sampling = {}

@@ -47,6 +47,8 @@ __all__ = [
     "matmul_plan",
     "tile_weight",
     "sample",
+    "measured_read_rate",
+    "measured_matrix_rate",
 ]
 
 _DT = {torch.float32: 0, torch.bfloat16: 1}
@@ -721,3 +723,42 @@ def sample(logits, temperature, top_k, seed, counter, out=None, any_top_k=True):
             _ptr(logits), _ptr(temperature), _ptr(top_k), _ptr(seed), _ptr(counter), _ptr(out),
             R, V, 1 if any_top_k else 0, _ptr(workspace), _stream()), "sample")
     return out
+
+
+def measured_read_rate(gigabytes=4.0, repeats=5):
+    """Bytes per second at which a kernel reads a buffer of `gigabytes` that no cache holds (the
+    fastest of `repeats` passes): what this GPU's memory delivers to a long, plain read."""
+    lib = library("probes")
+    count = int(gigabytes * 1e9) // 16 * 16
+    buffer = torch.zeros(count, dtype=torch.uint8, device="cuda")
+    sink = torch.zeros(1, dtype=torch.float32, device="cuda")
+    best = 0.0
+    for blocks in (2048, 4096, 8192):
+        for _ in range(repeats):
+            begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            begin.record()
+            _check(lib.q3_probe_read(_ptr(buffer), ctypes.c_size_t(count), _ptr(sink), blocks, _stream()), "probe_read")
+            end.record()
+            end.synchronize()
+            best = max(best, count / (begin.elapsed_time(end) * 1e-3))
+    return best
+
+
+def measured_matrix_rate(repeats=5, shape=None, blocks=256 * 8, iters=4096):
+    """Floating-point operations per second of the bfloat16 matrix instructions with their
+    operands in registers, all compute units busy: the better of v_mfma_f32_16x16x32_bf16 and
+    v_mfma_f32_32x32x16_bf16 (`shape` 0 or 1 asks for one of them)."""
+    lib = library("probes")
+    sink = torch.zeros(1, dtype=torch.float32, device="cuda")
+    flops = ctypes.c_double(0.0)
+    best = 0.0
+    for which in ((0, 1) if shape is None else (shape,)):
+        for _ in range(repeats):
+            begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            begin.record()
+            _check(lib.q3_probe_mfma(int(blocks), int(iters), which, _ptr(sink), ctypes.byref(flops), _stream()),
+                   "probe_mfma")
+            end.record()
+            end.synchronize()
+            best = max(best, flops.value / (begin.elapsed_time(end) * 1e-3))
+    return best

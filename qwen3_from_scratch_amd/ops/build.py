@@ -30,7 +30,7 @@ FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
 ]
-MODULES = ("elementwise", "norm", "rotary", "attention", "gemm", "matmul", "sampling")
+MODULES = ("elementwise", "norm", "rotary", "attention", "gemm", "matmul", "sampling", "probes")
 # what a module links besides the HIP runtime
 LINKS = {"matmul": ["-lhipblaslt"]}
 

@@ -41,6 +41,8 @@ class WeightError(ValueError):
 _KEPT = {
     torch.bfloat16: torch.bfloat16,
     torch.float32: torch.float32,
+    torch.float16: torch.float32,      # every float16 number is a float32 number: nothing is rounded here
+    torch.float64: torch.float32,
     torch.int32: torch.int32,
     torch.int64: torch.int32,
     torch.int16: torch.int32,
@@ -50,11 +52,14 @@ _KEPT = {
 
 
 def stored_to_kept(tensor, name="tensor"):
-    """bfloat16 stays bfloat16, a 32-bit float tensor stays so, integer tables
-    become int32; anything else is refused."""
+    """bfloat16 stays bfloat16, a 32-bit float tensor stays so, float16 and
+    float64 tensors become float32 (the reference keeps whatever the file holds,
+    src/qwen3_from_scratch/models/parameter_loader.py:35-41; the parts then bring
+    matrices to the engine's compute dtype, which is bfloat16 or float32), integer
+    tables become int32; anything else (8-bit floats, complex, bool) is refused."""
     if tensor.dtype not in _KEPT:
         raise ValueError(
-            "%s is stored as %s; only bfloat16, float32 and integer tensors are loaded"
+            "%s is stored as %s; only bfloat16, float16, float32, float64 and integer tensors are loaded"
             % (name, tensor.dtype)
         )
     return tensor.to(_KEPT[tensor.dtype])

@@ -33,3 +33,56 @@ def test_yaml_entry(cpu_ops, tmp_path, model_folders, capsys):
     assert len(capsys.readouterr().out.split()) == 3
     with pytest.raises(SystemExit):
         cli.main(["--prompt_ids", "1"])
+
+
+class _WordTokenizer:
+    """A stand-in for a model folder's tokenizer (no network, no files): words are numbers."""
+
+    eos_token_id = 7
+
+    def __init__(self):
+        self.templates = []
+
+    def apply_chat_template(self, messages, tokenize=False, add_generation_prompt=True):
+        assert tokenize is False and add_generation_prompt is True
+        self.templates.append(messages)
+        text = " ".join("%d %s" % (1 if m["role"] == "user" else 2, m["content"]) for m in messages)
+        return text + " 2"                                # the opening of the assistant's turn
+
+    def __call__(self, text):
+        class Encoded:
+            input_ids = [int(t) for t in text.split()]
+        return Encoded()
+
+    def decode(self, ids, skip_special_tokens=True):
+        return "".join("<%d>" % i for i in ids)
+
+
+def test_chat_messages_go_through_the_template(cpu_ops, model_folders, monkeypatch, capsys):
+    """Messages (a list of role/content dicts) are turned into text by the tokenizer's chat
+    template, with the assistant's turn opened, as the reference's engine does
+    (src/qwen3_from_scratch/inference/sync_engine.py:238-251); a string is encoded as it is; the
+    command line's --chat sends its prompts as a user's messages."""
+    from qwen3_from_scratch_amd.engine import SyncEngine, sync_engine
+
+    tokenizer = _WordTokenizer()
+    monkeypatch.setattr(sync_engine, "_load_tokenizer", lambda path: tokenizer)
+    engine = SyncEngine(path=model_folders["A"], dtype="float32", device="cpu", num_blocks=16, max_num_seqs=2)
+    assert 7 in engine.eos_ids
+    request = engine.add_request([{"role": "user", "content": "5 17 3"}])
+    assert request.prompt == [1, 5, 17, 3, 2] and tokenizer.templates == [[{"role": "user", "content": "5 17 3"}]]
+    engine.abort(request)
+    assert engine.add_request("5 17 3").prompt == [5, 17, 3]
+    while engine.scheduler.has_work():
+        engine.step()
+    text = engine.generate([{"role": "user", "content": "9 9"}], 4, temperature=0.0, ignore_eos=True)
+    assert text.count("<") == 4
+    same = engine.generate("1 9 9 2", 4, temperature=0.0, ignore_eos=True)
+    assert same == text
+    capsys.readouterr()
+    args = ["--path", model_folders["A"], "--device", "cpu", "--dtype", "float32", "--num_blocks", "16",
+            "--max_new_tokens", "4", "--temperature", "0", "--ignore_eos", "--prompt", "9 9"]
+    assert cli.main(args + ["--chat"]) == 0
+    assert capsys.readouterr().out.strip() == text
+    assert cli.main(args) == 0
+    assert capsys.readouterr().out.strip() != text

@@ -124,10 +124,34 @@ def test_stored_dtypes_are_kept(model_folders, tmp_path):
     def change16(t):
         t["model.norm.weight"] = t["model.norm.weight"].to(torch.float16)
     folder = _rewrite(model_folders["A"], str(tmp_path / "f16norm"), change16)
-    with pytest.raises(ValueError, match="float16"):
-        Checkpoint(folder).get("model.norm.weight", "cpu")
+    # a float16 tensor is read as float32, which holds every float16 number
+    got = Checkpoint(folder).get("model.norm.weight", "cpu")
+    assert got.dtype == torch.float32
+    assert torch.equal(got, Checkpoint(model_folders["A"]).get("model.norm.weight", "cpu").to(torch.float16).float())
     from qwen3_from_scratch_amd.weights.checkpoint import stored_to_kept
     assert stored_to_kept(torch.arange(4, dtype=torch.int64)).dtype == torch.int32
+    with pytest.raises(ValueError, match="float8"):
+        stored_to_kept(torch.zeros(4).to(torch.float8_e4m3fn), "w")
+
+
+def test_a_float16_checkpoint_loads_and_runs(cpu_ops, model_folders, tmp_path):
+    """All tensors stored in float16 (the reference keeps any stored dtype): the engine reads them
+    as float32, brings them to its compute dtype, and gives the plain implementation's logits
+    for the same file."""
+    import plain_qwen3
+    from helpers import random_tokens
+    from qwen3_from_scratch_amd.engine import StepEntry, load_runner
+
+    def halve(t):
+        for name in list(t):
+            t[name] = t[name].to(torch.float16)
+    folder = _rewrite(model_folders["A"], str(tmp_path / "f16"), halve)
+    cfg, w = plain_qwen3.read_model_folder(folder)
+    toks = random_tokens(20, cfg["vocab_size"], 4)
+    want = plain_qwen3.logits_of_sequence(cfg, w, toks)
+    runner = load_runner(folder, dtype="float32", device="cpu", page_size=16, max_tokens=64, max_requests=1)
+    got = runner.step([StepEntry("a", toks, list(range(20)))])
+    torch.testing.assert_close(got, want, rtol=2e-5, atol=2e-5)
 
 
 def test_random_weights_are_seeded_by_name_not_by_order(model_folders, tmp_path):

@@ -879,3 +879,13 @@ def test_operands_on_the_host_are_refused():
     ops = _ops()
     with pytest.raises(ValueError):
         ops.swiglu(torch.zeros(2, 8))
+
+
+def test_measured_peaks_are_plausible():
+    """The probes behind the benchmark's measured peaks: a read of a buffer no cache holds and the
+    matrix instruction from registers reach a fair share of the published rates and do not pass them."""
+    ops = _ops()
+    read = ops.measured_read_rate(gigabytes=2.0, repeats=3)
+    assert 2.0e12 < read < 8.0e12, read
+    matrix = ops.measured_matrix_rate(repeats=3)
+    assert 1.0e15 < matrix < 2.6e15, matrix

@@ -21,7 +21,13 @@
 // the copies taken out 233 us (1.77 PFLOP/s), with copies that always hit the cache 303, with
 // the copies issued and never waited for 328, as it is 323 (1.27; the matrix pipes are busy 59 %
 // of the cycles, no bank conflicts), the vendor library's best kernel 279. So it is the copies'
-// passage itself, not their latency, that takes the time from the operand reads. Tried and not
+// passage itself, not their latency, that takes the time from the operand reads. The other
+// matrix instruction, v_mfma_f32_32x32x16_bf16, runs at 2.4 PFLOP/s from registers where
+// this kernel's 16 x 16 x 32 runs at 1.4 (one wavefront a SIMD: 2.1 against 0.8), but in this
+// kernel it changed nothing (256 x 256 tiles 417 us beside the library's 312 on a box where the
+// 16 x 16 x 32 form took about 375; no bank conflicts, the matrix pipes busy 39 % of the time):
+// the time goes to the wait for each step's copies with only two stages in flight, not to
+// the multiplications. Tried and not
 // kept: steps of 32 in four stages with the next step's operands read while the current one is
 // multiplied (385); copies through registers and ds_write (365); wavefront tiles of 128 x 128,
 // one wavefront a SIMD (364).

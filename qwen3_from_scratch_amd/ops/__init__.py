@@ -101,8 +101,16 @@ def _matmul():
         _table_loaded = True
         if os.path.isfile(TABLE_FILE):
             with open(TABLE_FILE, encoding="utf-8") as fh:
-                matmul_table(json.load(fh)["entries"])
+                _add_to_table(lib, json.load(fh)["entries"])
     return lib
+
+
+def _add_to_table(lib, entries):
+    for e in entries:
+        out = _DT[getattr(torch, e.get("out", "bfloat16"))]
+        _check(lib.q3_matmul_table_add(_KINDS[e["kind"]], int(e["rows"]), int(e["N"]), int(e["K"]), out,
+                                       int(e.get("library", 0)), int(e.get("own", -1)), int(e.get("splits", 1))),
+               "matmul_table")
 
 
 def matmul_init():
@@ -116,14 +124,10 @@ def matmul_table(entries, clear=False):
     "rows": rounded rows (`matmul_rows_key`), "N", "K", "out": "bfloat16" | "float32",
     "library": the library's candidate number, or "own": tile shape and "splits": shares of K}.
     Sizes without an entry follow the rules of thumb. Sizes already met keep their kernel."""
-    lib = library("matmul")
+    lib = _matmul()                      # the package's own table first, if it is not in yet
     if clear:
         _check(lib.q3_matmul_table_clear(), "matmul_table")
-    for e in entries:
-        out = _DT[getattr(torch, e.get("out", "bfloat16"))]
-        _check(lib.q3_matmul_table_add(_KINDS[e["kind"]], int(e["rows"]), int(e["N"]), int(e["K"]), out,
-                                       int(e.get("library", 0)), int(e.get("own", -1)), int(e.get("splits", 1))),
-               "matmul_table")
+    _add_to_table(lib, entries)
 
 
 def matmul_rows_key(kind, M):

@@ -259,6 +259,8 @@ def main():
                          "prefix: 64 requests that share their first 2,048 tokens, with the prefix index on and off; "
                          "products: a layer's four products by the chosen kernel and by each tile shape of the "
                          "hand-written one")
+    ap.add_argument("--single-copy", action="store_true",
+                    help="hold the matrices once (no tile-ordered copy for steps of few rows): half the weights' memory, slower decoding")
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 points")
     ap.add_argument("--skip-prefill", action="store_true",
                     help="skip the prefill measurement (for profiles of decoding alone; the line then has no value for it)")
@@ -286,7 +288,7 @@ def main():
     torch.cuda.set_device(0)
     if args.workload == "products":
         return products(args, config, shape_name, torch.cuda.synchronize)
-    model = random_model(config, dtype=args.dtype, device="cuda:0", seed=0, std=0.02)
+    model = random_model(config, dtype=args.dtype, device="cuda:0", seed=0, std=0.02, tiled_weights=not args.single_copy)
     gen = torch.Generator().manual_seed(1)
 
     def prompts(n, length):

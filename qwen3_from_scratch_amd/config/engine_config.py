@@ -71,6 +71,9 @@ class EngineConfig:
     use_graphs: bool = True
     # launch a decode step before the previous step's tokens have reached the host
     lookahead: bool = True
+    # keep a second copy of every bfloat16 matrix in the order the few-row product kernel streams it:
+    # decoding is about a fifth faster with it, and the matrices take their memory twice
+    tiled_weights: bool = True
 
     def __post_init__(self):
         self.dtype = parse_dtype(self.dtype)

@@ -40,6 +40,9 @@ def main(argv=None):
     p.add_argument("--chunked_prefill_size", type=int, default=None)
     p.add_argument("--enable_prefix_cache", type=lambda v: str(v).lower() in ("1", "true", "yes", "on"), default=None,
                    metavar="BOOL", help="requests take over cached blocks of a prefix they share (default true)")
+    p.add_argument("--tiled_weights", type=lambda v: str(v).lower() in ("1", "true", "yes", "on"), default=None,
+                   metavar="BOOL", help="keep the second, tile-ordered copy of the matrices (default true: faster "
+                                        "decoding, twice the memory)")
     p.add_argument("--log_interval", type=int, default=0)
     p.add_argument("--write_random", metavar="DIR", help="write a random-weights model folder and exit")
     p.add_argument("--from_config", metavar="JSON", help="config.json for --write_random")
@@ -65,7 +68,8 @@ def main(argv=None):
 
     overrides = {k: getattr(args, k) for k in (
         "dtype", "device", "max_len", "max_num_seqs", "max_num_tokens", "block_size", "num_blocks",
-        "gpu_utilization", "chunked_prefill_size", "enable_prefix_cache") if getattr(args, k) is not None}
+        "gpu_utilization", "chunked_prefill_size", "enable_prefix_cache", "tiled_weights")
+        if getattr(args, k) is not None}
     overrides["seed"] = args.seed
     if args.config_path:
         if not args.model:

@@ -82,7 +82,8 @@ class SyncEngine:
         self.config = config
         self.model_name = model_name or config.name
         self.log_interval = log_interval
-        self.model = model if model is not None else load_model(config.path, config.dtype, config.device)
+        self.model = model if model is not None else load_model(config.path, config.dtype, config.device,
+                                                                 tiled_weights=config.tiled_weights)
         self.tokenizer = _load_tokenizer(config.path) if config.path else None
         mc = self.model.config
         self.max_len = min(config.max_len, mc.max_position_embeddings)

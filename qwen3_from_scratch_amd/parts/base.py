@@ -26,12 +26,12 @@ class Precision:
     tiled: bool = True
 
     @classmethod
-    def named(cls, name):
+    def named(cls, name, tiled=True):
         name = str(name).replace("torch.", "")
         if name in ("bfloat16", "bf16"):
-            return cls(torch.bfloat16)
+            return cls(torch.bfloat16, tiled=bool(tiled))
         if name in ("float32", "fp32"):
-            return cls(torch.float32)
+            return cls(torch.float32, tiled=bool(tiled))
         raise ValueError("dtype must be bfloat16 or float32, found %r" % (name,))
 
     @property

@@ -79,6 +79,21 @@ def test_every_cutting_matches_plain(model_folders, dtype, name, lengths, family
     assert runner.manager.num_free() == runner.manager.num_pages()
 
 
+@pytest.mark.parametrize("name,lengths", [("DS", [33, 1, 150, 64, 300]), ("EP", [129, 300, 70]), ("B", [1, 9, 64, 130])])
+def test_matrices_held_once(model_folders, name, lengths):
+    """Without the tile-ordered copy of the matrices (half the weights' memory) steps of few rows
+    take the row-major product kernels and the norms' own kernels: the same bounds hold."""
+    requests = _requests(name, lengths)
+    want = _plain(model_folders[name], name, requests)
+    steps = trace_mixed(requests)
+    page = TINY[name]["page_size"]
+    runner = load_runner(model_folders[name], dtype="bfloat16", device="cuda", page_size=page,
+                         max_tokens=max_live_tokens(steps, page=page), max_requests=4, tiled_weights=False)
+    assert all(getattr(part, "tiled", None) is None for layer in runner.model.layers
+               for part in (layer.mixer.qkv, layer.mixer.out, layer.feed_forward.gate_up, layer.feed_forward.down))
+    _compare(run_trace(runner, steps), want, "bfloat16")
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding(model_folders, dtype):
     """A short prompt and then hundreds of tokens one by one, across many pages."""

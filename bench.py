@@ -262,6 +262,8 @@ def main():
     ap.add_argument("--single-copy", action="store_true",
                     help="hold the matrices once (no tile-ordered copy for steps of few rows): half the weights' memory, slower decoding")
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 points")
+    ap.add_argument("--no-probes", action="store_true",
+                    help="skip the measurement of this GPU's read and matrix rates (for profiles of the engine alone)")
     ap.add_argument("--skip-prefill", action="store_true",
                     help="skip the prefill measurement (for profiles of decoding alone; the line then has no value for it)")
     args = ap.parse_args()
@@ -366,10 +368,12 @@ def main():
     resident = sum(t.untyped_storage().nbytes() for t in _model_tensors(model))
     # what this GPU delivers, measured here: a plain read of 4 GB, the matrix instruction from registers
     from qwen3_from_scratch_amd import ops
-    read_rate, matrix_rate = ops.measured_read_rate(), ops.measured_matrix_rate()
-    roofline["measured_peak"] = round(read_rate / 1e9, 1)
-    roofline["frac_of_measured"] = round(need / step_s / read_rate, 4)
-    if prefill is not None and args.dtype == "bfloat16":
+    read_rate = matrix_rate = None
+    if not args.no_probes:
+        read_rate, matrix_rate = ops.measured_read_rate(), ops.measured_matrix_rate()
+        roofline["measured_peak"] = round(read_rate / 1e9, 1)
+        roofline["frac_of_measured"] = round(need / step_s / read_rate, 4)
+    if prefill is not None and args.dtype == "bfloat16" and matrix_rate:
         prefill["measured_peak_tflops"] = round(matrix_rate / 1e12, 1)
         prefill["frac_of_measured"] = round(prefill_flops(config, PREFILL) / prefill_s / matrix_rate, 4)
 

@@ -94,6 +94,27 @@ def test_matrices_held_once(model_folders, name, lengths):
     _compare(run_trace(runner, steps), want, "bfloat16")
 
 
+@pytest.mark.parametrize("name,lengths", [("ES", [129, 31, 260]), ("D", [33, 1, 150, 64, 300])])
+def test_two_engines_give_the_same_bits(model_folders, name, lengths):
+    """Nothing on the path is chosen by a stopwatch: two engines built one after the other give
+    bit-equal bfloat16 logits for the same steps (prompt portions of 17 to 128 rows and more,
+    single tokens, graph replays), whatever was run between them."""
+    from qwen3_from_scratch_amd import ops
+
+    requests = _requests(name, lengths)
+    steps = trace_mixed(requests, seed=11)
+    page = TINY[name]["page_size"]
+    kw = dict(dtype="bfloat16", device="cuda", page_size=page, max_tokens=max_live_tokens(steps, page=page),
+              max_requests=4)
+    first = run_trace(load_runner(model_folders[name], **kw), steps)
+    # other sizes and other products in between
+    x = torch.randn(300, 256, device="cuda").to(torch.bfloat16)
+    ops.linear(x, torch.randn(512, 256, device="cuda").to(torch.bfloat16))
+    second = run_trace(load_runner(model_folders[name], **kw), steps)
+    assert first.keys() == second.keys()
+    assert all(torch.equal(first[k], second[k]) for k in first)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding(model_folders, dtype):
     """A short prompt and then hundreds of tokens one by one, across many pages."""

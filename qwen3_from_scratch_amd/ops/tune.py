@@ -32,7 +32,7 @@ def _entry(kind, rows, N, K, out, plan):
     return e
 
 
-def tune_layer(hidden, heads, kv_heads, head_dim, intermediate, rows_list, seed=0, vocab=0):
+def tune_layer(hidden, heads, kv_heads, head_dim, intermediate, rows_list, seed=0, vocab=0, only_head=False):
     device = torch.device("cuda")
     g = torch.Generator(device=device).manual_seed(seed)
 
@@ -44,6 +44,8 @@ def tune_layer(hidden, heads, kv_heads, head_dim, intermediate, rows_list, seed=
         "qkv": rand((qkv_n, hidden), 0.02), "o": rand((hidden, heads * head_dim), 0.02),
         "gate_up": rand((2 * intermediate, hidden), 0.02), "down": rand((hidden, intermediate), 0.02),
     }
+    if only_head:
+        weights = {}
     if vocab:
         weights["head"] = rand((vocab, hidden), 0.02)
     norm_weight = torch.ones(hidden, dtype=torch.bfloat16, device=device)
@@ -55,13 +57,14 @@ def tune_layer(hidden, heads, kv_heads, head_dim, intermediate, rows_list, seed=
             for name, w in weights.items():
                 N, K = w.shape
                 x = rand((M, K))
-                out_dtype = torch.bfloat16
-                ops.linear(x, w)
+                out_dtype = torch.float32 if name == "head" else torch.bfloat16     # logits are float32
+                out_name = "float32" if name == "head" else "bfloat16"
+                ops.linear(x, w, out_dtype=out_dtype)
                 p = ops.matmul_plan(M, N, K, out_dtype)
                 if p is not None:
                     rows = ops.matmul_rows_key("plain", M)
-                    entries[("plain", rows, N, K, "bfloat16")] = _entry(
-                        "plain", rows, N, K, "bfloat16", dict(own=p[4], splits=p[5], library=p[6], us=p[3]))
+                    entries[("plain", rows, N, K, out_name)] = _entry(
+                        "plain", rows, N, K, out_name, dict(own=p[4], splits=p[5], library=p[6], us=p[3]))
                 if name != "head" and 16 < M <= ops.FUSED_ROWS_MOST and ops.fused_rows_take(w, M):
                     residual = torch.zeros((M, N), dtype=torch.float32, device=device)
                     if name in ("o", "down") and N == hidden:
@@ -96,6 +99,7 @@ def main(argv=None):
     ap.add_argument("--intermediate", type=int, required=True)
     ap.add_argument("--vocab", type=int, default=0, help="also the vocabulary product of this many columns")
     ap.add_argument("--rows", default="24,32,48,64,96,128,256,512,1024,2048")
+    ap.add_argument("--only-head", action="store_true", help="the vocabulary product alone")
     ap.add_argument("--merge", default=None, help="an existing table to add to")
     args = ap.parse_args(argv)
     rows = [int(r) for r in args.rows.split(",") if r]
@@ -104,7 +108,7 @@ def main(argv=None):
         with open(args.merge, encoding="utf-8") as fh:
             for e in json.load(fh)["entries"]:
                 entries[(e["kind"], e["rows"], e["N"], e["K"], e.get("out", "bfloat16"))] = e
-    for e in tune_layer(args.hidden, args.heads, args.kv_heads, args.head_dim, args.intermediate, rows, vocab=args.vocab):
+    for e in tune_layer(args.hidden, args.heads, args.kv_heads, args.head_dim, args.intermediate, rows, vocab=args.vocab, only_head=args.only_head):
         entries[(e["kind"], e["rows"], e["N"], e["K"], e["out"])] = e
     ordered = [entries[k] for k in sorted(entries)]
     text = ",\n".join("  " + json.dumps(e, sort_keys=True) for e in ordered)

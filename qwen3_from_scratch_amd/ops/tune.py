@@ -84,6 +84,13 @@ def tune_layer(hidden, heads, kv_heads, head_dim, intermediate, rows_list, seed=
                             rows = ops.matmul_rows_key(kind, M)
                             entries[(kind, rows, N, K, "bfloat16")] = _entry(
                                 kind, rows, N, K, "bfloat16", dict(own=f[0], splits=f[1], library=0))
+                        # where the library serves a product that carries a norm, it is the plain product with
+                        # float32 output (the division follows in a kernel of its own): that size's choice too
+                        p32 = ops.matmul_plan(M, N, K, torch.float32)
+                        if f is not None and f[0] < 0 and kind != "residual" and p32 is not None:
+                            rows = ops.matmul_rows_key("plain", M)
+                            entries[("plain", rows, N, K, "float32")] = _entry(
+                                "plain", rows, N, K, "float32", dict(own=p32[4], splits=p32[5], library=p32[6], us=p32[3]))
             print("rows %d done" % M, file=sys.stderr, flush=True)
     finally:
         ops.matmul_tuner(False)

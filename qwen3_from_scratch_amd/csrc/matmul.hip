@@ -155,10 +155,8 @@ int ready_device(Device& d, hipStream_t stream) {
 
 // The tuner's own: events and the buffer that empties the caches.
 int set_up_tuner(Device& d, hipStream_t stream) {
-  if (!d.begin) {
-    HIP_TRY(hipEventCreate(&d.begin));
-    HIP_TRY(hipEventCreate(&d.end));
-  }
+  if (!d.begin) HIP_TRY(hipEventCreate(&d.begin));
+  if (!d.end) HIP_TRY(hipEventCreate(&d.end));
   if (!d.evict) {
     HIP_TRY(hipMalloc(&d.evict, EVICT_BYTES));
     HIP_TRY(hipMemsetAsync(d.evict, 0, EVICT_BYTES, stream));

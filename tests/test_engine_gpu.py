@@ -79,6 +79,21 @@ def test_every_cutting_matches_plain(model_folders, dtype, name, lengths, family
     assert runner.manager.num_free() == runner.manager.num_pages()
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,lengths,page", [("DS", [33, 1, 150, 64, 300], 64), ("EP", [129, 300, 70], 256),
+                                               ("B", [1, 9, 64, 130], 128)])
+def test_large_pages(model_folders, dtype, name, lengths, page):
+    """Pages of 64 to 256 tokens (a page holds several of the kernels' key tiles): portions and
+    single tokens mixed, with so few pages that they are used again."""
+    requests = _requests(name, lengths)
+    want = _plain(model_folders[name], name, requests)
+    steps = trace_mixed(requests)
+    runner = load_runner(model_folders[name], dtype=dtype, device="cuda", page_size=page,
+                         max_tokens=max_live_tokens(steps, page=page), max_requests=4)
+    _compare(run_trace(runner, steps), want, dtype)
+    assert runner.manager.num_free() == runner.manager.num_pages()
+
+
 @pytest.mark.parametrize("name,lengths", [("DS", [33, 1, 150, 64, 300]), ("EP", [129, 300, 70]), ("B", [1, 9, 64, 130])])
 def test_matrices_held_once(model_folders, name, lengths):
     """Without the tile-ordered copy of the matrices (half the weights' memory) steps of few rows

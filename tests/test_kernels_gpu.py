@@ -176,7 +176,8 @@ def _paged_case(dtype, B, Hq, Hkv, D, page, q_lens, kv_lens, seed, spread=True):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("Hq,Hkv,D,page", [(4, 2, 16, 16), (8, 2, 32, 8), (6, 3, 48, 16), (5, 5, 80, 4),
                                            (32, 8, 128, 16), (3, 1, 256, 32), (16, 2, 64, 16),
-                                           (40, 8, 128, 16), (64, 8, 128, 16), (14, 2, 64, 64), (9, 3, 128, 32)])
+                                           (40, 8, 128, 16), (64, 8, 128, 16), (14, 2, 64, 64), (9, 3, 128, 32),
+                                           (8, 2, 128, 128), (6, 2, 64, 256), (4, 1, 48, 128)])
 @pytest.mark.parametrize("window", [0, 19])
 def test_paged_attention_mixed_batch(dtype, Hq, Hkv, D, page, window):
     ops = _ops()
@@ -191,7 +192,8 @@ def test_paged_attention_mixed_batch(dtype, Hq, Hkv, D, page, window):
     torch.testing.assert_close(got.float(), want, **tol)
 
 
-@pytest.mark.parametrize("Hq,Hkv,D,page", [(32, 8, 128, 16), (8, 1, 64, 32), (3, 3, 128, 64), (16, 1, 128, 16)])
+@pytest.mark.parametrize("Hq,Hkv,D,page", [(32, 8, 128, 16), (8, 1, 64, 32), (3, 3, 128, 64), (16, 1, 128, 16),
+                                           (8, 2, 128, 128), (4, 1, 64, 256)])
 @pytest.mark.parametrize("window", [0, 300])
 def test_paged_attention_decoding_batches(Hq, Hkv, D, page, window):
     """Single tokens over contexts from one key to thousands: one split and many."""
@@ -207,7 +209,7 @@ def test_paged_attention_decoding_batches(Hq, Hkv, D, page, window):
 
 
 @pytest.mark.parametrize("Hq,Hkv,D,page", [(32, 8, 128, 16), (16, 2, 64, 16), (14, 2, 64, 64), (9, 3, 128, 32),
-                                           (16, 1, 128, 16)])
+                                           (16, 1, 128, 16), (8, 2, 128, 128), (6, 2, 64, 256)])
 @pytest.mark.parametrize("w_dtype", [torch.float32, torch.bfloat16, None])
 @pytest.mark.parametrize("window,rotate,store", [(0, True, True), (23, True, True), (0, False, True), (0, True, False)])
 def test_decode_attention_is_its_two_halves(Hq, Hkv, D, page, w_dtype, window, rotate, store):
@@ -260,11 +262,12 @@ def test_decode_attention_is_its_two_halves(Hq, Hkv, D, page, w_dtype, window, r
 
 @pytest.mark.parametrize("q_lens,kv_lens", [([512, 1, 100, 3, 33], [512, 900, 1100, 64, 2000]),
                                             ([700, 2], [3000, 50]), ([300], [9000]), ([40, 40, 40], [2100, 40, 700])])
-def test_paged_attention_portions_over_long_prefixes(q_lens, kv_lens):
+@pytest.mark.parametrize("page", [16, 128])
+def test_paged_attention_portions_over_long_prefixes(q_lens, kv_lens, page):
     """Portions of prompts with hundreds or thousands of cached keys before them, beside single
     tokens: few blocks of rows, whose keys are shared out over four blocks, over two, or not at all."""
     ops = _ops()
-    Hq, Hkv, D, page = 32, 8, 128, 16
+    Hq, Hkv, D = 32, 8, 128
     q, kc, vc, bt, cu, kvl = _paged_case(torch.bfloat16, len(q_lens), Hq, Hkv, D, page, q_lens, kv_lens, 31)
     scale = D ** -0.5
     got = ops.paged_attention(q, Hq, kc, vc, bt, cu, kvl, max(q_lens), max(kv_lens), scale, min_q_len=min(q_lens))

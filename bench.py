@@ -1,7 +1,8 @@
 """Decode and prefill throughput of the Qwen3-8B-shaped model on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L]
-                    [--shape 8b|14b|32b] [--prompt P] [--context C] [--workload decode|continuous|prefix|products]
+                    [--shape 8b|14b|32b|0.6b] [--prompt P] [--context C]
+                    [--workload decode|continuous|served|prefix|products]
 
 Random bfloat16 weights, uniform-random prompts of 2,048 tokens, greedy decoding
 through the engine's own step loop (scheduler, step function, sampling). A
@@ -29,7 +30,12 @@ QWEN3_8B = dict(architectures=["Qwen3ForCausalLM"], vocab_size=151936, hidden_si
                 rope_theta=1000000.0, tie_word_embeddings=False)
 QWEN3_14B = dict(QWEN3_8B, hidden_size=5120, num_hidden_layers=40, num_attention_heads=40, intermediate_size=17408)
 QWEN3_32B = dict(QWEN3_8B, hidden_size=5120, num_hidden_layers=64, num_attention_heads=64, intermediate_size=25600)
-SHAPES = {"8b": ("Qwen3-8B", QWEN3_8B), "14b": ("Qwen3-14B", QWEN3_14B), "32b": ("Qwen3-32B", QWEN3_32B)}
+# the model the reference's own measurements are of, by the sizes its configuration defaults to
+# (src/qwen3_from_scratch/factory/config.py:19-42)
+QWEN3_06B = dict(QWEN3_8B, hidden_size=1024, num_hidden_layers=28, num_attention_heads=16, intermediate_size=4096,
+                 rms_norm_eps=1e-5, rope_theta=100000.0)
+SHAPES = {"8b": ("Qwen3-8B", QWEN3_8B), "14b": ("Qwen3-14B", QWEN3_14B), "32b": ("Qwen3-32B", QWEN3_32B),
+          "0.6b": ("Qwen3-0.6B", QWEN3_06B)}
 PREFILL = 2048
 BLOCK = 16
 
@@ -119,6 +125,65 @@ def continuous(args, config, model, shape_name, gen, sync):
                    "prompt_tokens": tokens_in, "generated_tokens": tokens_out, "prefill_portion": portion,
                    "step_token_budget": portion + requests, "context_len": context, "kv_block_size": BLOCK,
                    "layers": config.num_hidden_layers, "sampling": "greedy"},
+    }))
+    return 0
+
+
+def served(args, config, model, shape_name, gen, sync):
+    """The load of the reference's own benchmark (docs/benchmark.md:40-68, exps/run_eval_scope_bench.sh):
+    200 requests, 20 in flight at any time, 512 prompt tokens and 512 generated tokens each (end-of-sequence
+    ignored), a new request admitted when one ends; without its HTTP server: requests enter and tokens leave
+    through the engine's own loop. Sampling as the engine defaults to (temperature 1.0, as the reference).
+    Run twice; the second run is the one reported."""
+    import torch
+
+    from qwen3_from_scratch_amd.engine import SyncEngine
+    from qwen3_from_scratch_amd.engine.scheduler import RequestStatus
+
+    number, parallel, prompt_tokens, new_tokens = 200, 20, 512, 512
+    context = prompt_tokens + new_tokens
+    engine = SyncEngine(model=model, path="", dtype=args.dtype, device="cuda:0", max_len=context, block_size=BLOCK,
+                        num_blocks=(parallel + 1) * (context // BLOCK + 1), max_num_seqs=parallel,
+                        max_num_tokens=512 + parallel, chunked_prefill_size=512, enable_prefix_cache=False)
+    for _ in range(2):
+        prompts = [torch.randint(0, config.vocab_size, (prompt_tokens,), generator=gen).tolist() for _ in range(number)]
+        admitted, first, ended, live, queued = {}, {}, {}, {}, 0
+        sync()
+        t0 = time.perf_counter()
+        steps = 0
+        while queued < number or live:
+            while queued < number and len(live) < parallel:
+                request = engine.add_request(prompts[queued], engine.default_params(new_tokens, ignore_eos=True))
+                admitted[request.request_id] = time.perf_counter()
+                live[request.request_id] = request
+                queued += 1
+            engine.step()
+            steps += 1
+            now = time.perf_counter()
+            for rid, request in list(live.items()):
+                if request.generated and rid not in first:
+                    first[rid] = now
+                if request.status == RequestStatus.FINISHED:
+                    ended[rid] = now
+                    del live[rid]
+        sync()
+        seconds = time.perf_counter() - t0
+    latency = [ended[r] - admitted[r] for r in ended]
+    ttft = [first[r] - admitted[r] for r in ended]
+    tpot = [(ended[r] - first[r]) / (new_tokens - 1) for r in ended]
+    mean = lambda xs: sum(xs) / len(xs)
+    print(json.dumps({
+        "metric": "output tokens/s, %d requests, %d in flight, %d in + %d out, %s %s"
+                  % (number, parallel, prompt_tokens, new_tokens, shape_name,
+                     "bf16" if args.dtype == "bfloat16" else "fp32"),
+        "value": round(number * new_tokens / seconds, 1), "unit": "tokens/s", "n_gpus": 1, "higher_is_better": True,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic", "seconds": round(seconds, 3),
+        "steps": steps, "requests_per_s": round(number / seconds, 2), "latency_avg_s": round(mean(latency), 3),
+        "ttft_avg_ms": round(1e3 * mean(ttft), 1), "tpot_avg_ms": round(1e3 * mean(tpot), 2),
+        "config": {"model": "%s-shaped, random weights N(0, 0.02)" % shape_name, "requests": number,
+                   "in_flight": parallel, "prompt_tokens": prompt_tokens, "generated_tokens": new_tokens,
+                   "prefill_portion": 512, "kv_block_size": BLOCK, "layers": config.num_hidden_layers,
+                   "sampling": "temperature 1.0", "server": "none: the engine's own loop"},
     }))
     return 0
 
@@ -253,7 +318,7 @@ def main():
     ap.add_argument("--shape", default="8b", choices=sorted(SHAPES))
     ap.add_argument("--prompt", type=int, default=2048, help="tokens every request holds when decoding starts")
     ap.add_argument("--context", type=int, default=8192, help="tokens of cache per request")
-    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "prefix", "products"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "served", "prefix", "products"],
                     help="continuous: 64 requests at once, prompts of 128 to 4,096 tokens, 64 to 512 generated "
                          "tokens each, prompts in portions of 512 (its own JSON line; --steps and --warmup unused); "
                          "prefix: 64 requests that share their first 2,048 tokens, with the prefix index on and off; "
@@ -308,6 +373,8 @@ def main():
 
     if args.workload == "continuous":
         return continuous(args, config, model, shape_name, gen, sync)
+    if args.workload == "served":
+        return served(args, config, model, shape_name, gen, sync)
     if args.workload == "prefix":
         return shared_prefix(args, config, model, shape_name, gen, sync)
 

@@ -148,6 +148,7 @@ struct SkinnyFusion {
   const void* norm_weight;
   int norm_weight_f32;
   float* sums_out;
+  int sums_stride;   // floats between two partial sums of a row, in row_sums and in sums_out: 16 or more, in steps of 4
 };
 
 #ifndef SKINNY_PAIR_SLABS
@@ -155,7 +156,7 @@ struct SkinnyFusion {
 #endif
 #define SKINNY_PRE 4  // float4 loads of partial sums a thread has in flight beside the main loop's
 
-template <typename OUT, int EPI, bool TILED, bool SCALED>
+template <typename OUT, int EPI, bool TILED, bool SCALED, bool GROUPS>
 __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restrict__ x,
                                                            const bf16_t* __restrict__ w, OUT* __restrict__ out,
                                                            int M, int N, int K, int kw, int k_per_wave,
@@ -165,6 +166,24 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
   const int col = lane & 15, grp = lane >> 4;
   const int nwaves = blockDim.x >> 6;
   const int sw = nwaves / kw;
+  // With GROUPS (more than 16 rows of x, for weights small enough to be read once per 16 rows): rows
+  // 16 y .. 16 y + 15 of x, and of everything that has a row per row of x, belong to the blocks with
+  // blockIdx.y = y, and a row's partial sums are fu.sums_stride floats apart. Without, the kernel is the
+  // one for up to 16 rows, partial sums 16 floats apart.
+  const int row0 = GROUPS ? 16 * (int)blockIdx.y : 0;
+  const int sums_stride = GROUPS ? fu.sums_stride : 16;
+  auto sums_at = [&](int i, int q) {   // rows 4 q .. 4 q + 3 of this group in partial sum i
+    if constexpr (GROUPS)
+      return reinterpret_cast<const float4*>(fu.row_sums + (size_t)i * sums_stride + row0)[q];
+    else
+      return reinterpret_cast<const float4*>(fu.row_sums)[i * 4 + q];
+  };
+  if constexpr (GROUPS) {
+    M = min(16, M - row0);
+    x += (size_t)row0 * K;
+    out += (size_t)row0 * (EPI == EPI_SWIGLU ? N / 2 : N);
+    if (EPI == EPI_RESIDUAL) fu.residual += (size_t)row0 * N;
+  }
   const int slab = blockIdx.x * sw + wave / kw;
   const int ksplit = wave % kw;
   const int n0 = slab * 16;
@@ -180,7 +199,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
 #pragma unroll
     for (int u = 0; u < SKINNY_PRE; ++u) {
       const int i = i0 + u * stride;
-      pre[u] = i < fu.sums_rows ? reinterpret_cast<const float4*>(fu.row_sums)[i * 4 + q] : make_float4(0.f, 0.f, 0.f, 0.f);
+      pre[u] = i < fu.sums_rows ? sums_at(i, q) : make_float4(0.f, 0.f, 0.f, 0.f);
     }
   }
   // the residual and the norm's weights of this lane's four outputs, asked for before the products
@@ -230,7 +249,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
     }
     const int q = threadIdx.x & 3, stride = blockDim.x >> 2;
     for (int i = (threadIdx.x >> 2) + SKINNY_PRE * stride; i < fu.sums_rows; i += stride) {
-      const float4 v = reinterpret_cast<const float4*>(fu.row_sums)[i * 4 + q];
+      const float4 v = sums_at(i, q);
       s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
     }
 #pragma unroll
@@ -279,7 +298,11 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16_t* __restr
     }
     ss += __shfl_xor(ss, 16, 64);
     ss += __shfl_xor(ss, 32, 64);
-    if (grp == 0 && n0 < N) fu.sums_out[slab * 16 + col] = ss;
+    if constexpr (GROUPS) {
+      if (grp == 0 && n0 < N) fu.sums_out[(size_t)slab * sums_stride + row0 + col] = ss;
+    } else {
+      if (grp == 0 && n0 < N) fu.sums_out[slab * 16 + col] = ss;
+    }
     return;
   }
   if (col >= M) return;
@@ -470,8 +493,9 @@ static int launch_skinny(const void* x, const void* w, void* out, int M, int N, 
   const int step = 32 * SKINNY_U;
   int k_per_wave = (K + kw - 1) / kw;
   k_per_wave = (k_per_wave + step - 1) / step * step;
+  const int groups = (M + 15) / 16;   // of 16 rows of x: one, or a few for a small weight (q3_linear_tiled)
   if constexpr (TILED && (EPI == EPI_PLAIN || EPI == EPI_SWIGLU)) {
-    if (slabs >= SKINNY_PAIR_SLABS && sw == 1 && M > 8) {
+    if (slabs >= SKINNY_PAIR_SLABS && sw == 1 && M > 8 && groups == 1) {
       const size_t pair_smem = (size_t)kw * (2 * 64 * 4 + 16) * sizeof(float);
       hipLaunchKernelGGL((gemm_skinny_pair_kernel<OUT, EPI, SCALED>), dim3((slabs + 1) / 2), dim3(64 * kw), pair_smem,
                          stream, (const bf16_t*)x, (const bf16_t*)w, (OUT*)out, M, N, K, kw, k_per_wave, fu);
@@ -480,8 +504,16 @@ static int launch_skinny(const void* x, const void* w, void* out, int M, int N, 
   }
   const int blocks = (slabs + sw - 1) / sw;
   const size_t smem = (size_t)sw * kw * (64 * 4 + 16) * sizeof(float);
-  hipLaunchKernelGGL((gemm_skinny_kernel<OUT, EPI, TILED, SCALED>), dim3(blocks), dim3(64 * sw * kw), smem, stream,
-                     (const bf16_t*)x, (const bf16_t*)w, (OUT*)out, M, N, K, kw, k_per_wave, fu);
+  if (groups > 1) {
+    if constexpr (TILED)
+      hipLaunchKernelGGL((gemm_skinny_kernel<OUT, EPI, TILED, SCALED, true>), dim3(blocks, groups), dim3(64 * sw * kw), smem,
+                         stream, (const bf16_t*)x, (const bf16_t*)w, (OUT*)out, M, N, K, kw, k_per_wave, fu);
+    else
+      return Q3_ERR_BAD_ARGUMENT;
+  } else {
+    hipLaunchKernelGGL((gemm_skinny_kernel<OUT, EPI, TILED, SCALED, false>), dim3(blocks), dim3(64 * sw * kw), smem, stream,
+                       (const bf16_t*)x, (const bf16_t*)w, (OUT*)out, M, N, K, kw, k_per_wave, fu);
+  }
   return q3_launch_status();
 }
 
@@ -595,18 +627,29 @@ extern "C" int q3_linear_swiglu(const void* x, const void* weight, void* out, in
 }
 
 // The same products from the tile-ordered copy of the weight (see gemm_skinny_kernel):
-// x (M, K) bfloat16, M <= 16, K a multiple of 32. `epilogue`: 0 output (M, N) in `out_dtype`;
+// x (M, K) bfloat16, K a multiple of 32. `epilogue`: 0 output (M, N) in `out_dtype`;
 // 1 the activation (output (M, N / 2) bfloat16); 2 the residual addition and the next norm's
 // preparation (N a multiple of 16; `residual` (M, N) float32 updated in place, `norm_weight`
 // (N,) of `norm_w_dtype`, output (M, N) bfloat16 = residual * norm_weight, `sums_out`
-// (N / 16, 16) float32). `row_sums` (sums_rows, 16) float32, if not null, says that x's rows
-// still lack the factor rsqrt(sum / width + eps), which the product's rows then receive.
+// (N / 16, sums_stride) float32). `row_sums` (sums_rows, sums_stride) float32, if not null, says that
+// x's rows still lack the factor rsqrt(sum / width + eps), which the product's rows then receive.
+// `sums_stride`: floats between two partial sums of one row: 16 for up to 16 rows, else a multiple of 4 and at
+// least M rounded up to 16.
+// M <= 16, or up to Q3_SKINNY_MAX_ROWS for a weight small enough that reading it once per 16 rows costs
+// less than a kernel more (the caller's rule; every group of 16 rows is a set of blocks of its own).
+#define Q3_SKINNY_MAX_ROWS 64
+extern "C" int q3_linear_tiled_max_rows() { return Q3_SKINNY_MAX_ROWS; }
+
 extern "C" int q3_linear_tiled(const void* x, const void* weight_tiled, void* out, int M, int N, int K,
                                int out_dtype, int epilogue, const float* row_sums, int sums_rows, float eps,
                                int width, float* residual, const void* norm_weight, int norm_w_dtype,
-                               float* sums_out, hipStream_t stream) {
-  if (M <= 0 || M > 16 || N <= 0 || K <= 0 || K % 32) return Q3_ERR_BAD_ARGUMENT;
+                               float* sums_out, int sums_stride, hipStream_t stream) {
+  if (M <= 0 || M > Q3_SKINNY_MAX_ROWS || N <= 0 || K <= 0 || K % 32) return Q3_ERR_BAD_ARGUMENT;
   SkinnyFusion fu{};
+  if (row_sums || sums_out) {
+    if (sums_stride % 4 || sums_stride < (M + 15) / 16 * 16 || (M <= 16 && sums_stride != 16)) return Q3_ERR_BAD_ARGUMENT;
+    fu.sums_stride = sums_stride;
+  }
   if (row_sums) {
     if (sums_rows <= 0 || width <= 0) return Q3_ERR_BAD_ARGUMENT;
     fu.row_sums = row_sums;

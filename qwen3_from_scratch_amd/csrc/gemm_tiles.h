@@ -91,8 +91,9 @@ __device__ inline uint2 pack_bf16x4(f32x4_t c) {
 
 // The rows of x may still lack the factor of the norm before this product: they hold
 // stream * norm_weight, and `sums` (chunks, rows) holds the rows' sums of squares of the stream in
-// partial sums of column chunks (tiles_residual_kernel leaves them so). Row m of the product is
-// then multiplied by rsqrt(sum_m * inv_width + eps): (x / rms) @ W^T = (x @ W^T) / rms.
+// partial sums of column chunks (tiles_residual_kernel and the few-row kernel of gemm.hip leave them
+// so; `rows` is the distance between two partial sums of one row, the number of rows or more). Row m
+// of the product is then multiplied by rsqrt(sum_m * inv_width + eps): (x / rms) @ W^T = (x @ W^T) / rms.
 struct RowScale {
   const float* sums = nullptr;
   int chunks = 0, rows = 0;
@@ -323,15 +324,16 @@ __global__ __launch_bounds__(256) void gemm_tiles_reduce_kernel(const float* __r
 // The product as a residual stream's next addend, with the next norm prepared: the sum of the
 // partial products is rounded to bfloat16 (what a separate addition would have read), added
 // into `residual` (M, N) float32 in place, (residual * norm_weight) goes to `values` as
-// bfloat16, and the row's sum of squares over this block's 1,024 columns to sums[chunk][row].
-// Grid (chunks of 1,024 columns, rows), 256 threads, four columns a thread; N a multiple of 4.
+// bfloat16, and the row's sum of squares over this block's 1,024 columns to sums[chunk][row]
+// (`sums_stride` floats a chunk). Grid (chunks of 1,024 columns, rows), 256 threads, four columns a
+// thread; N a multiple of 4.
 constexpr int CHUNK_COLUMNS = 1024;
 template <typename NW>
 __global__ __launch_bounds__(256) void tiles_residual_kernel(const float* __restrict__ partials, int splits,
                                                              float* __restrict__ residual,
                                                              const NW* __restrict__ norm_weight,
                                                              bf16_t* __restrict__ values, float* __restrict__ sums,
-                                                             int M, int N) {
+                                                             int sums_stride, int M, int N) {
   __shared__ float scratch[17];
   const int m = blockIdx.y, n = blockIdx.x * CHUNK_COLUMNS + 4 * threadIdx.x;
   float ss = 0.f;
@@ -354,7 +356,7 @@ __global__ __launch_bounds__(256) void tiles_residual_kernel(const float* __rest
     ss = r.x * r.x + r.y * r.y + r.z * r.z + r.w * r.w;
   }
   const float total = block_sum(ss, scratch);
-  if (threadIdx.x == 0) sums[(size_t)blockIdx.x * M + m] = total;
+  if (threadIdx.x == 0) sums[(size_t)blockIdx.x * sums_stride + m] = total;
 }
 
 // The tile shapes on offer: (BM, BN, STAGES).

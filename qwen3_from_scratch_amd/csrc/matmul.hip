@@ -532,13 +532,15 @@ extern "C" int q3_matmul_init() {
 // here). x (M, K) and w (N, K) bfloat16, K a multiple of 64, N of 4.
 //
 // q3_tiles_scaled: the rows of x hold stream * norm_weight and still lack the norm's division; `sums`
-// (chunks, M) float32 holds the rows' sums of squares of the stream in partial sums, `width` the stream's
-// width (= K). out = (x @ w^T) * rsqrt(sum / width + eps) row by row: epilogue 0 gives (M, N) in `out_dtype`,
-// 1 (rows of w interleave gate and up) gives (M, N / 2) bfloat16 = silu(gate) * up.
+// (chunks, sums_stride) float32 holds the rows' sums of squares of the stream in partial sums (row m in
+// column m, sums_stride >= M), `width` the stream's width (= K). out = (x @ w^T) * rsqrt(sum / width + eps)
+// row by row: epilogue 0 gives (M, N) in `out_dtype`, 1 (rows of w interleave gate and up) gives (M, N / 2)
+// bfloat16 = silu(gate) * up.
 extern "C" int q3_tiles_scaled(const void* x, const void* w, void* out, int M, int N, int K, int out_dtype,
-                               int epilogue, const float* sums, int chunks, float eps, int width, void* stream_) {
+                               int epilogue, const float* sums, int chunks, int sums_stride, float eps, int width,
+                               void* stream_) {
   if (!x || !w || !out || !sums || M < 1 || M > 256 || N % 4 || !tiles::takes(M, N, K)) return Q3_ERR_BAD_ARGUMENT;
-  if (chunks < 1 || width != K) return Q3_ERR_BAD_ARGUMENT;
+  if (chunks < 1 || sums_stride < M || width != K) return Q3_ERR_BAD_ARGUMENT;
   const bool swiglu = epilogue == tiles::EPI_SWIGLU;
   if (!swiglu && epilogue != tiles::EPI_PLAIN) return Q3_ERR_BAD_ARGUMENT;
   if (swiglu ? out_dtype != Q3_BF16 : (out_dtype != Q3_BF16 && out_dtype != Q3_F32)) return Q3_ERR_BAD_ARGUMENT;
@@ -552,7 +554,7 @@ extern "C" int q3_tiles_scaled(const void* x, const void* w, void* out, int M, i
   tiles::RowScale scale;
   scale.sums = sums;
   scale.chunks = chunks;
-  scale.rows = M;
+  scale.rows = sums_stride;
   scale.eps = eps;
   scale.inv_width = 1.f / (float)width;
   auto launch = [&](int config, int splits) {
@@ -597,15 +599,15 @@ extern "C" int q3_tiles_scaled(const void* x, const void* w, void* out, int M, i
 }
 
 // q3_tiles_residual: residual (M, N) float32 += bfloat16(x @ w^T) in place; values (M, N) bfloat16 =
-// residual * norm_weight; sums (ceil(N / 1024), M) float32 = the rows' sums of squares of the new residual over
-// chunks of 1,024 columns: what q3_tiles_scaled takes for the next product. Returns Q3_DECLINED, and has done
+// residual * norm_weight; sums (ceil(N / 1024), sums_stride) float32 = the rows' sums of squares of the new
+// residual over chunks of 1,024 columns (row m in column m): what q3_tiles_scaled takes for the next product. Returns Q3_DECLINED, and has done
 // nothing, where the plain product followed by the norm's own kernel is the way for this size.
 extern "C" int q3_tiles_residual_chunks(int N) { return (N + tiles::CHUNK_COLUMNS - 1) / tiles::CHUNK_COLUMNS; }
 
 extern "C" int q3_tiles_residual(const void* x, const void* w, int M, int N, int K, float* residual,
                                  const void* norm_weight, int norm_weight_dtype, void* values, float* sums,
-                                 void* stream_) {
-  if (!x || !w || !residual || !norm_weight || !values || !sums) return Q3_ERR_BAD_ARGUMENT;
+                                 int sums_stride, void* stream_) {
+  if (!x || !w || !residual || !norm_weight || !values || !sums || sums_stride < M) return Q3_ERR_BAD_ARGUMENT;
   if (M < 1 || M > 256 || N % 4 || !tiles::takes(M, N, K)) return Q3_ERR_BAD_ARGUMENT;
   if (norm_weight_dtype != Q3_BF16 && norm_weight_dtype != Q3_F32) return Q3_ERR_BAD_ARGUMENT;
   hipStream_t stream = (hipStream_t)stream_;
@@ -636,10 +638,10 @@ extern "C" int q3_tiles_residual(const void* x, const void* w, int M, int N, int
   const dim3 grid(q3_tiles_residual_chunks(N), M);
   if (norm_weight_dtype == Q3_F32)
     hipLaunchKernelGGL(tiles::tiles_residual_kernel<float>, grid, dim3(256), 0, stream, d.partials, used, residual,
-                       (const float*)norm_weight, (bf16_t*)values, sums, M, N);
+                       (const float*)norm_weight, (bf16_t*)values, sums, sums_stride, M, N);
   else
     hipLaunchKernelGGL(tiles::tiles_residual_kernel<bf16_t>, grid, dim3(256), 0, stream, d.partials, used, residual,
-                       (const bf16_t*)norm_weight, (bf16_t*)values, sums, M, N);
+                       (const bf16_t*)norm_weight, (bf16_t*)values, sums, sums_stride, M, N);
   return q3_launch_status();
 }
 

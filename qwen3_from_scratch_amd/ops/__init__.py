@@ -504,8 +504,30 @@ def tile_weight(weight):
     return tiles.contiguous().view(-1)
 
 
+FEW_ROWS = 16                   # the few-row kernel's rows: one matrix instruction's worth of x
+SMALL_WEIGHT_BYTES = 18 << 20   # up to this size the few-row kernel serves 32 rows, up to half of it 64
+
+
+def few_rows_limit(weight):
+    """Up to how many rows of x the few-row kernel serves a product with `weight` from its tiled
+    copy: 16, or 32 or 64 for a small weight. The kernel works on 16 rows of x at a time; more
+    rows are further sets of blocks that read the weight again. For a small weight that reading
+    comes out of the caches and costs less than what the tiled kernel needs beyond 16 rows, a
+    second kernel that adds its shares of K. Measured inside a graph, the product with its norm's
+    work, few-row kernel against tiled kernel, in microseconds: 8 MB (4,096 x 1,024) at 24, 32, 48
+    and 64 rows 5.8, 6.1, 8.4, 9.6 against 9.2, 9.6, 10.1, 10.9; 17 MB at 24, 32 and 48 rows 8.1,
+    8.8, 11.9 against 9.9, 10.3, 11.5; 50 MB at 24 rows 20.0 against 15.0."""
+    size = weight.numel() * weight.element_size()
+    return FEW_ROWS * (4 if 2 * size <= SMALL_WEIGHT_BYTES else 2 if size <= SMALL_WEIGHT_BYTES else 1)
+
+
+def sums_stride(M):
+    """Columns of a tensor of rows' partial sums of squares for M rows (see `linear_residual_norm`)."""
+    return -(-M // 16) * 16
+
+
 def _tiled_ok(tiled, weight, M):
-    if tiled is None or not 1 <= M <= 16:
+    if tiled is None or not 1 <= M <= few_rows_limit(weight):
         return False
     N, K = weight.shape
     _need(tiled.is_cuda and tiled.dtype == torch.bfloat16 and tiled.is_contiguous()
@@ -514,26 +536,31 @@ def _tiled_ok(tiled, weight, M):
     return True
 
 
-def _row_sums_args(unscaled, M, K):
-    """The kernel's arguments for rows that still lack their 1 / rms factor:
-    `unscaled` = (sums (P, 16) float32, eps, width) as `linear_residual_norm` leaves them."""
-    if unscaled is None:
-        return None, 0, ctypes.c_float(0.0), 0
-    sums, eps, width = unscaled
+def _check_sums(sums, M):
     _dev(sums)
-    _need(sums.dtype == torch.float32 and sums.dim() == 2 and sums.shape[1] == 16 and sums.shape[0] > 0
-          and sums.is_contiguous(), "row sums must be float32 (P, 16)")
+    _need(sums.dtype == torch.float32 and sums.dim() == 2 and sums.shape[1] == sums_stride(M) and sums.shape[0] > 0
+          and sums.is_contiguous(), "row sums must be float32 (P, M rounded up to 16)")
+
+
+def _row_sums_args(unscaled, M, K):
+    """The few-row kernel's arguments for rows that still lack their 1 / rms factor: `unscaled` =
+    (sums (P, M rounded up to 16) float32, eps, width) as `linear_residual_norm` leaves them."""
+    if unscaled is None:
+        return None, 0, ctypes.c_float(0.0), 0, 0
+    sums, eps, width = unscaled
+    _check_sums(sums, M)
     _need(width == K, "the rows' width must be the product's inner size")
-    return _ptr(sums), sums.shape[0], ctypes.c_float(eps), int(width)
+    return _ptr(sums), sums.shape[0], ctypes.c_float(eps), int(width), sums.shape[1]
 
 
-FUSED_ROWS_FEW, FUSED_ROWS_MOST = 16, 128
+FUSED_ROWS_FEW, FUSED_ROWS_MOST = FEW_ROWS, 128
 
 
 def fused_rows_take(weight, M):
     """Whether the tiled kernel carries a norm for `M` rows of a product with `weight` (N, K):
-    more rows than the few-row kernel takes, at most 128 (beyond that the vendor library's products with the norms as kernels of
-    their own are faster), bfloat16, K a multiple of 64 and N of 4."""
+    more than 16 rows, at most 128 (beyond that the vendor library's products with the norms as
+    kernels of their own are faster), bfloat16, K a multiple of 64 and N of 4. (Where the few-row
+    kernel takes the rows too, a small weight's 17 to 32 or 64, that one is used.)"""
     return (FUSED_ROWS_FEW < M <= FUSED_ROWS_MOST and weight.dtype == torch.bfloat16 and weight.dim() == 2
             and weight.shape[1] % 64 == 0 and weight.shape[0] % 4 == 0 and weight.is_contiguous())
 
@@ -541,14 +568,12 @@ def fused_rows_take(weight, M):
 def _tiles_scaled(x, weight, out, unscaled, swiglu, what):
     sums, eps, width = unscaled
     M, K = x.shape
-    _dev(sums)
-    _need(sums.dtype == torch.float32 and sums.dim() == 2 and sums.shape[1] == M and sums.shape[0] > 0
-          and sums.is_contiguous(), "row sums must be float32 (chunks, M)")
+    _check_sums(sums, M)
     _need(width == K, "the rows' width must be the product's inner size")
     _need(x.is_contiguous() and out.is_contiguous(), "operands must be contiguous")
     _check(_matmul().q3_tiles_scaled(
         _ptr(x), _ptr(weight), _ptr(out), M, weight.shape[0], K, _DT[out.dtype], 1 if swiglu else 0, _ptr(sums),
-        sums.shape[0], ctypes.c_float(eps), int(width), _stream()), what)
+        sums.shape[0], sums.shape[1], ctypes.c_float(eps), int(width), _stream()), what)
     return out
 
 
@@ -574,10 +599,10 @@ def linear(x, weight, out_dtype=None, out=None, tiled=None, unscaled=None):
         out = torch.empty((M, N), dtype=out_dtype, device=x.device)
     _need(out.shape == (M, N) and out.dtype == out_dtype, "out must be (M, N) of out_dtype")
     if M and x.dtype == torch.bfloat16 and _tiled_ok(tiled, weight, M):
-        sums, sums_rows, eps, width = _row_sums_args(unscaled, M, K)
+        sums, sums_rows, eps, width, stride = _row_sums_args(unscaled, M, K)
         _check(library("gemm").q3_linear_tiled(
             _ptr(x), _ptr(tiled), _ptr(out), M, N, K, _DT[out_dtype], 0, sums, sums_rows, eps, width,
-            None, None, 0, None, _stream()), "linear")
+            None, None, 0, None, stride, _stream()), "linear")
         return out
     if unscaled is not None and x.dtype == torch.bfloat16 and fused_rows_take(weight, M):
         return _tiles_scaled(x, weight, out, unscaled, False, "linear")
@@ -635,10 +660,10 @@ def linear_swiglu(x, weight, tiled=None, unscaled=None):
     N = weight.shape[0]
     if M and x.dtype == torch.bfloat16 and _tiled_ok(tiled, weight, M):
         out = torch.empty((M, N // 2), dtype=x.dtype, device=x.device)
-        sums, sums_rows, eps, width = _row_sums_args(unscaled, M, K)
+        sums, sums_rows, eps, width, stride = _row_sums_args(unscaled, M, K)
         _check(library("gemm").q3_linear_tiled(
             _ptr(x), _ptr(tiled), _ptr(out), M, N, K, 1, 1, sums, sums_rows, eps, width,
-            None, None, 0, None, _stream()), "linear_swiglu")
+            None, None, 0, None, stride, _stream()), "linear_swiglu")
         return out
     if unscaled is not None and x.dtype == torch.bfloat16 and fused_rows_take(weight, M):
         out = torch.empty((M, N // 2), dtype=x.dtype, device=x.device)
@@ -656,20 +681,20 @@ def linear_swiglu(x, weight, tiled=None, unscaled=None):
 def linear_residual_norm(x, weight, tiled, residual, norm_weight):
     """residual += x @ weight^T, and the next norm's input prepared in the same kernel.
 
-    x (M, K) bfloat16 with M <= 16, weight (N, K) with its tiled copy, N a multiple of 16;
-    residual (M, N) float32 is updated in place (the product is rounded to bfloat16 before the
-    addition, as a product written out and added by the norm kernel would be). Returns
-    (values, sums): values (M, N) bfloat16 = residual * norm_weight, and sums (N / 16, 16)
-    float32, the rows' sums of squares of the new residual in partial sums of 16 columns (row m
-    of the stream in column m). The norm's result is values * rsqrt(sum / N + eps) row by row;
-    `linear` and `linear_swiglu` apply that factor to their products when given
-    `unscaled=(sums, eps, N)`.
+    x (M, K) bfloat16, weight (N, K); residual (M, N) float32 is updated in place (the product
+    is rounded to bfloat16 before the addition, as a product written out and added by the norm
+    kernel would be). Returns (values, sums): values (M, N) bfloat16 = residual * norm_weight,
+    and sums (P, M rounded up to 16) float32, the rows' sums of squares of the new residual in P
+    partial sums (row m of the stream in column m). The norm's result is
+    values * rsqrt(sum / N + eps) row by row; `linear` and `linear_swiglu` apply that factor to
+    their products when given `unscaled=(sums, eps, N)`.
 
-    With 17 to 128 rows (`fused_rows_take`; `tiled` is not used) the tiled kernel's partial
-    products are added by a second kernel that does the same; sums is then (ceil(N / 1024), M),
-    partial sums over 1,024 columns, row m of the stream in column m. There the result is None,
-    and nothing was done, for a size at which timing found the plain product (`linear`) followed
-    by the norm's own kernel faster."""
+    Up to `few_rows_limit(weight)` rows, with the weight's tiled copy and N a multiple of 16, it
+    is the few-row kernel's epilogue (P = N / 16, partial sums of 16 columns). With more rows, up
+    to 128 (`fused_rows_take`; `tiled` is not used), the tiled kernel's partial products are added
+    by a second kernel that does the same (P = ceil(N / 1024)). There the result is None, and
+    nothing was done, for a size at which the plain product (`linear`) followed by the norm's own
+    kernel is the faster way."""
     _dev(x, weight, tiled, residual, norm_weight)
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1], "x (M, K) and weight (N, K)")
     M, K = x.shape
@@ -678,23 +703,25 @@ def linear_residual_norm(x, weight, tiled, residual, norm_weight):
           "residual must be float32 (M, N)")
     _need(norm_weight.shape == (N,) and norm_weight.dtype in _DT and norm_weight.is_contiguous(), "norm weight (N,)")
     values = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
-    if x.dtype == torch.bfloat16 and fused_rows_take(weight, M):
+    few = x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and N % 16 == 0 and _tiled_ok(tiled, weight, M)
+    if not few and x.dtype == torch.bfloat16 and fused_rows_take(weight, M):
         _need(x.is_contiguous(), "x must be contiguous")
         lib = _matmul()
-        sums = torch.empty((lib.q3_tiles_residual_chunks(N), M), dtype=torch.float32, device=x.device)
+        sums = torch.empty((lib.q3_tiles_residual_chunks(N), sums_stride(M)), dtype=torch.float32, device=x.device)
         status = lib.q3_tiles_residual(
             _ptr(x), _ptr(weight), M, N, K, _ptr(residual), _ptr(norm_weight), _DT[norm_weight.dtype], _ptr(values),
-            _ptr(sums), _stream())
+            _ptr(sums), sums.shape[1], _stream())
         if status == _DECLINED:
             return None
         _check(status, "linear_residual_norm")
         return values, sums
-    _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and _tiled_ok(tiled, weight, M) and N % 16 == 0,
-          "bfloat16, 1 to 16 rows, a tiled weight and a width that is a multiple of 16")
-    sums = torch.empty((N // 16, 16), dtype=torch.float32, device=x.device)
+    _need(few, "bfloat16, a tiled weight with a width that is a multiple of 16 and no more rows than few_rows_limit, "
+          "or 17 to 128 rows with an inner size that is a multiple of 64")
+    sums = torch.empty((N // 16, sums_stride(M)), dtype=torch.float32, device=x.device)
     _check(library("gemm").q3_linear_tiled(
         _ptr(x), _ptr(tiled), _ptr(values), M, N, K, 1, 2, None, 0, ctypes.c_float(0.0), 0,
-        _ptr(residual), _ptr(norm_weight), _DT[norm_weight.dtype], _ptr(sums), _stream()), "linear_residual_norm")
+        _ptr(residual), _ptr(norm_weight), _DT[norm_weight.dtype], _ptr(sums), sums.shape[1], _stream()),
+        "linear_residual_norm")
     return values, sums
 
 

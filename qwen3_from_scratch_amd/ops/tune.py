@@ -71,7 +71,7 @@ def tune_layer(hidden, heads, kv_heads, head_dim, intermediate, rows_list, seed=
                         ops.linear_residual_norm(x, w, None, residual, norm_weight)
                         kinds = ["residual"]
                     else:
-                        sums = torch.ones((-(-K // 1024), M), dtype=torch.float32, device=device)
+                        sums = torch.ones((-(-K // 1024), ops.sums_stride(M)), dtype=torch.float32, device=device)
                         if name == "gate_up":
                             ops.linear_swiglu(x, w, unscaled=(sums, 1e-6, K))
                             kinds = ["scaled_swiglu"]

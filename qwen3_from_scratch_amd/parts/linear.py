@@ -35,8 +35,9 @@ class LinearWeight:
     @property
     def fuses(self):
         """Whether steps of few rows go through kernels whose epilogues carry the
-        norm fusion, UnscaledRows in, a NormSink out: up to 16 rows the few-row
-        kernel on the tiled copy, up to 128 the tiled matrix-core kernel. A
+        norm fusion, UnscaledRows in, a NormSink out: up to 16 rows (32 or 64 for a
+        small weight) the few-row kernel on the tiled copy, up to 128 the tiled
+        matrix-core kernel. A
         reader of UnscaledRows must have output rows in steps of 4."""
         return self.tiled is not None and self.weight.shape[0] % 4 == 0
 
@@ -44,8 +45,8 @@ class LinearWeight:
         """x @ W^T added into the sink's residual and prepared for its norm, as
         UnscaledRows; or, where the kernels do not take the case, returned."""
         rows = x.shape[0]
-        if self.tiled is None or not (ops.fused_rows_take(self.weight, rows) if rows > ops.FUSED_ROWS_FEW
-                                      else self.weight.shape[0] % 16 == 0):
+        if self.tiled is None or not (self.weight.shape[0] % 16 == 0 if rows <= ops.few_rows_limit(self.weight)
+                                      else ops.fused_rows_take(self.weight, rows)):
             return self.forward(x)
         fused = ops.linear_residual_norm(x, self.weight, self.tiled, sink.residual, sink.weight)
         if fused is None:                       # the kernel leaves this size to the plain product

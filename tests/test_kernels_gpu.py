@@ -678,7 +678,11 @@ def test_linear_swiglu(dtype, M, I, K):
 @pytest.mark.parametrize("norm_dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("M,H,K,N2", [(1, 4096, 4096, 6144), (8, 4096, 12288, 24576), (16, 96, 224, 160),
                                       (5, 992, 64, 330), (3, 32, 32, 48), (12, 4096, 1024, 24576),
-                                      (16, 1024, 512, 6152)])
+                                      (16, 1024, 512, 6152),
+                                      # small weights: 17 to 64 rows are two to four groups of the few-row kernel's blocks
+                                      (17, 1024, 512, 6152), (24, 1024, 2048, 4096), (32, 96, 224, 160),
+                                      (31, 1024, 4096, 8192), (20, 992, 64, 330), (48, 256, 128, 512),
+                                      (64, 1024, 512, 2048), (33, 96, 224, 160), (50, 1024, 2048, 4096)])
 def test_linear_residual_norm_and_unscaled_rows(M, H, K, N2, norm_dtype):
     """A product that adds itself into the residual stream and prepares the next norm, and the
     product after it, which applies the norm's division: together they give what the product,
@@ -702,10 +706,10 @@ def test_linear_residual_norm_and_unscaled_rows(M, H, K, N2, norm_dtype):
     fused_stream = residual.clone()
     values, sums = ops.linear_residual_norm(x, w1, t1, fused_stream, nw)
     assert torch.equal(fused_stream, stream)                      # the stream itself is the same to the bit
-    assert sums.shape == (H // 16, 16)
+    assert sums.shape == (H // 16, ops.sums_stride(M))
     ms = (stream.double() ** 2).sum(dim=1)
     torch.testing.assert_close(sums.double().sum(dim=0)[:M], ms, rtol=1e-5, atol=1e-6)
-    assert float(sums[:, M:].abs().max()) == 0.0 if M < 16 else True
+    assert float(sums[:, M:].abs().max()) == 0.0 if M < sums.shape[1] else True
     torch.testing.assert_close(values.float(), (stream * nw.float()), rtol=8e-3, atol=1e-6)
     got = ops.linear(values, w2, out_dtype=torch.float32, tiled=t2, unscaled=(sums, eps, H))
     # both roundings of the norm's output are to bfloat16, of numbers that differ by the row's factor
@@ -724,9 +728,10 @@ def test_linear_residual_norm_and_unscaled_rows(M, H, K, N2, norm_dtype):
         assert torch.equal(a[0], got[0])
     # what the kernel does not take is refused
     with pytest.raises(ops.OperandError):
-        ops.linear(_rand((17, H), torch.bfloat16, 1), w2, tiled=t2, unscaled=(sums, eps, H))
-    with pytest.raises(ops.OperandError):
-        ops.linear(values, w2, unscaled=(sums, eps, H))
+        ops.linear(_rand((M + 16, H), torch.bfloat16, 1), w2, tiled=t2, unscaled=(sums, eps, H))
+    if M <= 16:
+        with pytest.raises(ops.OperandError):
+            ops.linear(values, w2, unscaled=(sums, eps, H))
 
 
 @pytest.mark.parametrize("norm_dtype", [torch.float32, torch.bfloat16])
@@ -760,13 +765,13 @@ def test_linear_residual_norm_and_unscaled_rows_beyond_sixteen(M, H, K, N2, norm
         assert float(differs.float().mean()) < 0.02               # roundings at a bfloat16 tie aside
         torch.testing.assert_close(fused_stream, stream, rtol=0, atol=2 ** -7 * float(exact_delta.abs().max()))
         stream = fused_stream
-        assert sums.shape == (-(-H // 1024), M)
-        torch.testing.assert_close(sums.double().sum(dim=0), (stream.double() ** 2).sum(dim=1), rtol=1e-5, atol=1e-6)
+        assert sums.shape == (-(-H // 1024), ops.sums_stride(M))
+        torch.testing.assert_close(sums.double().sum(dim=0)[:M], (stream.double() ** 2).sum(dim=1), rtol=1e-5, atol=1e-6)
         assert torch.equal(values, (stream * nw.float()).bfloat16())
         # a second call gives the same bits (the choice of tile shape is kept, the additions are ordered)
         again_stream = residual.clone()
         v2, s2 = ops.linear_residual_norm(x, w1, None, again_stream, nw)
-        assert torch.equal(again_stream, fused_stream) and torch.equal(v2, values) and torch.equal(s2, sums)
+        assert torch.equal(again_stream, fused_stream) and torch.equal(v2, values) and torch.equal(s2[:, :M], sums[:, :M])
 
         h = ops.rmsnorm(stream.clone(), nw, eps, torch.bfloat16)
         want = ops.linear(h, w2, out_dtype=torch.float32)

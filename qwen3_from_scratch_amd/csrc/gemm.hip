@@ -92,7 +92,8 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const IN* __restrict__ a,
 
 
 // ---------------------------------------------------------------------------
-// bfloat16 with at most 16 rows: a weight-streaming kernel. Every weight is
+// bfloat16 with at most 16 rows (and, for small weights, a few groups of 16 rows, each a set of
+// blocks of its own: q3_linear_tiled): a weight-streaming kernel. Every weight is
 // read once from HBM and that read is the cost; the matrix cores do the sums
 // (v_mfma_f32_16x16x32_bf16) with 16 weight rows as the A operand and the rows
 // of x as the B operand, so out^T tiles come out with x's row in the lane's low

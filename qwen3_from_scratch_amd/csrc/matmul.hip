@@ -528,7 +528,7 @@ extern "C" int q3_matmul_init() {
 }
 
 // Products of up to 256 rows that carry a norm, by the hand-written tiled kernel (the few-row kernel of
-// gemm.hip does the same for up to 16 rows and is faster there; the callers' policy decides which rows come
+// gemm.hip does the same for up to 16 rows, or 64 of a small weight, and is faster there; the callers' policy decides which rows come
 // here). x (M, K) and w (N, K) bfloat16, K a multiple of 64, N of 4.
 //
 // q3_tiles_scaled: the rows of x hold stream * norm_weight and still lack the norm's division; `sums`

@@ -584,8 +584,9 @@ def linear(x, weight, out_dtype=None, out=None, tiled=None, unscaled=None):
     the product's rows receive it. Only the few-row kernel on a tiled weight does this.
 
     float32 operands take a float32 kernel with no reduced-precision mode;
-    bfloat16 operands with at most 16 rows take a weight-streaming matrix-core
-    kernel; bfloat16 with more rows is the vendor library's product.
+    bfloat16 operands with at most 16 rows (32 or 64 with the tiled copy of a small
+    weight, `few_rows_limit`) take a weight-streaming matrix-core kernel; bfloat16 with
+    more rows is the vendor library's product or the tiled kernel's.
     """
     _dev(x, weight, out)
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1], "x (M, K) and weight (N, K)")
@@ -606,8 +607,8 @@ def linear(x, weight, out_dtype=None, out=None, tiled=None, unscaled=None):
         return out
     if unscaled is not None and x.dtype == torch.bfloat16 and fused_rows_take(weight, M):
         return _tiles_scaled(x, weight, out, unscaled, False, "linear")
-    _need(unscaled is None, "unscaled rows need bfloat16 and at most 16 rows with a tiled weight, or 17 to 128 rows "
-          "with an inner size that is a multiple of 64")
+    _need(unscaled is None, "unscaled rows need bfloat16 and few rows with a tiled weight (few_rows_limit), or 17 to "
+          "128 rows with an inner size that is a multiple of 64")
     if M and x.dtype == torch.bfloat16 and not library("gemm").q3_linear_is_skinny(M, N, K, 1):
         # bfloat16 products with many rows go to the vendor library (hipBLASLt), as the
         # reference's engine uses its vendor library for them, or to the hand-written tiled
@@ -668,8 +669,8 @@ def linear_swiglu(x, weight, tiled=None, unscaled=None):
     if unscaled is not None and x.dtype == torch.bfloat16 and fused_rows_take(weight, M):
         out = torch.empty((M, N // 2), dtype=x.dtype, device=x.device)
         return _tiles_scaled(x, weight, out, unscaled, True, "linear_swiglu")
-    _need(unscaled is None, "unscaled rows need bfloat16 and at most 16 rows with a tiled weight, or 17 to 128 rows "
-          "with an inner size that is a multiple of 64")
+    _need(unscaled is None, "unscaled rows need bfloat16 and few rows with a tiled weight (few_rows_limit), or 17 to "
+          "128 rows with an inner size that is a multiple of 64")
     if M and library("gemm").q3_linear_is_skinny(M, N, K, _DT[x.dtype]):
         out = torch.empty((M, N // 2), dtype=x.dtype, device=x.device)
         _check(library("gemm").q3_linear_swiglu(_ptr(x), _ptr(weight), _ptr(out), M, N, K, _DT[x.dtype], _stream()),

@@ -123,8 +123,8 @@ class NormSink:
 @dataclass
 class UnscaledRows:
     """A norm's output before the division by the root mean square: `values`
-    (T, width) hold residual * weight in the activation dtype, `sums` (P, 16)
-    float32 (P, T beyond 16 rows) hold the rows' sums of squares in P partial
+    (T, width) hold residual * weight in the activation dtype, `sums` (P, T
+    rounded up to 16) float32 hold the rows' sums of squares in P partial
     sums (row t in column t). A part whose `takes_unscaled` is true accepts this in place of its
     input tensor and applies rsqrt(sum / width + eps) to its first product."""
 

@@ -10,9 +10,9 @@ from .base import UnscaledRows
 class LinearWeight:
     """y = x @ W^T, no bias. W (N, K) is kept row-major for products with many
     rows (the vendor library's) and for float32; when the precision asks for
-    it, a tile-ordered bfloat16 copy serves steps with at most 16 rows, where
-    every weight is read once and the order in memory decides the bandwidth.
-    The copy doubles the weight's memory."""
+    it, a tile-ordered bfloat16 copy serves steps with few rows (16, or 32 or 64
+    for a small weight), where every weight is read once and the order in memory
+    decides the bandwidth. The copy doubles the weight's memory."""
 
     def __init__(self, weight, precision):
         self.weight = weight

@@ -65,7 +65,9 @@ def test_linear_part_falls_back_where_the_kernel_declines(cpu_ops, monkeypatch):
     monkeypatch.setattr(ops, "linear_residual_norm", lambda *a: 1 / 0, raising=False)
     many = torch.randn(200, 64).bfloat16()
     assert torch.equal(part.forward_into(many, NormSink(torch.zeros(200, 128), norm.weight, norm.eps, norm.size)), part.forward(many))
-    odd = LinearWeight((torch.randn(128, 96) * 0.1).bfloat16(), precision)          # inner size 96: not in steps of 64
-    odd.tiled = torch.zeros(1)
-    x96 = torch.randn(40, 96).bfloat16()
-    assert torch.equal(odd.forward_into(x96, NormSink(torch.zeros(40, 128), norm.weight, norm.eps, norm.size)), odd.forward(x96))
+    odd = LinearWeight((torch.randn(128, 96) * 0.1).bfloat16(), precision)          # inner size 96: not in steps of 64,
+    odd.tiled = torch.zeros(1)                                                      # which the tiled kernel asks for
+    x96 = torch.randn(100, 96).bfloat16()                                           # (more rows than the few-row kernel takes)
+    assert torch.equal(odd.forward_into(x96, NormSink(torch.zeros(100, 128), norm.weight, norm.eps, norm.size)), odd.forward(x96))
+    assert ops.few_rows_limit(odd.weight) == 64 and ops.few_rows_limit(torch.zeros(24576, 4096, dtype=torch.bfloat16)) == 16
+    assert ops.few_rows_limit(torch.zeros(8192, 1024, dtype=torch.bfloat16)) == 32

@@ -69,5 +69,5 @@ def test_linear_part_falls_back_where_the_kernel_declines(cpu_ops, monkeypatch):
     odd.tiled = torch.zeros(1)                                                      # which the tiled kernel asks for
     x96 = torch.randn(100, 96).bfloat16()                                           # (more rows than the few-row kernel takes)
     assert torch.equal(odd.forward_into(x96, NormSink(torch.zeros(100, 128), norm.weight, norm.eps, norm.size)), odd.forward(x96))
-    assert ops.few_rows_limit(odd.weight) == 64 and ops.few_rows_limit(torch.zeros(24576, 4096, dtype=torch.bfloat16)) == 16
-    assert ops.few_rows_limit(torch.zeros(8192, 1024, dtype=torch.bfloat16)) == 32
+    assert ops.few_rows_limit(odd.weight) == 64 and ops.few_rows_limit(torch.empty(24576, 4096, dtype=torch.bfloat16, device="meta")) == 16
+    assert ops.few_rows_limit(torch.empty(8192, 1024, dtype=torch.bfloat16, device="meta")) == 32

@@ -64,7 +64,15 @@ def _ptr(t):
     return ctypes.c_void_p(0 if t is None else t.data_ptr())
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)   # the handle without a Stream object around it
+
+
 def _stream():
+    """The current device's current stream, as the launchers take it. Every operation asks, some
+    hundreds of times in a step that is not a graph replay, so the short way is taken where this
+    PyTorch has it (a fifth of such a step's host time otherwise)."""
+    if _raw_stream is not None:
+        return ctypes.c_void_p(_raw_stream(torch.cuda.current_device()))
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 

@@ -17,10 +17,12 @@ from qwen3_from_scratch_amd.engine import LLMEngine  # noqa: E402
 
 
 async def main(args):
+    options = {k: v for k, v in (("dtype", args.dtype),) if v is not None}
     if args.config_path:
-        engine = LLMEngine(args.config_path, args.model)
+        engine = LLMEngine(args.config_path, args.model, **options)
     else:
-        engine = LLMEngine(path=args.path)
+        engine = LLMEngine(path=args.path, **options)
+    sampling = {} if args.temperature is None else {"temperature": args.temperature}
     try:
         await engine.warmup()
         has_text = engine.engine.tokenizer is not None
@@ -29,7 +31,8 @@ async def main(args):
 
         async def ask(tag, prompt):
             chunk = None
-            async for chunk in engine.generate_stream(prompt, max_new_tokens=args.max_new_tokens, ignore_eos=True):
+            async for chunk in engine.generate_stream(prompt, max_new_tokens=args.max_new_tokens, ignore_eos=True,
+                                                      **sampling):
                 print("[%s] %s" % (tag, chunk.delta if has_text else chunk.token_id), flush=True)
             return tag, chunk
 
@@ -47,6 +50,8 @@ if __name__ == "__main__":
     p.add_argument("--model")
     p.add_argument("--path")
     p.add_argument("--max_new_tokens", type=int, default=16)
+    p.add_argument("--dtype", default=None, help="bfloat16 or float32; default: the configuration's")
+    p.add_argument("--temperature", type=float, default=None, help="0 = greedy; default: the configuration's")
     a = p.parse_args()
     if not (a.path or (a.config_path and a.model)):
         p.error("give --config_path and --model, or --path")

@@ -15,22 +15,25 @@ from qwen3_from_scratch_amd.engine import SyncEngine  # noqa: E402
 
 
 def main(args):
-    engine = SyncEngine(args.config_path, args.model) if args.config_path else SyncEngine(path=args.path)
+    options = {k: v for k, v in (("dtype", args.dtype),) if v is not None}
+    engine = (SyncEngine(args.config_path, args.model, **options) if args.config_path
+              else SyncEngine(path=args.path, **options))
+    sampling = {} if args.temperature is None else {"temperature": args.temperature}
     engine.warmup()
     has_text = engine.tokenizer is not None
     one = [{"role": "user", "content": "介绍一下自己"}] if has_text else [5, 17, 3, 9]
     print("=== one request, streamed ===")
     chunk = None
-    for chunk in engine.generate_stream(one, max_new_tokens=args.max_new_tokens):
+    for chunk in engine.generate_stream(one, max_new_tokens=args.max_new_tokens, **sampling):
         print(chunk.delta if has_text else chunk.token_id, end="" if has_text else " ", flush=True)
     m = chunk.metrics
     print("\nTTFT: %.4fs | tokens: %d | TPS: %.2f | total: %.4fs" % (m.ttft, m.token_count, m.tps, m.total_elapsed))
     print("=== one request, whole ===")
-    print(engine.generate("你好" if has_text else [2, 4, 6], max_new_tokens=args.max_new_tokens))
+    print(engine.generate("你好" if has_text else [2, 4, 6], max_new_tokens=args.max_new_tokens, **sampling))
     print("=== a batch ===")
     prompts = ([[{"role": "user", "content": t}] for t in ("介绍一下自己", "1+1等于几", "什么是深度学习")]
                if has_text else [[5, 17, 3], [2, 4, 6, 8], [9]])
-    texts, batch = engine.batch_generate(prompts, max_new_tokens=args.max_new_tokens)
+    texts, batch = engine.batch_generate(prompts, max_new_tokens=args.max_new_tokens, **sampling)
     for t in texts:
         print("- %s" % t)
     print("requests: %d | tokens: %d | total: %.4fs | throughput: %.2f tokens/s"
@@ -45,6 +48,8 @@ if __name__ == "__main__":
     p.add_argument("--model")
     p.add_argument("--path")
     p.add_argument("--max_new_tokens", type=int, default=16)
+    p.add_argument("--dtype", default=None, help="bfloat16 or float32; default: the configuration's")
+    p.add_argument("--temperature", type=float, default=None, help="0 = greedy; default: the configuration's")
     a = p.parse_args()
     if not (a.path or (a.config_path and a.model)):
         p.error("give --config_path and --model, or --path")

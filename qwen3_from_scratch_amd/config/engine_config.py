@@ -74,9 +74,30 @@ class EngineConfig:
     # keep a second copy of every bfloat16 matrix in the order the few-row product kernel streams it:
     # decoding is about a fifth faster with it, and the matrices take their memory twice
     tiled_weights: bool = True
+    # other registered implementations for some kinds of parts: {slot: name, or {name, kwargs}}
+    # (batch_config.py:209-229); checked here, applied when the model is built
+    components: dict = field(default_factory=dict)
+    # the reference's option for the cache's dtype (batch_config.py:164,275). The cache here is kept
+    # in the compute dtype; any other value is refused rather than ignored. None: not given.
+    kv_cache_dtype: str = None
+    # further tokens that end a request, beside those the model folder names
+    eos_ids: tuple = ()
 
     def __post_init__(self):
+        from .registry import resolve_components
+
         self.dtype = parse_dtype(self.dtype)
+        self.components = dict(self.components or {})
+        resolve_components(self.components)           # fails here, not when the model is built
+        if self.kv_cache_dtype is not None:
+            self.kv_cache_dtype = parse_dtype(self.kv_cache_dtype)
+            if self.kv_cache_dtype != self.dtype:
+                raise ConfigError(
+                    "kv_cache_dtype %s differs from dtype %s: this engine keeps the cache in the compute dtype "
+                    "(leave kv_cache_dtype out, or set it to the model's dtype)" % (self.kv_cache_dtype, self.dtype))
+        self.eos_ids = tuple(int(t) for t in (self.eos_ids or ()))
+        if any(t < 0 for t in self.eos_ids):
+            raise ConfigError("eos_ids must be token ids, found %r" % (self.eos_ids,))
         if self.max_len <= 0:
             raise ConfigError("max_len must be positive, found %d" % self.max_len)
         if self.block_size <= 0:
@@ -93,9 +114,10 @@ class EngineConfig:
         """Read the reference's YAML layout and pick `model_name` from `models`.
 
         Per-model `generation` entries override the global block field by field
-        (batch_config.py:194-207). `components` and `kv_cache_dtype` entries
-        are accepted and ignored: this engine has one implementation of each
-        part and keeps the cache in the compute dtype.
+        (batch_config.py:194-207). A model's `components` are checked against
+        the part registry and a top-level `kv_cache_dtype` against the model's
+        dtype; what this engine cannot honour is an error, as in the reference
+        (batch_config.py:369-382).
         """
         import yaml
 
@@ -131,7 +153,10 @@ class EngineConfig:
             dtype=entry.get("dtype", "bfloat16"),
             max_len=entry.get("max_len", 2048),
             generation=generation,
+            components=entry.get("components") or {},
         )
+        if "kv_cache_dtype" in raw:
+            kwargs["kv_cache_dtype"] = raw["kv_cache_dtype"]
         for key in ("max_num_seqs", "max_num_tokens", "block_size", "gpu_utilization",
                     "chunked_prefill_size", "num_blocks", "enable_prefix_cache"):
             if key in sched:

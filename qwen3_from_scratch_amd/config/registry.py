@@ -102,3 +102,52 @@ def lookup_part(kind, name):
 
 def part_names(kind):
     return sorted(_PARTS.get(kind, {}))
+
+
+# The reference names the slots of its component registry self_attn, mlp, norm, attn, rope and
+# decoder_layer (src/qwen3_from_scratch/factory/factory.py:7-9) and calls the implementation a
+# model starts with "base". Its slot names are understood beside this package's kinds.
+COMPONENT_SLOTS = {"self_attn": "mixer", "mlp": "feed_forward", "norm": "norm", "rope": "position",
+                   "decoder_layer": "block"}
+DEFAULT_COMPONENT = "base"
+
+
+def resolve_components(components):
+    """A user's `components` mapping, checked and brought to {part kind: (name or None, kwargs)}.
+
+    Each entry is `slot: name` or `slot: {name: ..., kwargs: {...}}`
+    (src/qwen3_from_scratch/factory/batch_config.py:209-229); a slot is one of this package's
+    part kinds or one of the reference's slot names; the name "base" keeps the part the
+    architecture names (None here). An unknown slot or a name that is not registered under the
+    slot's kind is an error that lists what there is
+    (src/qwen3_from_scratch/inference/model_loader.py:24-35): nothing is dropped silently."""
+    resolved = {}
+    if components is None:
+        return resolved
+    if not isinstance(components, dict):
+        raise ConfigError("components must be a mapping of slot to part name, found %r" % (components,))
+    for slot, value in components.items():
+        if slot == "attn":
+            raise ConfigError("components: the slot 'attn' has no counterpart here: attention over the paged "
+                              "cache is part of the mixer; name a mixer under 'self_attn' instead")
+        kind = COMPONENT_SLOTS.get(slot, slot)
+        if kind not in PART_KINDS:
+            raise ConfigError("components: unknown slot %r; valid: %s"
+                              % (slot, ", ".join(sorted(set(PART_KINDS) | set(COMPONENT_SLOTS)))))
+        if isinstance(value, str):
+            name, kwargs = value, {}
+        elif isinstance(value, dict):
+            if "name" not in value:
+                raise ConfigError("components: the entry of %r needs a 'name', found %r" % (slot, value))
+            name, kwargs = value["name"], dict(value.get("kwargs") or {})
+        else:
+            raise ConfigError("components: the entry of %r must be a name or a mapping with 'name' and 'kwargs', "
+                              "found %s" % (slot, type(value).__name__))
+        if kind in resolved:
+            raise ConfigError("components: the %s part is named twice" % kind)
+        if name == DEFAULT_COMPONENT and name not in _PARTS.get(kind, {}):
+            resolved[kind] = (None, kwargs)
+            continue
+        lookup_part(kind, name)           # raises, listing what is registered
+        resolved[kind] = (name, kwargs)
+    return resolved

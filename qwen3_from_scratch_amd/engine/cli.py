@@ -32,6 +32,12 @@ def main(argv=None):
     p.add_argument("--top_k", type=int, default=None)
     p.add_argument("--seed", type=int, default=0, help="sampling seed, and the seed of --write_random")
     p.add_argument("--ignore_eos", action="store_true")
+    p.add_argument("--eos_id", type=int, action="append", default=[], metavar="TOKEN",
+                   help="a token that ends a request, beside those the model folder names; repeatable")
+    p.add_argument("--component", action="append", default=[], metavar="SLOT=NAME",
+                   help="another registered implementation for a kind of part (the YAML's `components`), e.g. "
+                        "mlp=my_feed_forward; repeatable")
+    p.add_argument("--kv_cache_dtype", default=None, help="must equal --dtype: the cache is kept in the compute dtype")
     p.add_argument("--max_num_seqs", type=int, default=None)
     p.add_argument("--max_num_tokens", type=int, default=None)
     p.add_argument("--block_size", type=int, default=None)
@@ -71,6 +77,17 @@ def main(argv=None):
         "gpu_utilization", "chunked_prefill_size", "enable_prefix_cache", "tiled_weights")
         if getattr(args, k) is not None}
     overrides["seed"] = args.seed
+    if args.eos_id:
+        overrides["eos_ids"] = tuple(args.eos_id)
+    if args.kv_cache_dtype is not None:
+        overrides["kv_cache_dtype"] = args.kv_cache_dtype
+    if args.component:
+        overrides["components"] = {}
+        for item in args.component:
+            slot, _, name = item.partition("=")
+            if not slot or not name:
+                p.error("--component takes SLOT=NAME, found %r" % item)
+            overrides["components"][slot] = name
     if args.config_path:
         if not args.model:
             p.error("--config_path needs --model")

@@ -8,12 +8,14 @@ from ..parts.base import Precision
 from ..weights import Checkpoint, RandomWeights
 
 
-def load_model(model_dir, dtype="bfloat16", device="cuda", tiled_weights=True):
+def load_model(model_dir, dtype="bfloat16", device="cuda", tiled_weights=True, components=None):
     """Read config.json, pick the model by its architecture, load model.safetensors.
     `tiled_weights`: keep the second, tile-ordered copy of every bfloat16 matrix that makes steps
-    of few rows fast (see `Precision`); without it the matrices are held once."""
+    of few rows fast (see `Precision`); without it the matrices are held once.
+    `components`: {slot: part name, or {name, kwargs}}, other registered implementations for
+    some kinds of parts (src/qwen3_from_scratch/inference/model_loader.py:18-35)."""
     config = load_model_config(model_dir)
-    model = build_model(config, Precision.named(dtype, tiled=tiled_weights), device)
+    model = build_model(config, Precision.named(dtype, tiled=tiled_weights), device, components=components)
     model.load(Checkpoint(model_dir))
     model.config = config
     return model
@@ -29,9 +31,9 @@ def random_model(config, dtype="bfloat16", device="cuda", seed=0, std=0.02, norm
 
 
 def load_runner(model_dir, dtype="bfloat16", device="cuda", page_size=16, max_tokens=8192, max_requests=32,
-                use_graphs=True, tiled_weights=True):
+                use_graphs=True, tiled_weights=True, prefix_cache=False, components=None):
     from .runner import ModelRunner
 
-    model = load_model(model_dir, dtype, device, tiled_weights=tiled_weights)
+    model = load_model(model_dir, dtype, device, tiled_weights=tiled_weights, components=components)
     num_pages = -(-max_tokens // page_size)
-    return ModelRunner(model, page_size, num_pages, max_requests, use_graphs=use_graphs)
+    return ModelRunner(model, page_size, num_pages, max_requests, use_graphs=use_graphs, prefix_cache=prefix_cache)

@@ -83,7 +83,8 @@ class SyncEngine:
         self.model_name = model_name or config.name
         self.log_interval = log_interval
         self.model = model if model is not None else load_model(config.path, config.dtype, config.device,
-                                                                 tiled_weights=config.tiled_weights)
+                                                                 tiled_weights=config.tiled_weights,
+                                                                 components=config.components)
         self.tokenizer = _load_tokenizer(config.path) if config.path else None
         mc = self.model.config
         self.max_len = min(config.max_len, mc.max_position_embeddings)
@@ -131,7 +132,7 @@ class SyncEngine:
         return max(1, min(wanted, enough))
 
     def _eos_ids(self):
-        ids = set(self.model.config.eos_token_ids)
+        ids = set(self.model.config.eos_token_ids) | set(self.config.eos_ids)
         gen = os.path.join(self.config.path, "generation_config.json") if self.config.path else ""
         if gen and os.path.isfile(gen):
             with open(gen) as fh:

@@ -126,9 +126,11 @@ def expected_tensors(spec):
     return DecoderModel(spec, Precision(torch.bfloat16), "cpu").tensors()
 
 
-def build_model(config, precision, device):
-    """The model of `config`'s architecture, unloaded."""
-    from ..config.registry import lookup_architecture
+def build_model(config, precision, device, components=None):
+    """The model of `config`'s architecture, unloaded. `components`: a user's choice of other
+    registered implementations for some kinds of parts (`resolve_components`)."""
+    from ..config.registry import lookup_architecture, resolve_components
+    from .spec import with_components
 
     _, build_spec = lookup_architecture(config.architecture)
-    return DecoderModel(build_spec(config), precision, device)
+    return DecoderModel(with_components(build_spec(config), resolve_components(components)), precision, device)

@@ -61,3 +61,26 @@ class ModelSpec:
                 if not (0 <= j < i) or self.order[j].reads_cache_of is not None:
                     raise ValueError(
                         "run order entry %d must read the cache of an earlier entry that owns one" % i)
+
+
+def with_components(spec, resolved):
+    """`spec` with every part of a kind that `resolved` names (see
+    `config.registry.resolve_components`) replaced by the named implementation. The replacement
+    stands where the other stood: it is built with the same parameters (the sizes and constants
+    the architecture gave that place) plus the user's `kwargs`, so it must take them."""
+    if not resolved:
+        return spec
+    import dataclasses
+
+    def swap(part):
+        if part is None or part.kind not in resolved:
+            return part
+        name, kwargs = resolved[part.kind]
+        return PartSpec(part.kind, name or part.name, part.params).with_params(**kwargs)
+
+    layers = tuple(dataclasses.replace(
+        ls, mixer=swap(ls.mixer), feed_forward=swap(ls.feed_forward), mixer_norm=swap(ls.mixer_norm),
+        feed_forward_norm=swap(ls.feed_forward_norm), block=swap(ls.block), position=swap(ls.position))
+        for ls in spec.layers)
+    return dataclasses.replace(spec, embedding=swap(spec.embedding), position=swap(spec.position), layers=layers,
+                               final_norm=swap(spec.final_norm), head=swap(spec.head))

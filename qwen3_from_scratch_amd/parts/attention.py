@@ -8,6 +8,7 @@ from .base import CacheNeed, Part, TensorShape
 from .linear import LinearWeight
 
 
+@register_part("mixer", "paged_attn")        # the reference's name for this component (models/self_attn.py:300)
 @register_part("mixer", "attention")
 class PagedAttention(Part):
     """q, k, v projections (no bias), optional per-head RMSNorm of q and k before

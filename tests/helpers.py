@@ -41,6 +41,14 @@ TINY = {
                     num_key_value_heads=1, head_dim=128, intermediate_size=160, rms_norm_eps=1e-5,
                     rope_theta=500000.0, tie_word_embeddings=False),
         seed=43, std=0.04, norm_jitter=0.2, page_size=32),
+    # a width and inner sizes in steps of 64, so that steps of 65 to 128 rows take the tiled
+    # matrix-core product with the norms in its epilogues; weights so large that logits span tens
+    "F": dict(
+        config=dict(architectures=["Qwen3ForCausalLM"], vocab_size=520, hidden_size=128, hidden_act="silu",
+                    num_hidden_layers=2, max_position_embeddings=1024, num_attention_heads=4,
+                    num_key_value_heads=2, head_dim=64, intermediate_size=192, rms_norm_eps=1e-6,
+                    rope_theta=10000.0, tie_word_embeddings=False),
+        seed=53, std=0.2, norm_jitter=0.2, page_size=16),
 }
 # D and E with weights so large that logits span ten units or more, where a rounding of bfloat16
 # is small beside a fault; and with query norms twice as large, so that every query's

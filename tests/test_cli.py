@@ -23,6 +23,16 @@ def test_write_random_then_generate(cpu_ops, tmp_path, capsys):
     assert cli.main(args + ["--prompt_ids", "5,17,3", "--prompt_ids", "9,9"]) == 0
     lines = capsys.readouterr().out.strip().split("\n")
     assert len(lines) == 2 and lines[0].split() == one
+    # a token named with --eos_id ends the request that produces it (the folder names none)
+    args.remove("--ignore_eos")
+    assert cli.main(args + ["--prompt_ids", "5,17,3", "--eos_id", "100000", "--eos_id", one[2]]) == 0
+    assert capsys.readouterr().out.split() == one[:one.index(one[2]) + 1]
+    with pytest.raises(Exception) as caught:
+        cli.main(args + ["--prompt_ids", "5,17,3", "--component", "mlp=nothing_of_that_name"])
+    assert "nothing_of_that_name" in str(caught.value)
+    with pytest.raises(Exception) as caught:
+        cli.main(args + ["--prompt_ids", "5,17,3", "--kv_cache_dtype", "bfloat16"])
+    assert "kv_cache_dtype" in str(caught.value)
 
 
 def test_yaml_entry(cpu_ops, tmp_path, model_folders, capsys):

@@ -208,7 +208,61 @@ kv_cache_dtype: bfloat16
     assert cfg.generation.temperature == 0.7 and cfg.generation.top_k == 40
     assert cfg.generation.max_new_tokens == 512 and cfg.max_len == 2048
     assert cfg.enable_prefix_cache is False and EngineConfig().enable_prefix_cache is True
+    assert cfg.components == {"self_attn": "paged_attn"} and cfg.kv_cache_dtype == "bfloat16"
     with pytest.raises(KeyError):
         EngineConfig.from_yaml(str(path), "other")
     with pytest.raises(ConfigError):
         EngineConfig(dtype="float16")
+    # what the engine cannot honour is an error, not silence
+    for wrong, word in (("self_attn: \"paged_attn\"", "self_attn: \"my_op\""),
+                        ("self_attn: \"paged_attn\"", "sefl_attn: \"paged_attn\""),
+                        ("kv_cache_dtype: bfloat16", "kv_cache_dtype: float32")):
+        path.write_text(text.replace(wrong, word))
+        with pytest.raises(ConfigError) as caught:
+            EngineConfig.from_yaml(str(path), "tiny", device="cpu")
+        assert word.split(":")[0] in str(caught.value) or "my_op" in str(caught.value)
+
+
+def test_components_name_registered_parts_or_fail(cpu_ops, model_folders):
+    """`components` swaps in another registered implementation of a kind of part, under this
+    package's kind names or the reference's slot names; an unknown slot or name is an error
+    that lists what there is (src/qwen3_from_scratch/inference/model_loader.py:24-35)."""
+    from qwen3_from_scratch_amd.config import register_part
+    from qwen3_from_scratch_amd.config.registry import resolve_components
+    from qwen3_from_scratch_amd.engine import SyncEngine, load_model
+    from qwen3_from_scratch_amd.parts.norm import RMSNorm
+
+    @register_part("norm", "counted_rms")
+    class CountedNorm(RMSNorm):
+        calls = 0
+
+        def __init__(self, *args, bonus=0, **kw):
+            super().__init__(*args, **kw)
+            self.bonus = bonus
+
+        def forward(self, *args, **kw):
+            CountedNorm.calls += 1
+            return super().forward(*args, **kw)
+
+    assert resolve_components({"mlp": "base", "norm": {"name": "counted_rms", "kwargs": {"bonus": 2}}}) == {
+        "feed_forward": (None, {}), "norm": ("counted_rms", {"bonus": 2})}
+    model = load_model(model_folders["A"], "float32", "cpu", components={"norm": {"name": "counted_rms",
+                                                                                  "kwargs": {"bonus": 2}}})
+    norms = [model.final_norm] + [n for layer in model.layers for n in (layer.mixer_norm, layer.feed_forward_norm)]
+    assert all(type(n) is CountedNorm and n.bonus == 2 for n in norms)
+    plain = SyncEngine(path=model_folders["A"], dtype="float32", device="cpu", num_blocks=8)
+    swapped = SyncEngine(path=model_folders["A"], dtype="float32", device="cpu", num_blocks=8,
+                         components={"norm": "counted_rms", "decoder_layer": "base"})
+    before = CountedNorm.calls
+    ids = swapped.generate_ids([[5, 17, 3]], 4, temperature=0.0, ignore_eos=True)
+    assert CountedNorm.calls > before
+    assert ids == plain.generate_ids([[5, 17, 3]], 4, temperature=0.0, ignore_eos=True)
+    for wrong, word in (({"norm": "layer_norm_of_nowhere"}, "layer_norm_of_nowhere"), ({"norms": "rms"}, "norms"),
+                        ({"attn": "flash"}, "attn"), ({"mlp": {"kwargs": {}}}, "name"), ({"mlp": 3}, "mlp"),
+                        ({"mlp": "swiglu", "feed_forward": "swiglu"}, "twice")):
+        with pytest.raises(ConfigError) as caught:
+            EngineConfig(components=wrong)
+        assert word in str(caught.value)
+    with pytest.raises(ConfigError):
+        EngineConfig(dtype="bfloat16", kv_cache_dtype="fp32")
+    assert EngineConfig(dtype="float32", kv_cache_dtype="fp32").kv_cache_dtype == "float32"

@@ -60,7 +60,8 @@ def _compare(got, want, dtype):
 
 CASES = [("A", [5, 17, 33, 80]), ("B", [1, 9, 64, 130]), ("C", [40, 70, 3, 201]),
          ("D", [33, 1, 150, 64, 300]), ("E", [129, 31, 260]),
-         ("DS", [33, 1, 150, 64, 300]), ("ES", [129, 31, 260]), ("DP", [200, 17, 330, 64]), ("EP", [129, 300, 70])]
+         ("DS", [33, 1, 150, 64, 300]), ("ES", [129, 31, 260]), ("DP", [200, 17, 330, 64]), ("EP", [129, 300, 70]),
+         ("F", [70, 100, 128, 230])]
 FAMILIES = {"whole": trace_whole, "tail": trace_tail_decoded, "portions": trace_portions, "mixed": trace_mixed}
 
 
@@ -76,6 +77,49 @@ def test_every_cutting_matches_plain(model_folders, dtype, name, lengths, family
                          max_tokens=max_live_tokens(steps, page=page), max_requests=4)
     got = run_trace(runner, steps)
     _compare(got, want, dtype)
+    assert runner.manager.num_free() == runner.manager.num_pages()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("family", ["portions", "mixed"])
+def test_steps_of_65_to_128_rows(model_folders, dtype, family):
+    """Configuration F (width 128, inner sizes 192 and 256) in steps of 65 to 128 rows: in bfloat16
+    those take the tiled matrix-core product with the residual addition and the norms in its
+    epilogues, which no other tiny configuration reaches (their widths are no multiple of 64).
+    Portions of 70, 100 and 128 tokens of one request, and portions of 40 to 60 tokens of two or
+    three requests side by side."""
+    from qwen3_from_scratch_amd import ops
+
+    name = "F"
+    requests = _requests(name, [298, 170, 230, 129])
+    want = _plain(model_folders[name], name, requests)
+    if family == "portions":
+        steps = trace_portions(requests, sizes=(70, 100, 128))
+    else:
+        steps, at, live = [], {rid: 0 for rid in requests}, ["r0", "r1"]
+        waiting = ["r2", "r3"]
+        k = 0
+        while live:
+            entries, ends = [], []
+            for rid in list(live):
+                n = min((40, 47, 60, 33)[k % 4], len(requests[rid]) - at[rid])
+                k += 1
+                entries.append((rid, requests[rid][at[rid]:at[rid] + n], list(range(n))))
+                at[rid] += n
+                if at[rid] == len(requests[rid]):
+                    ends.append(rid)
+                    live.remove(rid)
+                    if waiting:
+                        live.append(waiting.pop(0))
+            steps.append((entries, ends))
+    rows = [sum(len(t) for _, t, _ in entries) for entries, _ in steps]
+    assert sum(64 < r <= 128 for r in rows) >= 6
+    runner = load_runner(model_folders[name], dtype=dtype, device="cuda", page_size=16,
+                         max_tokens=max_live_tokens(steps, page=16), max_requests=4)
+    if dtype == "bfloat16":          # the sizes are the tiled kernel's: the test would say nothing otherwise
+        mixer = runner.model.layers[0].mixer
+        assert ops.fused_rows_take(mixer.qkv.weight, 100) and ops.few_rows_limit(mixer.qkv.weight) == 64
+    _compare(run_trace(runner, steps), want, dtype)
     assert runner.manager.num_free() == runner.manager.num_pages()
 
 

@@ -7,7 +7,7 @@ import pytest
 import torch
 
 import plain_qwen3
-from helpers import max_live_tokens, random_tokens, run_trace, trace_mixed, trace_portions
+from helpers import max_live_tokens, off_by, random_tokens, run_trace, trace_mixed, trace_portions
 from qwen3_from_scratch_amd.config import ModelConfig
 from qwen3_from_scratch_amd.engine import load_runner
 from qwen3_from_scratch_amd.weights import write_random_model
@@ -34,22 +34,47 @@ CONFIGS = {
 }
 
 
-@pytest.mark.parametrize("name", sorted(CONFIGS))
-def test_edge_sizes_match_plain(name, tmp_path):
+# configurations whose query norms are doubled after the weights are drawn: every query's softmax
+# then stands on a few keys, most of them far back, and a key that the general attention kernel
+# dropped would move the rows that stood on it by many times the bound
+PEAKED = {"head_96_groups_of_6", "head_128_groups_of_20"}
+CASES = sorted(CONFIGS) + sorted(name + "+peaked" for name in PEAKED)
+
+
+def _double_query_norms(folder):
+    import os
+
+    from safetensors.torch import load_file, save_file
+
+    path = os.path.join(folder, "model.safetensors")
+    tensors = load_file(path)
+    for key in tensors:
+        if key.endswith("q_norm.weight"):
+            tensors[key] = (tensors[key].float() * 2.0).to(tensors[key].dtype)
+    save_file(tensors, path, metadata={"format": "pt"})
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_edge_sizes_match_plain(case, tmp_path):
+    """Weights of standard deviation 0.2, so that logits span tens of units and a rounding of
+    bfloat16 is small beside a fault; a row may be off by 2e-4 of its largest magnitude in
+    float32 and by a fiftieth of its own spread in bfloat16 (`helpers.off_by`)."""
+    name = case.split("+")[0]
     config = CONFIGS[name]
     folder = str(tmp_path / name)
-    write_random_model(folder, ModelConfig.from_dict(config), seed=5, std=0.03, norm_jitter=0.2)
+    write_random_model(folder, ModelConfig.from_dict(config), seed=5, std=0.2, norm_jitter=0.2)
+    if case.endswith("+peaked"):
+        _double_query_norms(folder)
     plain_config, weights = plain_qwen3.read_model_folder(folder)
     requests = {"r%d" % i: random_tokens(n, config["vocab_size"], 50 + i) for i, n in enumerate([70, 300, 9, 41])}
     want = {rid: plain_qwen3.logits_of_sequence(plain_config, weights, toks) for rid, toks in requests.items()}
-    for dtype, tol in (("float32", 2e-5), ("bfloat16", 4e-2)):
+    for dtype in ("float32", "bfloat16"):
         for make in (trace_portions, trace_mixed):
             steps = make(requests)
             runner = load_runner(folder, dtype=dtype, device="cuda", page_size=16, max_tokens=max_live_tokens(steps),
                                  max_requests=8)
             got = run_trace(runner, steps)
             for rid, logits in want.items():
-                scale = max(1.0, float(logits.abs().max()))
-                mine = torch.stack([got[(rid, p)] for p in range(logits.shape[0])])
-                assert float((mine - logits).abs().max()) <= tol * scale, (dtype, make.__name__, rid)
+                worst = max(off_by(got[(rid, p)], logits[p], dtype) for p in range(logits.shape[0]))
+                assert worst <= 1.0, (dtype, make.__name__, rid, worst)
             assert runner.manager.num_free() == runner.manager.num_pages()

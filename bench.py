@@ -10,7 +10,7 @@ through the engine's own step loop (scheduler, step function, sampling). A
 `value` is decoded tokens per second at the default batch; `prefill` is one
 2,048-token prompt in one step (the median of three); `roofline` prices the decode step against HBM
 bandwidth, the published peak and the rate a plain read kernel reaches on this GPU (`measured_peak`);
-`points` holds decoding at batch 1 and 64, `points_roofline` their fractions of the published peak. The default run is the
+`points` holds decoding at batch 1 and 64 and a prompt of 8,192 tokens in one step (tokens a second), `points_roofline` their fractions of the published peaks. The default run is the
 8B shape with prompts of 2,048 in a context of 8,192; `--shape`, `--prompt` and
 `--context` move the decode measurement to the larger shapes and to longer
 contexts (the prefill measurement stays at 2,048 tokens).
@@ -37,6 +37,7 @@ QWEN3_06B = dict(QWEN3_8B, hidden_size=1024, num_hidden_layers=28, num_attention
 SHAPES = {"8b": ("Qwen3-8B", QWEN3_8B), "14b": ("Qwen3-14B", QWEN3_14B), "32b": ("Qwen3-32B", QWEN3_32B),
           "0.6b": ("Qwen3-0.6B", QWEN3_06B)}
 PREFILL = 2048
+LONG_PREFILL = 8192          # a second prompt length, reported under `points`
 BLOCK = 16
 
 
@@ -329,6 +330,8 @@ def main():
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 points")
     ap.add_argument("--no-probes", action="store_true",
                     help="skip the measurement of this GPU's read and matrix rates (for profiles of the engine alone)")
+    ap.add_argument("--prefill-tokens", type=int, default=PREFILL,
+                    help="length of the prompt whose one step is the prefill measurement (2,048 in the default line)")
     ap.add_argument("--skip-prefill", action="store_true",
                     help="skip the prefill measurement (for profiles of decoding alone; the line then has no value for it)")
     args = ap.parse_args()
@@ -378,25 +381,33 @@ def main():
     if args.workload == "prefix":
         return shared_prefix(args, config, model, shape_name, gen, sync)
 
-    # ---- prefill: one prompt of 2,048 tokens in one step ----
-    engine = engine_for(1)
-    timings = []
-    for _ in range(0 if args.skip_prefill else 4):   # a warm-up, then three timed ones, each a new prompt
-        engine.add_request(prompts(1, PREFILL)[0], engine.default_params(1, temperature=0.0, ignore_eos=True))
-        sync()
-        t0 = time.perf_counter()
-        plan = engine.step()
-        sync()
-        timings.append(time.perf_counter() - t0)
-        assert len(plan) == 1 and plan[0].num_tokens == PREFILL
-        while engine.scheduler.has_work():
-            engine.step()
+    # ---- prefill: one prompt of 2,048 tokens in one step (and of 8,192 for `points`) ----
+    def prefill_of(tokens, timed=3):
+        """Seconds of one step that is one whole prompt of `tokens` tokens: a warm-up, then the
+        median of `timed` runs, each a new prompt."""
+        room = tokens + 64
+        engine = SyncEngine(model=model, path="", dtype=args.dtype, device="cuda:0", max_len=room,
+                            block_size=BLOCK, num_blocks=-(-room // BLOCK), max_num_seqs=1,
+                            max_num_tokens=tokens, chunked_prefill_size=tokens, enable_prefix_cache=False)
+        timings = []
+        for _ in range(1 + timed):
+            engine.add_request(prompts(1, tokens)[0], engine.default_params(1, temperature=0.0, ignore_eos=True))
+            sync()
+            t0 = time.perf_counter()
+            plan = engine.step()
+            sync()
+            timings.append(time.perf_counter() - t0)
+            assert len(plan) == 1 and plan[0].num_tokens == tokens
+            while engine.scheduler.has_work():
+                engine.step()
+        return sorted(timings[1:])[timed // 2]
+
     prefill = None
-    prefill_s = sorted(timings[1:])[1] if timings else None      # the median of the timed three
+    prefill_s = None if args.skip_prefill else prefill_of(args.prefill_tokens)
     if prefill_s is not None:
-        prefill = {"value": round(PREFILL / prefill_s, 1), "tokens": PREFILL, "ms": round(prefill_s * 1e3, 3),
-                   "frac": round(prefill_flops(config, PREFILL) / prefill_s / PEAK_FLOPS[args.dtype], 4)}
-    del engine
+        prefill = {"value": round(args.prefill_tokens / prefill_s, 1), "tokens": args.prefill_tokens,
+                   "ms": round(prefill_s * 1e3, 3),
+                   "frac": round(prefill_flops(config, args.prefill_tokens) / prefill_s / PEAK_FLOPS[args.dtype], 4)}
 
     # ---- decode ----
     def decode(batch, steps, warmup):
@@ -423,6 +434,11 @@ def main():
     roofline = {"bound": "hbm", "achieved": round(need / step_s / 1e9, 1), "peak": PEAK_HBM / 1e9,
                 "unit": "GB/s", "frac": round(need / step_s / PEAK_HBM, 4)}
     points, points_roofline = {}, {}
+    if not args.no_points and not args.skip_prefill and config.max_position_embeddings > LONG_PREFILL + 64:
+        long_s = prefill_of(LONG_PREFILL, timed=1)          # one more step of a tenth of a second
+        points["prefill_%d" % LONG_PREFILL] = round(LONG_PREFILL / long_s, 1)
+        points_roofline["prefill_%d" % LONG_PREFILL] = round(
+            prefill_flops(config, LONG_PREFILL) / long_s / PEAK_FLOPS[args.dtype], 4)
     if not args.no_points:
         for b in (1, 64):
             if b == args.batch:
@@ -442,7 +458,7 @@ def main():
         roofline["frac_of_measured"] = round(need / step_s / read_rate, 4)
     if prefill is not None and args.dtype == "bfloat16" and matrix_rate:
         prefill["measured_peak_tflops"] = round(matrix_rate / 1e12, 1)
-        prefill["frac_of_measured"] = round(prefill_flops(config, PREFILL) / prefill_s / matrix_rate, 4)
+        prefill["frac_of_measured"] = round(prefill_flops(config, args.prefill_tokens) / prefill_s / matrix_rate, 4)
 
     line = {
         "metric": "decode tok/s at batch 1/8/64 + prefill tok/s at 2048 tokens, %s %s"

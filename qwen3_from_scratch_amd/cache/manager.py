@@ -1,8 +1,8 @@
 """The cache manager: which pages and which state slot every live request holds.
 
 Layers are put in groups by what their mixers keep (`CacheNeed`): layers that
-keep all keys and values of a given (kv_heads, head_dim) share a group, layers
-that keep a window of them form another, and so on. A group has a page pool of
+keep the same paged tensors for all tokens share a group, layers that keep a
+window of them form another, and so on. A group has a page pool of
 its own and, per request, one block table that serves all its layers: page p of
 a group exists once in each of the group's layers' planes. A request's pages
 go back to the pool when it ends, and, in a windowed group, as soon as every
@@ -38,8 +38,7 @@ from .pages import OutOfPages, PagePool
 
 @dataclass
 class _Group:
-    kv_heads: int
-    head_dim: int
+    tensors: tuple                       # the PagedTensors that every layer of the group keeps
     window: int
     planes: list
     pool: PagePool
@@ -89,9 +88,9 @@ class CacheManager:
         for plane, need in enumerate(needs):
             g = s = -1
             if need is not None and need.paged:
-                key = (need.kv_heads, need.head_dim, need.window)
+                key = (tuple(need.paged), need.window)
                 for i, grp in enumerate(self.groups):
-                    if (grp.kv_heads, grp.head_dim, grp.window) == key:
+                    if (grp.tensors, grp.window) == key:
                         g = i
                 if g < 0:
                     self.groups.append(_Group(*key, planes=[], pool=PagePool(num_pages)))

@@ -1538,13 +1538,15 @@ extern "C" int q3_decode_attention_takes(int Hq, int Hkv, int D, int page, int d
 // of q and k (weights of `w_dtype`, both or neither), rotation by `table` (or null), the new
 // key and value written to the caches at position kv_lens[b] - 1 (if `store`), and attention
 // over the cache, in one kernel and, with more than one split, the merge of its partial
-// results (workspace as for q3_paged_attention). out (B, Hq D) bfloat16.
+// results (workspace as for q3_paged_attention). out (B, Hq D) bfloat16. `max_kv_len`: a bound
+// on kv_lens that the host knows; a step that would pass the rotation table's end is refused.
 extern "C" int q3_decode_attention(const void* qkv, void* out, void* k_cache, void* v_cache, int num_pages,
                                    const int* block_table, int bt_stride, const int* cu_q, const int* kv_lens,
                                    int B, int Hq, int Hkv, int D, int page, float scale, int window, int splits,
                                    float* workspace, const void* q_weight, const void* k_weight, int w_dtype,
                                    float eps, const float* table, int rotary_dim, int max_pos, int store,
-                                   hipStream_t stream) {
+                                   int max_kv_len, hipStream_t stream) {
+  if (table && max_kv_len > max_pos) return Q3_ERR_BAD_ARGUMENT;
   if (B <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || page <= 0) return Q3_ERR_BAD_ARGUMENT;
   if (B > 65535) return Q3_ERR_UNSUPPORTED;
   if (!q3_decode_attention_takes(Hq, Hkv, D, page, Q3_BF16, table ? rotary_dim : 0)) return Q3_ERR_UNSUPPORTED;

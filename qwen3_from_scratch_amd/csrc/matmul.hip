@@ -112,11 +112,11 @@ enum { MODE_RULE = 0, MODE_TUNE = 1 };
 int g_mode = MODE_RULE;
 
 // Sizes that differ only within a step of rows share a table entry (a serving loop meets dozens of them, a
-// prompt's portion plus however many requests decode): plain products up to 64 rows by their own count, beyond
-// in steps of 32; the products that carry a norm in steps of 8.
+// prompt's portion plus however many requests decode): up to 64 rows, and the products that carry a norm at
+// any count, in steps of 8; plain products beyond 64 rows in steps of 32.
 int rows_key(int kind, int M) {
-  if (kind != KIND_PLAIN) return (M + 7) / 8 * 8;
-  return M <= 64 ? M : (M + 31) / 32 * 32;
+  if (kind != KIND_PLAIN || M <= 64) return (M + 7) / 8 * 8;
+  return (M + 31) / 32 * 32;
 }
 
 #define HIP_TRY(call)                    \
@@ -391,8 +391,10 @@ int run_plan(Device& d, const Plan& p, const void* x, const void* w, void* out, 
   return s == HIPBLAS_STATUS_SUCCESS ? 0 : Q3_ERR_LIBRARY + (int)s;
 }
 
-// Makes the plan ready by `c`: for the library, its candidate number c.library for this exact size (its last
-// one if it offers fewer; the hand-written kernel if it offers none and that takes the size).
+// Makes the plan ready by `c`: for the library, its candidate number c.library for this exact size (its first
+// one, the rule of thumb, if it offers fewer: an entry is made at one row count and shared by its neighbours,
+// whose ranked lists may be shorter, and the last of a short list is the library's worst offer; the
+// hand-written kernel if the library offers none and that takes the size). q3_matmul_plan tells which it was.
 int settle(Device& d, Plan& p, Choice c, int M, int N, int K) {
   p.choice = c;
   p.candidates = 1;
@@ -405,7 +407,7 @@ int settle(Device& d, Plan& p, Choice c, int M, int N, int K) {
     } else if (status) {
       return status;
     } else {
-      p.choice.library = c.library < (int)found.size() ? c.library : (int)found.size() - 1;
+      p.choice.library = c.library < (int)found.size() ? c.library : 0;
       p.algo = found[p.choice.library].algo;
     }
   }

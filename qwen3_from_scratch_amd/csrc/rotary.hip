@@ -375,14 +375,17 @@ static int launch_qk_vec(void* qkv, const void* qw, const void* kw, float eps, c
 }
 
 // `cu_q`, `kv_lens`, `B`, `max_q_len` describe the step's sequences (they may be null / 0: then
-// only the one-wavefront-per-head kernel is used).
+// only the one-wavefront-per-head kernel is used). `max_kv_len`: what the host knows of the
+// step's last position + 1 (0: nothing); a step that would pass the rotation table's end is
+// refused, since a row without its rotation is a wrong answer, not an error anyone sees.
 extern "C" int q3_qk_norm_rope_store(void* qkv, const void* q_weight, const void* k_weight, int w_dtype,
                                      float eps, const float* table, int rotary_dim, int max_pos,
                                      const int* positions, const int* seq_index, const int* block_table,
                                      int bt_stride, int bt_rows, void* k_cache, void* v_cache,
                                      int page_size, int num_pages, int T_, int Hq, int Hkv, int D,
                                      int act_dtype, const int* cu_q, const int* kv_lens, int B, int max_q_len,
-                                     hipStream_t stream) {
+                                     int max_kv_len, hipStream_t stream) {
+  if (table && max_kv_len > max_pos) return Q3_ERR_BAD_ARGUMENT;
   if (T_ <= 0 || Hq <= 0 || Hkv <= 0 || D <= 0 || (Hq + 2 * Hkv + 3) / 4 > 65535) return Q3_ERR_BAD_ARGUMENT;
   if (table && (rotary_dim <= 0 || rotary_dim % 2 || rotary_dim > D)) return Q3_ERR_BAD_ARGUMENT;
   if (k_cache && (!v_cache || !block_table || page_size <= 0)) return Q3_ERR_BAD_ARGUMENT;

@@ -28,6 +28,9 @@ int q3_sample(const float* logits, const float* temperature, const int* top_k, c
 // refused with Q3_ERR_UNSUPPORTED (10002) and launches nothing. All calls on one GPU share that
 // GPU's array: calls that overlap there (two streams, two threads) race; calls on one stream do
 // not. Inputs and outputs are the caller's, as for q3_sample, and the result is the same.
+// The first call on a device asks the runtime for the address of that device's array
+// (hipGetSymbolAddress, under a lock); make it outside a graph capture. Later calls launch
+// kernels only and may be captured.
 int q3_sample_static(const float* logits, const float* temperature, const int* top_k, const long long* seed,
                      const int* counter, int* out, int R, int V, int with_top_k, hipStream_t stream);
 }

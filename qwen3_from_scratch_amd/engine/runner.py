@@ -189,7 +189,10 @@ class ModelRunner:
         self.manager = CacheManager(model.plane_needs, page_size, num_pages, max_requests, prefix_cache=prefix_cache)
         self.storage = CacheStorage(self.manager, model.precision.act, self.device)
         self.vocab_size = model.spec.vocab_size
-        self.max_positions = getattr(model.position, "max_positions", None)
+        # the shortest table of positions among the model's position part and the layers' own
+        tables = [getattr(part, "max_positions", None)
+                  for part in [model.position] + list(getattr(model, "layer_positions", {}).values())]
+        self.max_positions = min((n for n in tables if n is not None), default=None)
         self.max_request_tokens = self.manager.capacity_tokens()
         if self.max_positions is not None:
             self.max_request_tokens = min(self.max_request_tokens, self.max_positions)

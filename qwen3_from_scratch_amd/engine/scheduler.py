@@ -73,9 +73,16 @@ class Scheduled:
 
 class Scheduler:
     def __init__(self, manager, max_num_seqs, max_num_tokens, chunked_prefill_size,
-                 max_len=None, release=None):
+                 max_len=None, release=None, portion_multiple=1):
         """`manager`: the cache manager (asked what fits; pages are taken by the
-        step itself). `release(request_id)`: gives back what a request holds."""
+        step itself). `release(request_id)`: gives back what a request holds.
+        `portion_multiple`: every portion of a prompt except its last is cut to a
+        multiple of this many tokens (what the model's parts ask for); the
+        reference has no counterpart."""
+        if portion_multiple < 1 or portion_multiple > min(chunked_prefill_size, max_num_tokens):
+            raise ValueError("portions must be multiples of %d tokens, which chunked_prefill_size (%d) and "
+                             "max_num_tokens (%d) must allow" % (portion_multiple, chunked_prefill_size, max_num_tokens))
+        self.portion_multiple = portion_multiple
         if max_num_seqs > manager.max_requests:
             raise ValueError("max_num_seqs (%d) exceeds the cache's request slots (%d)"
                              % (max_num_seqs, manager.max_requests))
@@ -152,14 +159,25 @@ class Scheduler:
         self.running = deque(prefilling + list(ready) + [s.request for s in scheduled])
         return scheduled
 
+    def _portion(self, req, room):
+        """How many of the request's tokens go into a step with `room` left in its token budget:
+        all that are left, or as many as the limits allow, cut so that the portion ends at a
+        multiple of the portion multiple, counted from the request's first token (a request that
+        starts behind shared pages or again after a preemption keeps the same cuts)."""
+        left = req.prefill_target - req.computed
+        n = min(left, self.chunked_prefill_size, room)
+        if n < left:
+            n -= (req.computed + n) % self.portion_multiple
+        return n
+
     def _schedule_prefill(self, max_seqs, max_tokens, spare):
         scheduled = []
         tokens = 0
         for req in [r for r in self.running if r.is_prefill]:
             if len(scheduled) >= max_seqs or tokens >= max_tokens:
                 break
-            n = min(req.prefill_target - req.computed, self.chunked_prefill_size, max_tokens - tokens)
-            if not self.manager.can_grow(req.request_id, n, spare):
+            n = self._portion(req, max_tokens - tokens)
+            if n <= 0 or not self.manager.can_grow(req.request_id, n, spare):
                 continue
             scheduled.append(Scheduled(req, n, req.computed + n == req.num_tokens))
             tokens += n
@@ -167,8 +185,8 @@ class Scheduler:
                 and len(self.running) < self.max_num_seqs:
             req = self.waiting[0]
             shared = self._share_prefix(req)
-            n = min(req.prefill_target - req.computed, self.chunked_prefill_size, max_tokens - tokens)
-            if not self.manager.can_grow(req.request_id, n, spare):
+            n = self._portion(req, max_tokens - tokens)
+            if n <= 0 or not self.manager.can_grow(req.request_id, n, spare):
                 if shared:                              # it waits on: what it took over goes back
                     self.manager.prefix_hits -= req.computed
                     self.manager.release(req.request_id)

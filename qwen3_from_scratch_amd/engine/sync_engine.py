@@ -94,7 +94,7 @@ class SyncEngine:
         self.sampler = Sampler(self.model.device)
         self.scheduler = Scheduler(
             self.runner.manager, config.max_num_seqs, config.max_num_tokens, config.chunked_prefill_size,
-            max_len=self.max_len, release=self.runner.finish)
+            max_len=self.max_len, release=self.runner.finish, portion_multiple=self.model.portion_multiple())
         self.eos_ids = self._eos_ids()
         self._ids = itertools.count()
         self.steps = 0
@@ -106,21 +106,15 @@ class SyncEngine:
     # ---- set-up ----
     def _blocks_from_memory(self):
         """Pages that fit in `gpu_utilization` of the free memory beside the
-        requests' fixed-size states, halved for keys and values, as the reference
+        requests' fixed-size states, as the reference
         sizes its cache (src/qwen3_from_scratch/inference/kv_cache/paged_cache.py:36-49).
         A page stands for its tokens in every layer of every group."""
         per_token = per_request = 0
-        itemsize = 2 if self.model.precision.act == torch.bfloat16 else 4
         for need in self.model.plane_needs:
             if need is None:
                 continue
-            if need.paged:
-                per_token += 2 * need.kv_heads * need.head_dim * itemsize
-            if need.has_state:           # a slot per request (and a spare one) in every plane that keeps a state
-                size = torch.empty((), dtype=need.state_dtype).element_size()
-                for n in need.state_shape:
-                    size *= n
-                per_request += size
+            per_token += need.bytes_per_token(self.model.precision.act)
+            per_request += need.bytes_of_state()    # a slot per request (and a spare one) in every plane with a state
         per_page = max(1, per_token * self.config.block_size)
         if self.model.device.type == "cuda":
             free = torch.cuda.mem_get_info(self.model.device)[0]

@@ -9,20 +9,30 @@ from ..weights.checkpoint import check_tensors
 
 
 class _Layer:
+    """A layer's block and the parts it arranges, built from a LayerSpec. The parts are also
+    reachable by the names the spec gave them (`layer.mixer`, `layer.feed_forward_norm`, ...)."""
+
     def __init__(self, spec, precision, device, position):
-        p = spec.prefix
-        self.block = build_part(spec.block, p, precision, device)
-        self.mixer = build_part(spec.mixer, p + "." + spec.mixer_prefix, precision, device)
-        self.feed_forward = build_part(spec.feed_forward, p + "." + spec.feed_forward_prefix, precision, device)
-        self.mixer_norm = build_part(spec.mixer_norm, p + "." + spec.mixer_norm_prefix, precision, device)
-        self.feed_forward_norm = build_part(
-            spec.feed_forward_norm, p + "." + spec.feed_forward_norm_prefix, precision, device)
-        if hasattr(self.mixer, "attach_position"):
-            self.mixer.attach_position(position)
-        self.block.attach(self.mixer, self.feed_forward, self.mixer_norm, self.feed_forward_norm)
+        self.block = build_part(spec.block, spec.prefix, precision, device)
+        self.named = {slot.name: build_part(slot.part, spec.prefix + "." + slot.prefix, precision, device)
+                      for slot in spec.slots}
+        keepers = [name for name, part in self.named.items() if hasattr(part, "cache_need")]
+        if len(keepers) > 1:
+            raise ValueError("layer %s: more than one part keeps a cache (%s)" % (spec.prefix, ", ".join(keepers)))
+        self.cache_owner = self.named[keepers[0]] if keepers else None
+        for part in self.named.values():
+            if hasattr(part, "attach_position"):
+                part.attach_position(position)
+        self.block.attach(**self.named)
+
+    def __getattr__(self, name):
+        named = self.__dict__.get("named", {})
+        if name in named:
+            return named[name]
+        raise AttributeError(name)
 
     def parts(self):
-        return (self.block, self.mixer, self.feed_forward, self.mixer_norm, self.feed_forward_norm)
+        return (self.block,) + tuple(self.named.values())
 
 
 class DecoderModel:
@@ -46,8 +56,8 @@ class DecoderModel:
         self.plane_needs = []
         for i, step in enumerate(spec.order):
             if step.reads_cache_of is None:
-                mixer = self.layers[step.layer].mixer
-                need = mixer.cache_need() if hasattr(mixer, "cache_need") else None
+                owner = self.layers[step.layer].cache_owner
+                need = owner.cache_need() if owner is not None else None
                 self.plane_of_step.append(len(self.plane_needs))
                 self.plane_needs.append(need)
             else:
@@ -61,6 +71,19 @@ class DecoderModel:
             yield from layer.parts()
         yield self.final_norm
         yield self.head
+
+    def portion_multiple(self):
+        """The number of tokens that every portion of a prompt except its last must be a
+        multiple of: the least common multiple of what the parts say (`Part.portion_multiple`)."""
+        import math
+
+        multiple = 1
+        for part in self.parts():
+            n = int(getattr(part, "portion_multiple", 1) or 1)
+            if n < 1:
+                raise ValueError("%s: portion_multiple must be positive" % type(part).__name__)
+            multiple = multiple * n // math.gcd(multiple, n)
+        return multiple
 
     def graph_safe(self):
         """Whether every part's forward may be captured in a HIP graph (no

@@ -7,7 +7,7 @@ embedding when `tie_word_embeddings` is set."""
 from ..config.model_config import ModelConfig
 from ..config.registry import register_architecture
 from ..parts.base import PartSpec
-from .spec import LayerSpec, ModelSpec, RunStep
+from .spec import ModelSpec, RunStep, pre_norm_layer
 
 
 def qwen3_spec(config):
@@ -26,8 +26,8 @@ def qwen3_spec(config):
         "feed_forward", "swiglu",
         hidden_size=config.hidden_size, intermediate_size=config.intermediate_size)
     layers = tuple(
-        LayerSpec(prefix="model.layers.%d" % i, mixer=mixer, feed_forward=feed_forward,
-                  mixer_norm=norm, feed_forward_norm=norm)
+        pre_norm_layer("model.layers.%d" % i, mixer=mixer, feed_forward=feed_forward,
+                       mixer_norm=norm, feed_forward_norm=norm)
         for i in range(config.num_hidden_layers)
     )
     tied = config.tie_word_embeddings

@@ -302,7 +302,7 @@ def rope_table(inv_freq, max_positions):
 def qk_norm_rope_store(qkv, num_q_heads, num_kv_heads, head_dim, positions, seq_index,
                        q_weight=None, k_weight=None, eps=0.0, table=None,
                        block_table=None, k_cache=None, v_cache=None,
-                       cu_seqlens_q=None, kv_lens=None, max_q_len=0):
+                       cu_seqlens_q=None, kv_lens=None, max_q_len=0, max_kv_len=0):
     """Per-head RMSNorm of q and k, rotation by position, and the cache write, in one pass.
 
     qkv (T, (Hq + 2 Hkv) D) holds [q heads | k heads | v heads]. q heads are
@@ -318,7 +318,9 @@ def qk_norm_rope_store(qkv, num_q_heads, num_kv_heads, head_dim, positions, seq_
     describe the step's sequences; with them, bfloat16 steps use kernels with
     16-byte accesses that write values page by page. positions must then be
     kv_lens[b] - q_len[b] + i for row i of sequence b, as the step function
-    makes them.
+    makes them. `max_kv_len`: the step's last position + 1, if the caller knows it;
+    a step that passes the end of the rotation table is refused (a position
+    the table does not hold would go without its rotation).
     """
     _dev(qkv, positions, seq_index, q_weight, k_weight, table, block_table, k_cache, v_cache,
          cu_seqlens_q, kv_lens)
@@ -347,6 +349,8 @@ def qk_norm_rope_store(qkv, num_q_heads, num_kv_heads, head_dim, positions, seq_
         _need(table.dim() == 2 and table.dtype == torch.float32, "table must be float32 (P, R)")
         max_pos, rotary_dim = table.shape
         _need(rotary_dim % 2 == 0 and rotary_dim <= D, "rotary dim must be even and at most D")
+        _need(max_kv_len <= max_pos, "the step reaches position %d, the rotation table ends at %d"
+              % (max_kv_len - 1, max_pos - 1))
     page, stride = 0, 0
     if k_cache is not None:
         _need(v_cache is not None and block_table is not None, "a cache needs k, v and a block table")
@@ -363,7 +367,8 @@ def qk_norm_rope_store(qkv, num_q_heads, num_kv_heads, head_dim, positions, seq_
             _ptr(block_table), stride, 0 if block_table is None else block_table.shape[0],
             _ptr(k_cache), _ptr(v_cache), page, 0 if k_cache is None else k_cache.shape[0],
             T, Hq, Hkv, D, _DT[qkv.dtype], _ptr(cu_seqlens_q), _ptr(kv_lens),
-            0 if kv_lens is None else kv_lens.shape[0], int(max_q_len), _stream()), "qk_norm_rope_store")
+            0 if kv_lens is None else kv_lens.shape[0], int(max_q_len), int(max_kv_len), _stream()),
+            "qk_norm_rope_store")
     return qkv
 
 
@@ -482,6 +487,8 @@ def decode_attention(qkv, num_q_heads, num_kv_heads, head_dim, k_cache, v_cache,
     if table is not None:
         _need(table.dtype == torch.float32 and table.dim() == 2, "rotation table float32 (positions, rotary_dim)")
         max_pos, rotary_dim = table.shape
+        _need(max_kv_len <= max_pos, "the step reaches position %d, the rotation table ends at %d"
+              % (max_kv_len - 1, max_pos - 1))
     _need(decode_attention_takes(Hq, Hkv, D, page, qkv.dtype, rotary_dim), "sizes the decoding kernel does not take")
     out = torch.empty((B, Hq * D), dtype=qkv.dtype, device=qkv.device)
     if B:
@@ -495,7 +502,8 @@ def decode_attention(qkv, num_q_heads, num_kv_heads, head_dim, k_cache, v_cache,
             _ptr(qkv), _ptr(out), _ptr(k_cache), _ptr(v_cache), k_cache.shape[0], _ptr(block_table),
             block_table.shape[1], _ptr(cu_seqlens_q), _ptr(kv_lens), B, Hq, Hkv, D, page, ctypes.c_float(scale),
             int(window), splits, _ptr(workspace), _ptr(q_weight), _ptr(k_weight), w_dtype, ctypes.c_float(eps),
-            _ptr(table), int(rotary_dim), int(max_pos), 1 if store else 0, _stream()), "decode_attention")
+            _ptr(table), int(rotary_dim), int(max_pos), 1 if store else 0, int(max_kv_len), _stream()),
+            "decode_attention")
     return out
 
 

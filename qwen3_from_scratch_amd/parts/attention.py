@@ -4,8 +4,18 @@ import torch
 
 from .. import ops
 from ..config.registry import register_part
-from .base import CacheNeed, Part, TensorShape
+from .base import CacheNeed, PagedTensor, Part, TensorShape
 from .linear import LinearWeight
+
+
+def keys_and_values(kv_heads, head_dim, window=0):
+    """What softmax attention keeps in pages, as its kernels read it: a page of keys is
+    (kv_heads, page, head_dim), one head's keys contiguous, so a workgroup that serves one key
+    head streams page * head_dim elements at a time; a page of values is (kv_heads, head_dim,
+    page), transposed within the page, so that the values a matrix-core lane multiplies
+    together lie side by side in memory and need no transposition on the way to the registers."""
+    return CacheNeed(paged=(PagedTensor("keys", (kv_heads, head_dim), token_axis=1),
+                            PagedTensor("values", (kv_heads, head_dim), token_axis=2)), window=int(window))
 
 
 @register_part("mixer", "paged_attn")        # the reference's name for this component (models/self_attn.py:300)
@@ -51,7 +61,7 @@ class PagedAttention(Part):
         self.position = position
 
     def cache_need(self):
-        return CacheNeed(kv_heads=self.num_kv_heads, head_dim=self.head_dim, window=self.window)
+        return keys_and_values(self.num_kv_heads, self.head_dim, self.window)
 
     def tensors(self):
         H, Hq, Hkv, D = self.hidden_size, self.num_heads, self.num_kv_heads, self.head_dim
@@ -86,12 +96,13 @@ class PagedAttention(Part):
     def forward(self, x, batch, cache, sink=None):
         Hq, Hkv, D = self.num_heads, self.num_kv_heads, self.head_dim
         qkv = self.qkv.forward(x)
+        keys, values = cache.paged["keys"], cache.paged["values"]
         table = self.position.rotation_table() if self.position is not None else None
         if batch.max_q_len == 1 and qkv.shape[0] == batch.kv_lens.shape[0] and ops.decode_attention_takes(
-                Hq, Hkv, D, cache.keys.shape[2], qkv.dtype, 0 if table is None else table.shape[1]):
+                Hq, Hkv, D, keys.shape[2], qkv.dtype, 0 if table is None else table.shape[1]):
             # every sequence brings one token: preparation, cache write and attention are one kernel
             o = ops.decode_attention(
-                qkv, Hq, Hkv, D, cache.keys, cache.values, cache.block_table, batch.cu_seqlens_q, batch.kv_lens,
+                qkv, Hq, Hkv, D, keys, values, cache.block_table, batch.cu_seqlens_q, batch.kv_lens,
                 batch.max_kv_len, self.scale, window=self.window, q_weight=self.q_weight, k_weight=self.k_weight,
                 eps=self.qk_norm_eps, table=table, store=cache.writes)
             return self.out.forward(o) if sink is None else self.out.forward_into(o, sink)
@@ -99,13 +110,14 @@ class PagedAttention(Part):
             qkv, Hq, Hkv, D, batch.positions, batch.seq_index,
             q_weight=self.q_weight, k_weight=self.k_weight, eps=self.qk_norm_eps, table=table,
             block_table=cache.block_table if cache.writes else None,
-            k_cache=cache.keys if cache.writes else None,
-            v_cache=cache.values if cache.writes else None,
+            k_cache=keys if cache.writes else None,
+            v_cache=values if cache.writes else None,
             cu_seqlens_q=batch.cu_seqlens_q, kv_lens=batch.kv_lens, max_q_len=batch.max_q_len,
+            max_kv_len=batch.max_kv_len,
         )
         q = qkv[:, : Hq * D].unflatten(1, (Hq, D))
         o = ops.paged_attention(
-            q, Hq, cache.keys, cache.values, cache.block_table, batch.cu_seqlens_q, batch.kv_lens,
+            q, Hq, keys, values, cache.block_table, batch.cu_seqlens_q, batch.kv_lens,
             batch.max_q_len, batch.max_kv_len, self.scale, window=self.window,
             min_q_len=batch.min_q_len, max_kv_len_of_many=getattr(batch, "max_kv_len_portions", None),
         )

@@ -85,6 +85,10 @@ class Part:
     # takes `sink=`, and whether it takes UnscaledRows for its input
     feeds_sink = False
     takes_unscaled = False
+    # a part that works on a request's tokens in runs of fixed length (a mixer that keeps its
+    # state per run of N tokens, say) sets N here: the scheduler then cuts every portion of a
+    # prompt except its last to a multiple of N. The step function itself takes any cut.
+    portion_multiple = 1
 
     def __init__(self, prefix, precision, device):
         self.prefix = prefix
@@ -142,26 +146,77 @@ def build_part(spec, prefix, precision, device):
     return cls(prefix=prefix, precision=precision, device=device, **dict(spec.params))
 
 
-@dataclass
+@dataclass(frozen=True)
+class PagedTensor:
+    """One tensor that a mixer keeps in pages: every token adds one element of `shape` to it.
+
+    A page of it holds `page_size` tokens and is shaped shape[:token_axis] + (page_size,) +
+    shape[token_axis:], so the mixer says where in a page the tokens' axis stands: 0 puts a
+    token's numbers side by side, the last place puts the same number of consecutive tokens
+    side by side. `dtype`: None for the engine's activation dtype. The mixer finds the tensor
+    under `name` in its view of the cache (`LayerCacheView.paged[name]`, shaped (pages, *page))."""
+
+    name: str
+    shape: tuple
+    token_axis: int = 0
+    dtype: object = None
+
+    def __post_init__(self):
+        object.__setattr__(self, "shape", tuple(int(n) for n in self.shape))
+        if not self.shape or min(self.shape) <= 0:
+            raise ValueError("paged tensor %r: a token's shape needs positive sizes, found %r" % (self.name, self.shape))
+        if not 0 <= self.token_axis <= len(self.shape):
+            raise ValueError("paged tensor %r: token_axis %d is outside 0..%d"
+                             % (self.name, self.token_axis, len(self.shape)))
+
+    def page_shape(self, page_size):
+        return self.shape[:self.token_axis] + (int(page_size),) + self.shape[self.token_axis:]
+
+    def numbers_per_token(self):
+        n = 1
+        for size in self.shape:
+            n *= size
+        return n
+
+
+@dataclass(frozen=True)
 class CacheNeed:
     """What a mixer keeps per request between steps.
 
-    paged: keys and values that grow by one row per token, (kv_heads, head_dim)
-    each, all of them kept (window == 0) or the last `window`. state: a tensor
-    of fixed `state_shape` and `state_dtype` per request. A mixer may need
-    neither, either or both.
+    paged: the tensors that grow by one element per token (`PagedTensor`s: for softmax
+    attention a request's keys and values; another mixer may page one tensor, or tensors of
+    different widths), all tokens kept (window == 0) or the last `window`. state: a tensor of
+    fixed `state_shape` and `state_dtype` per request. A mixer may need neither, either or
+    both. Mixers whose needs are equal share page numbers: one block table serves them all.
     """
 
-    kv_heads: int = 0
-    head_dim: int = 0
+    paged: tuple = ()
     window: int = 0
     state_shape: tuple = ()
     state_dtype: torch.dtype = torch.float32
 
-    @property
-    def paged(self):
-        return self.kv_heads > 0
+    def __post_init__(self):
+        object.__setattr__(self, "paged", tuple(self.paged))
+        object.__setattr__(self, "state_shape", tuple(self.state_shape))
+        names = [t.name for t in self.paged]
+        if len(set(names)) != len(names):
+            raise ValueError("paged tensors of one mixer need different names, found %r" % (names,))
 
     @property
     def has_state(self):
         return len(self.state_shape) > 0
+
+    def bytes_per_token(self, act_dtype):
+        """Bytes that one token adds to one layer's pages."""
+        total = 0
+        for t in self.paged:
+            total += t.numbers_per_token() * torch.empty((), dtype=t.dtype or act_dtype).element_size()
+        return total
+
+    def bytes_of_state(self):
+        if not self.has_state:
+            return 0
+        n = torch.empty((), dtype=self.state_dtype).element_size()
+        for size in self.state_shape:
+            n *= size
+        return n

@@ -28,6 +28,8 @@ class PreNormBlock(Part):
         self.mixer = self.feed_forward = self.mixer_norm = self.feed_forward_norm = None
 
     def attach(self, mixer, feed_forward, mixer_norm, feed_forward_norm):
+        """The layer's parts, under the names its LayerSpec gave them: a block's `attach` names
+        the parts it arranges as its keywords, and a layer that brings others does not build."""
         self.mixer = mixer
         self.feed_forward = feed_forward
         self.mixer_norm = mixer_norm

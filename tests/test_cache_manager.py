@@ -8,6 +8,7 @@ import torch
 
 from qwen3_from_scratch_amd.cache import CacheManager, OutOfPages, PagePool
 from qwen3_from_scratch_amd.parts import CacheNeed
+from qwen3_from_scratch_amd.parts.attention import keys_and_values
 
 
 def test_pool_refuses_double_free_and_overdraw():
@@ -26,7 +27,7 @@ def test_pool_refuses_double_free_and_overdraw():
 
 def test_pages_follow_the_references_arithmetic():
     # test/inference/test_block_manager.py:9-97, block size 16
-    m = CacheManager([CacheNeed(kv_heads=2, head_dim=8)], page_size=16, num_pages=2, max_requests=4)
+    m = CacheManager([keys_and_values(2, 8)], page_size=16, num_pages=2, max_requests=4)
     assert not m.can_grow("a", 33)               # 33 tokens need 3 pages, 2 exist
     assert m.can_grow("a", 32)
     m.admit("a")
@@ -45,7 +46,7 @@ def test_pages_follow_the_references_arithmetic():
 
 
 def test_reserve_is_all_or_nothing_across_groups():
-    needs = [CacheNeed(2, 8), CacheNeed(2, 8, window=16), CacheNeed(2, 8)]
+    needs = [keys_and_values(2, 8), keys_and_values(2, 8, window=16), keys_and_values(2, 8)]
     m = CacheManager(needs, page_size=8, num_pages=4, max_requests=2)
     assert len(m.groups) == 2 and m.groups[0].planes == [0, 2] and m.groups[1].planes == [1]
     m.admit("a")
@@ -59,7 +60,7 @@ def test_reserve_is_all_or_nothing_across_groups():
 
 
 def test_window_gives_pages_back_as_it_passes_them():
-    m = CacheManager([CacheNeed(1, 8, window=20)], page_size=8, num_pages=6, max_requests=1)
+    m = CacheManager([keys_and_values(1, 8, window=20)], page_size=8, num_pages=6, max_requests=1)
     m.admit("w")
     length = 0
     for n in [5, 9, 1, 1, 30, 2]:
@@ -95,7 +96,7 @@ def test_state_slots_are_unique_and_come_back():
 @pytest.mark.parametrize("seed", range(6))
 def test_random_orders_lose_nothing(seed):
     rng = random.Random(seed)
-    needs = [CacheNeed(2, 16), CacheNeed(2, 16, window=rng.choice([9, 24, 40])), CacheNeed(2, 16)]
+    needs = [keys_and_values(2, 16), keys_and_values(2, 16, window=rng.choice([9, 24, 40])), keys_and_values(2, 16)]
     page = rng.choice([4, 8, 16])
     m = CacheManager(needs, page_size=page, num_pages=rng.randint(6, 20), max_requests=4)
     live, counter = {}, 0
@@ -148,7 +149,7 @@ def _run(m, rid, tokens, register=True):
 
 
 def test_prefix_blocks_are_shared_counted_and_kept_after_their_holders():
-    m = CacheManager([CacheNeed(2, 8), CacheNeed(4, 16)], page_size=4, num_pages=10, max_requests=4, prefix_cache=True)
+    m = CacheManager([keys_and_values(2, 8), keys_and_values(4, 16)], page_size=4, num_pages=10, max_requests=4, prefix_cache=True)
     assert m.prefix_cache and len(m.groups) == 2
     a = list(range(100, 111))                     # 11 tokens: two full blocks and three tokens
     assert _run(m, "a", a) == 0
@@ -173,7 +174,7 @@ def test_prefix_blocks_are_shared_counted_and_kept_after_their_holders():
 
 
 def test_prefix_nodes_are_forgotten_oldest_first_when_pages_run_out():
-    m = CacheManager([CacheNeed(2, 8)], page_size=4, num_pages=6, max_requests=3, prefix_cache=True)
+    m = CacheManager([keys_and_values(2, 8)], page_size=4, num_pages=6, max_requests=3, prefix_cache=True)
     first, second = list(range(10, 18)), list(range(50, 58))
     _run(m, "a", first + [1])
     m.release("a")                                # two idle nodes (and a private page that went back)
@@ -198,10 +199,10 @@ def test_prefix_nodes_are_forgotten_oldest_first_when_pages_run_out():
 
 
 def test_prefix_index_stays_off_for_windows_and_state():
-    assert not CacheManager([CacheNeed(2, 8, window=16)], 4, 8, 2, prefix_cache=True).prefix_cache
-    assert not CacheManager([CacheNeed(2, 8), CacheNeed(state_shape=(3,), state_dtype=torch.float32)], 4, 8, 2,
+    assert not CacheManager([keys_and_values(2, 8, window=16)], 4, 8, 2, prefix_cache=True).prefix_cache
+    assert not CacheManager([keys_and_values(2, 8), CacheNeed(state_shape=(3,), state_dtype=torch.float32)], 4, 8, 2,
                             prefix_cache=True).prefix_cache
-    m = CacheManager([CacheNeed(2, 8)], 4, 8, 2)
+    m = CacheManager([keys_and_values(2, 8)], 4, 8, 2)
     assert not m.prefix_cache
     m.admit("a")
     assert m.share_prefix("a", list(range(9))) == 0
@@ -212,7 +213,7 @@ def test_prefix_index_stays_off_for_windows_and_state():
 @pytest.mark.parametrize("seed", range(6))
 def test_random_orders_with_shared_prefixes_lose_nothing(seed):
     rng = random.Random(seed)
-    m = CacheManager([CacheNeed(2, 8), CacheNeed(1, 16)], page_size=4, num_pages=24, max_requests=5, prefix_cache=True)
+    m = CacheManager([keys_and_values(2, 8), keys_and_values(1, 16)], page_size=4, num_pages=24, max_requests=5, prefix_cache=True)
     stems = [[rng.randrange(5) for _ in range(rng.randrange(4, 20))] for _ in range(3)]
     live = {}                                     # rid -> (tokens, computed)
     count = 0

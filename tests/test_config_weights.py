@@ -65,9 +65,9 @@ def test_spec_is_data_and_sizes_come_from_the_config():
     cfg = tiny_config("B")
     spec = qwen3_spec(cfg)
     assert len(spec.layers) == cfg.num_hidden_layers and [s.layer for s in spec.order] == [0, 1, 2]
-    mixer = spec.layers[1].mixer
+    mixer = spec.layers[1].slot("mixer").part
     assert mixer.get("num_heads") == 8 and mixer.get("num_kv_heads") == 2 and mixer.get("head_dim") == 32
-    assert spec.layers[0].mixer_norm.get("eps") == 1e-5 and spec.position.get("theta") == 1e6
+    assert spec.layers[0].slot("mixer_norm").part.get("eps") == 1e-5 and spec.position.get("theta") == 1e6
     names = expected_tensors(spec)
     assert names["model.layers.2.self_attn.q_proj.weight"] == (256, 96)
     assert names["model.layers.0.self_attn.k_norm.weight"] == (32,)

@@ -214,3 +214,56 @@ def test_trace_run_answers_step_by_step(model_folders, tmp_path):
     finally:
         if proc.poll() is None:
             proc.kill()
+
+
+def _run(arguments, timeout=300):
+    proc = subprocess.run([sys.executable] + arguments, capture_output=True, text=True, timeout=timeout, cwd=ROOT)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    return proc.stdout
+
+
+def test_the_command_line_and_the_examples_as_a_user_runs_them(tmp_path):
+    """`python -m qwen3_from_scratch_amd` writes a random-weights folder and generates from it,
+    and the two example scripts run on that folder, each as a process of its own on the GPU;
+    with float32 and temperature 0 the ids they print are the plain implementation's."""
+    config = tmp_path / "config.json"
+    config.write_text(json.dumps(TINY["D"]["config"]))
+    folder = str(tmp_path / "model")
+    module = ["-m", "qwen3_from_scratch_amd"]
+    assert "wrote" in _run(module + ["--write_random", folder, "--from_config", str(config), "--seed", "3",
+                                     "--std", "0.05"])
+    cfg, w = plain_qwen3.read_model_folder(folder)
+
+    def plain(prompt, n):
+        return plain_qwen3.greedy_generate(cfg, w, prompt, n)
+
+    greedy = ["--dtype", "float32", "--temperature", "0"]
+    out = _run(module + ["--path", folder, "--prompt_ids", "5,17,3", "--max_new_tokens", "8", "--ignore_eos"] + greedy)
+    want = plain([5, 17, 3], 8)
+    assert [int(t) for t in out.split()] == want
+    # a stop token on the command line: generation ends with its first occurrence
+    out = _run(module + ["--path", folder, "--prompt_ids", "5,17,3", "--max_new_tokens", "8", "--eos_id", str(want[3])]
+               + greedy)
+    assert [int(t) for t in out.split()] == want[:want.index(want[3]) + 1]
+    out = _run(module + ["--path", folder, "--prompt_ids", "5,17,3", "--prompt_ids", "9,9", "--max_new_tokens", "5",
+                         "--ignore_eos"] + greedy)
+    assert [[int(t) for t in line.split()] for line in out.strip().split("\n")] == [plain([5, 17, 3], 5), plain([9, 9], 5)]
+
+    out = _run([os.path.join(ROOT, "examples", "sync_engine_example.py"), "--path", folder, "--max_new_tokens", "6"]
+               + greedy)
+    lines = out.split("\n")
+    streamed = lines[lines.index("=== one request, streamed ===") + 1]
+    assert [int(t) for t in streamed.split()] == plain([5, 17, 3, 9], 6)
+    whole = lines[lines.index("=== one request, whole ===") + 1]
+    assert [int(t) for t in whole.split()] == plain([2, 4, 6], 6)
+    batch = [l[2:] for l in lines if l.startswith("- ")]
+    assert [[int(t) for t in l.split()] for l in batch] == [plain(p, 6) for p in ([5, 17, 3], [2, 4, 6, 8], [9])]
+    assert any(l.startswith("requests: 3 | tokens: 18") for l in lines)
+
+    out = _run([os.path.join(ROOT, "examples", "llm_runner.py"), "--path", folder, "--max_new_tokens", "6"] + greedy)
+    for tag, prompt in (("req0", [5, 17, 3, 9]), ("req1", [2, 4, 6])):
+        ids = [int(l.split("]")[1]) for l in out.split("\n") if l.startswith("[%s]" % tag)]
+        assert ids == plain(prompt, 6), tag
+    # the default precision and sampling run too
+    assert len(_run(module + ["--path", folder, "--prompt_ids", "5,17,3", "--max_new_tokens", "8", "--seed", "2",
+                              "--ignore_eos"]).split()) == 8

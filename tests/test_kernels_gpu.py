@@ -163,7 +163,7 @@ def _paged_case(dtype, B, Hq, Hkv, D, page, q_lens, kv_lens, seed, spread=True):
     W = max(-(-L // page) for L in kv_lens) + 1
     npages = B * W + 3
     perm = torch.randperm(npages, generator=g)[: B * W].view(B, W).to(torch.int32)
-    for b in range(B):                                    # -1 padding beyond the last page is never read
+    for b in range(B):      # entries beyond the last page: the kernels may read them, but never the pages they name
         perm[b, -(-kv_lens[b] // page):] = -1
     kc = (torch.randn((npages, Hkv, page, D), generator=g)).to(dtype).cuda()
     vc = (torch.randn((npages, Hkv, D, page), generator=g)).to(dtype).cuda()   # values: transposed in the page
@@ -258,6 +258,83 @@ def test_decode_attention_is_its_two_halves(Hq, Hkv, D, page, w_dtype, window, r
     ref = torch_ops.paged_attention(q.float(), Hq, k1.float(), v1.float(), bt, cu, kvl, 1, max(kv_lens), scale,
                                     window=window)
     torch.testing.assert_close(got.float().view(B, Hq, D), ref.view(B, Hq, D), rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("Hq,Hkv,D,page", [(32, 8, 128, 16), (8, 2, 64, 32)])
+@pytest.mark.parametrize("kv_lens", [[1, 17, 40, 64, 65], [700, 2500, 3]])
+def test_nothing_past_a_sequences_end_is_read_into_the_result(Hq, Hkv, D, page, kv_lens):
+    """Block tables that list real pages beyond a sequence's last one (a table that a graph
+    keeps from a longer step, a page taken ahead), and slots at and past the sequence's end that
+    hold NaN in keys and values, the slot the fused kernel writes among them: the decoding
+    kernels look at whole tiles and whole tables before they know the length, and must mask
+    what lies past it. One split and many, with and without a window."""
+    ops = _ops()
+    B = len(kv_lens)
+    _, kc, vc, bt, cu, kvl = _paged_case(torch.bfloat16, B, Hq, Hkv, D, page, [1] * B, kv_lens, 91)
+    W = bt.shape[1]
+    spare = iter(sorted(set(range(kc.shape[0])) - set(bt[bt >= 0].tolist())) * W)
+    clean_k, clean_v = kc.clone(), vc.clone()
+    for b, L in enumerate(kv_lens):
+        used = -(-L // page)
+        for j in range(used, W):                      # real pages listed past the end, full of NaN
+            pg = next(spare)
+            bt[b, j] = pg
+            kc[pg], vc[pg] = float("nan"), float("nan")
+        last = int(bt[b, used - 1])
+        first_free = (L - 1) % page                   # the new token's slot, and all slots after it
+        kc[last, :, first_free:], vc[last, :, :, first_free:] = float("nan"), float("nan")
+        clean_k[last, :, first_free:], clean_v[last, :, :, first_free:] = 0.0, 0.0
+    qkv = _rand((B, (Hq + 2 * Hkv) * D), torch.bfloat16, 92, scale=1.5)
+    inv_freq = (1.0 / (10000.0 ** (torch.arange(0, D, 2, dtype=torch.float32) / D))).cuda()
+    table = ops.rope_table(inv_freq, 4096)
+    scale = D ** -0.5
+    for window in (0, 50):
+        k2, v2 = kc.clone(), vc.clone()
+        got = ops.decode_attention(qkv.clone(), Hq, Hkv, D, k2, v2, bt, cu, kvl, max(kv_lens), scale, window=window,
+                                   table=table)
+        k1, v1, qkv1 = clean_k.clone(), clean_v.clone(), qkv.clone()
+        ops.qk_norm_rope_store(qkv1, Hq, Hkv, D, (kvl - 1).to(torch.int32), torch.arange(B, dtype=torch.int32).cuda(),
+                               table=table, block_table=bt, k_cache=k1, v_cache=v1, cu_seqlens_q=cu, kv_lens=kvl,
+                               max_q_len=1)
+        q = qkv1[:, : Hq * D].unflatten(1, (Hq, D))
+        want = torch_ops.paged_attention(q.float(), Hq, k1.float(), v1.float(), bt, cu, kvl, 1, max(kv_lens), scale,
+                                         window=window)
+        assert torch.isfinite(got.float()).all(), window
+        torch.testing.assert_close(got.float().view(B, Hq, D), want.view(B, Hq, D), rtol=2e-2, atol=2e-2)
+        # the two-kernel path over the same poisoned caches (the new key and value written first)
+        k3, v3 = kc.clone(), vc.clone()
+        ops.qk_norm_rope_store(qkv.clone(), Hq, Hkv, D, (kvl - 1).to(torch.int32),
+                               torch.arange(B, dtype=torch.int32).cuda(), table=table, block_table=bt, k_cache=k3,
+                               v_cache=v3, cu_seqlens_q=cu, kv_lens=kvl, max_q_len=1)
+        again = ops.paged_attention(q, Hq, k3, v3, bt, cu, kvl, 1, max(kv_lens), scale, window=window)
+        assert torch.isfinite(again.float()).all(), window
+        torch.testing.assert_close(again.float().view(B, Hq, D), want.view(B, Hq, D), rtol=2e-2, atol=2e-2)
+
+
+def test_a_step_past_the_rotation_table_is_refused():
+    """A position that the rotation table does not hold would go without its rotation: the
+    operations refuse a step whose last position the caller says lies beyond the table."""
+    ops = _ops()
+    Hq, Hkv, D, page = 4, 2, 64, 16
+    _, kc, vc, bt, cu, kvl = _paged_case(torch.bfloat16, 2, Hq, Hkv, D, page, [1, 1], [40, 41], 5)
+    qkv = _rand((2, (Hq + 2 * Hkv) * D), torch.bfloat16, 6)
+    table = ops.rope_table((1.0 / (10000.0 ** (torch.arange(0, D, 2, dtype=torch.float32) / D))).cuda(), 40)
+    positions, seq = torch.tensor([39, 40], dtype=torch.int32).cuda(), torch.tensor([0, 1], dtype=torch.int32).cuda()
+    with pytest.raises(ValueError, match="rotation table ends at 39"):
+        ops.qk_norm_rope_store(qkv, Hq, Hkv, D, positions, seq, table=table, block_table=bt, k_cache=kc, v_cache=vc,
+                               cu_seqlens_q=cu, kv_lens=kvl, max_q_len=1, max_kv_len=41)
+    with pytest.raises(ValueError, match="rotation table ends at 39"):
+        ops.decode_attention(qkv, Hq, Hkv, D, kc, vc, bt, cu, kvl, 41, D ** -0.5, table=table)
+    # the launchers say the same to a caller that comes without the wrappers
+    import ctypes
+
+    from qwen3_from_scratch_amd.ops.build import library
+
+    status = library("rotary").q3_qk_norm_rope_store(
+        ctypes.c_void_p(qkv.data_ptr()), None, None, 0, ctypes.c_float(0.0), ctypes.c_void_p(table.data_ptr()), D, 40,
+        ctypes.c_void_p(positions.data_ptr()), ctypes.c_void_p(seq.data_ptr()), None, 0, 0, None, None, 0, 0,
+        2, Hq, Hkv, D, 1, None, None, 0, 0, 41, None)
+    assert status != 0
 
 
 @pytest.mark.parametrize("q_lens,kv_lens", [([512, 1, 100, 3, 33], [512, 900, 1100, 64, 2000]),
@@ -477,7 +554,8 @@ def test_the_table_decides_a_size():
     N, K = 1184, 640
     w = _rand((N, K), torch.bfloat16, 45, scale=0.05)
     rows = ops.matmul_rows_key("plain", 200)
-    assert rows == 224 and ops.matmul_rows_key("plain", 50) == 50 and ops.matmul_rows_key("scaled", 50) == 56
+    assert rows == 224 and ops.matmul_rows_key("plain", 50) == 56 and ops.matmul_rows_key("scaled", 50) == 56
+    assert ops.matmul_rows_key("plain", 17) == 24 and ops.matmul_rows_key("plain", 64) == 64
     try:
         ops.matmul_table([{"kind": "plain", "rows": rows, "N": N, "K": K, "own": 1, "splits": 2},
                           {"kind": "plain", "rows": rows, "N": N, "K": K, "out": "float32", "library": 1},
@@ -496,6 +574,12 @@ def test_the_table_decides_a_size():
         x3, w3 = _rand((64, 72), torch.bfloat16, 57), _rand((96, 72), torch.bfloat16, 58, scale=0.05)
         torch.testing.assert_close(ops.linear(x3, w3, out_dtype=torch.float32).double(), x3.double() @ w3.double().T,
                                    rtol=2e-3, atol=2e-3)
+        # an entry that names a place the library's list for this size does not reach: its first candidate
+        ops.matmul_table([{"kind": "plain", "rows": 320, "N": N, "K": K, "library": 63}])
+        x4 = _rand((300, K), torch.bfloat16, 59)
+        torch.testing.assert_close(ops.linear(x4, w).double(), x4.double() @ w.double().T, rtol=2e-2, atol=2e-2)
+        offered = ops.matmul_plan(300, N, K)
+        assert offered[4] == -1 and offered[6] in (0, 63)
     finally:
         import json
         with open(ops.TABLE_FILE) as fh:

@@ -8,12 +8,12 @@ import pytest
 
 from qwen3_from_scratch_amd.cache import CacheManager
 from qwen3_from_scratch_amd.engine import Request, RequestStatus, Scheduler
-from qwen3_from_scratch_amd.parts import CacheNeed
+from qwen3_from_scratch_amd.parts.attention import keys_and_values
 from qwen3_from_scratch_amd.sampling import SamplingParams
 
 
 def make(num_pages, page=16, max_num_seqs=32, max_num_tokens=3000, chunk=512):
-    m = CacheManager([CacheNeed(2, 16)], page_size=page, num_pages=num_pages, max_requests=max(max_num_seqs, 1))
+    m = CacheManager([keys_and_values(2, 16)], page_size=page, num_pages=num_pages, max_requests=max(max_num_seqs, 1))
     return m, Scheduler(m, max_num_seqs, max_num_tokens, chunk)
 
 
@@ -205,7 +205,7 @@ def test_a_request_starts_behind_the_blocks_the_prefix_index_holds():
     request whose first blocks are cached is scheduled from behind them; a whole hit keeps its
     last block to compute; one that cannot get its remaining pages gives back what it took over
     and waits."""
-    m = CacheManager([CacheNeed(2, 16)], page_size=4, num_pages=8, max_requests=4, prefix_cache=True)
+    m = CacheManager([keys_and_values(2, 16)], page_size=4, num_pages=8, max_requests=4, prefix_cache=True)
     s = Scheduler(m, 4, 100, 100)
     s.add(Request("a", list(range(10)), SamplingParams(max_new_tokens=1)))
     plan = run_step(m, s)
@@ -229,3 +229,47 @@ def test_a_request_starts_behind_the_blocks_the_prefix_index_holds():
     assert [e.request.request_id for e in plan] == ["b", "c"] and s.waiting[0].computed == 0
     assert not m.has("d") and m.prefix_hits == before
     m.audit()
+
+
+def test_portions_end_at_multiples_that_a_part_asks_for():
+    """A part may ask that every portion of a prompt but the last be a multiple of N tokens
+    (`Part.portion_multiple`; the reference has no counterpart). Cuts are counted from the
+    request's first token, so a request that was preempted is cut at the same places again, and
+    whatever room decoding requests leave in the budget is rounded down, not overrun."""
+    m = CacheManager([keys_and_values(2, 16)], page_size=16, num_pages=64, max_requests=8)
+    s = Scheduler(m, max_num_seqs=8, max_num_tokens=100, chunked_prefill_size=50, portion_multiple=8)
+    a, b = req("a", 131, max_new=3), req("b", 45, max_new=3)
+    s.add(a)
+    s.add(b)
+    seen = {"a": [], "b": []}
+    for _ in range(20):
+        if not s.has_work():
+            break
+        for e in run_step(m, s):
+            if e.num_tokens > 1 or e.request.is_prefill:
+                seen[e.request.request_id].append(e.num_tokens)
+    assert not s.has_work()
+    # a: 48 (of 50), b: 45 whole (it fits in the 52 left); then a beside b's decoding: 48, then the last 35
+    assert seen["a"] == [48, 48, 35] and seen["b"] == [45]
+    for cuts in seen.values():
+        at = 0
+        for n in cuts[:-1]:
+            at += n
+            assert at % 8 == 0
+    # a budget that cannot hold one multiple is refused when the scheduler is made
+    with pytest.raises(ValueError):
+        Scheduler(m, max_num_seqs=8, max_num_tokens=100, chunked_prefill_size=6, portion_multiple=8)
+    # room smaller than a multiple beside decoding requests: the prompt waits a step, nothing is cut to less
+    m2 = CacheManager([keys_and_values(2, 16)], page_size=16, num_pages=64, max_requests=8)
+    s2 = Scheduler(m2, max_num_seqs=8, max_num_tokens=10, chunked_prefill_size=10, portion_multiple=8)
+    for i in range(3):
+        s2.add(req("d%d" % i, 2, max_new=30))
+    run_step(m2, s2)
+    s2.add(req("long", 30, max_new=2))
+    portions = []
+    for _ in range(40):
+        if not s2.has_work():
+            break
+        portions += [e.num_tokens for e in run_step(m2, s2) if e.request.request_id == "long" and e.request.computed <= 30
+                     and e.num_tokens > 1]
+    assert portions and all(n % 8 == 0 for n in portions[:-1]) and sum(portions) == 30

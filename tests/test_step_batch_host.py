@@ -13,6 +13,7 @@ from qwen3_from_scratch_amd.engine import StepEntry, pack_step
 from qwen3_from_scratch_amd.engine.batch import packed_layout
 from qwen3_from_scratch_amd.engine.runner import DecodeDescription, collector_paused, padded_batch
 from qwen3_from_scratch_amd.parts import CacheNeed
+from qwen3_from_scratch_amd.parts.attention import keys_and_values
 
 
 def _pack(entries, lengths, tables=None):
@@ -140,7 +141,7 @@ def test_a_patched_description_equals_a_fresh_one():
     """Growth across page ends, a windowed group whose entries turn -1, requests that leave a
     step out or end and come back under the same name, and batch sizes that share a row count."""
     rng = random.Random(3)
-    needs = [CacheNeed(2, 8), CacheNeed(2, 8, window=12), CacheNeed(2, 8)]
+    needs = [keys_and_values(2, 8), keys_and_values(2, 8, window=12), keys_and_values(2, 8)]
     d = _Decoding(needs, page_size=4, num_pages=200, max_requests=8, max_tokens=160)
     for i, n in enumerate([3, 9, 16, 1, 30, 7]):
         d.prompt("r%d" % i, n)

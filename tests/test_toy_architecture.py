@@ -1,8 +1,10 @@
 """An architecture defined in tests/toy_architecture.py, with config.json keys of its own, a
-mixer that keeps a state per request and, in its second example, a norm and a block arrangement
-of its own, goes through the framework's model folder writer, loader,
+mixer that keeps a state per request, in its second example a norm and a block arrangement
+of its own, and in its third a block with four norms, a mixer that pages one tensor of a width
+of its own and a layer without a feed-forward, goes through the framework's model folder writer, loader,
 cache manager, step function, engine and replay program without a change to the framework."""
 
+import dataclasses
 import json
 import os
 import subprocess
@@ -22,7 +24,7 @@ from qwen3_from_scratch_amd.weights import write_random_model
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-EXAMPLES = {"sequential": toy.EXAMPLE, "parallel": toy.EXAMPLE_PARALLEL}
+EXAMPLES = {"sequential": toy.EXAMPLE, "parallel": toy.EXAMPLE_PARALLEL, "sandwich": toy.EXAMPLE_SANDWICH}
 
 
 @pytest.fixture(scope="module", params=sorted(EXAMPLES))
@@ -79,6 +81,71 @@ def test_a_layer_with_a_position_part_of_its_own(folder):
     assert own[0].get("rotary_dim") == config.head_size // 2 and own[0] != spec.position
 
 
+def test_a_block_with_four_norms_a_paged_tensor_of_its_own_and_a_layer_without_feed_forward(cpu_ops, tmp_path):
+    """The third example's parts are declarations only: the layer says which parts its block
+    gets, the mixer says what it pages (one float32 tensor of 24 numbers a token, the last twelve
+    tokens kept), and the cache storage builds exactly that."""
+    config = toy.ToyHybridConfig.from_dict(toy.EXAMPLE_SANDWICH)
+    folder = write_random_model(str(tmp_path / "m"), config, seed=9, std=0.08, norm_jitter=0.2)
+    runner = load_runner(folder, dtype="float32", device="cpu", page_size=8, max_tokens=256, max_requests=4)
+    layers = runner.model.layers
+    kinds = dict(zip(config.pattern, layers))
+    assert set(kinds["p"].named) == {"mixer", "feed_forward", "mixer_norm", "mixer_out_norm", "feed_forward_norm",
+                                     "feed_forward_out_norm"}
+    assert set(kinds["n"].named) == {"mixer", "mixer_norm"}
+    names = set(load_file(os.path.join(folder, "model.safetensors")))
+    n_at = config.pattern.index("n")
+    assert "hybrid.layers.%d.post_mlp_norm.weight" % config.pattern.index("p") in names
+    assert not any(name.startswith("hybrid.layers.%d.mlp" % n_at) for name in names)
+    groups = runner.manager.groups
+    mine = [g for g in groups if [t.name for t in g.tensors] == ["memory"]]
+    assert len(mine) == 1 and mine[0].window == toy.LAG + 1 and len(mine[0].planes) == 2     # layers p and n
+    stored = runner.storage.paged[groups.index(mine[0])]["memory"]
+    assert stored.dtype == torch.float32 and stored.shape[2:] == (8, toy.MEMORY)
+    attention = [g for g in groups if [t.name for t in g.tensors] == ["keys", "values"]]
+    assert sorted(g.window for g in attention) == [0, config.window]
+    # pages behind the mixer's window go back while the request lives
+    from qwen3_from_scratch_amd.engine import StepEntry
+
+    tokens = random_tokens(100, config.vocab, 3)
+    for at in range(0, 100, 10):
+        runner.step([StepEntry("r", tokens[at:at + 10], [])])
+    table = runner.manager.block_table("r", groups.index(mine[0]))
+    assert table[:10] == [-1] * 10 and min(table[11:]) >= 0
+    # the storage is sized by what the parts declare
+    per_token = sum(n.bytes_per_token(torch.float32) for n in runner.model.plane_needs if n is not None)
+    assert per_token == 2 * (4 * toy.MEMORY) + 2 * (2 * 4 * config.kv_heads * config.head_size)
+
+
+def test_a_layers_own_position_table_bounds_a_request(cpu_ops, tmp_path):
+    """A position beyond a rotation table would go without its rotation; the step function bounds
+    a request by the shortest table among the model's and the layers' own, and the operation
+    itself refuses a step that passes the table it is given."""
+    from qwen3_from_scratch_amd.config import register_architecture
+    from qwen3_from_scratch_amd.engine import StepEntry
+
+    def short_table(c):
+        spec = toy.toy_hybrid_spec(c)
+        layers = tuple(dataclasses.replace(ls, position=ls.position.with_params(max_positions=40))
+                       if ls.position is not None else ls for ls in spec.layers)
+        return dataclasses.replace(spec, layers=layers)
+
+    register_architecture("ToyShortTableForCausalLM", toy.ToyHybridConfig, short_table)
+    config = toy.ToyHybridConfig.from_dict(dict(toy.EXAMPLE, architectures=["ToyShortTableForCausalLM"]))
+    folder = write_random_model(str(tmp_path / "m"), config, seed=9, std=0.08, norm_jitter=0.2)
+    runner = load_runner(folder, dtype="float32", device="cpu", page_size=8, max_tokens=256, max_requests=2)
+    assert runner.max_positions == 40 and runner.max_request_tokens == 40
+    runner.step([StepEntry("r", random_tokens(40, config.vocab, 1), [39])])
+    with pytest.raises(ValueError, match="position 39"):
+        runner.step([StepEntry("r", [5], [0])])
+    # the operation on its own: a table of 40 positions and a step that reaches position 40
+    D, table = 16, cpu_ops.rope_table(torch.ones(8), 40)
+    qkv = torch.zeros(3, 3 * D)
+    positions, seq = torch.tensor([38, 39, 40], dtype=torch.int32), torch.zeros(3, dtype=torch.int32)
+    with pytest.raises(ValueError, match="rotation table ends at 39"):
+        cpu_ops.qk_norm_rope_store(qkv, 1, 1, D, positions, seq, table=table, max_kv_len=41)
+
+
 def test_every_cutting_and_generation_on_the_host(cpu_ops, folder):
     requests = _requests(folder)
     config, w, want = _plain(folder, requests)
@@ -107,7 +174,7 @@ def test_cache_sizing_counts_the_states(cpu_ops, folder):
               gpu_utilization=3e-4)                       # of the gigabyte a host engine pretends to have
     few, many = SyncEngine(max_num_seqs=2, **kw), SyncEngine(max_num_seqs=40, **kw)
     needs = few.model.plane_needs
-    per_page = sum(2 * n.kv_heads * n.head_dim * 4 for n in needs if n is not None and n.paged) * 8
+    per_page = sum(n.bytes_per_token(torch.float32) for n in needs if n is not None) * 8
     per_request = sum(4 * int(np.prod(n.state_shape)) for n in needs if n is not None and n.has_state)
     assert per_request > 0
     budget = int((1 << 30) * 3e-4)

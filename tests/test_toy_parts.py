@@ -18,7 +18,7 @@ import plain_qwen3 as plain
 from helpers import max_live_tokens, random_tokens, run_trace, trace_mixed, trace_portions, trace_tail_decoded, trace_whole
 from qwen3_from_scratch_amd.config import register_part
 from qwen3_from_scratch_amd.engine import ModelRunner
-from qwen3_from_scratch_amd.models import DecoderModel, LayerSpec, ModelSpec, RunStep
+from qwen3_from_scratch_amd.models import DecoderModel, ModelSpec, RunStep, pre_norm_layer
 from qwen3_from_scratch_amd.parts import CacheNeed, Part, PartSpec, Precision
 from qwen3_from_scratch_amd.weights import RandomWeights
 
@@ -140,8 +140,8 @@ def toy_spec(position, with_state=True):
     routed = PartSpec.of("feed_forward", "toy_routed", hidden_size=H, intermediate_size=EXPERT_I, num_experts=EXPERTS)
 
     def layer(i, mixer):
-        return LayerSpec(prefix="toy.layers.%d" % i, mixer=mixer, feed_forward=routed if i == 2 else ff,
-                         mixer_norm=norm, feed_forward_norm=norm)
+        return pre_norm_layer("toy.layers.%d" % i, mixer=mixer, feed_forward=routed if i == 2 else ff,
+                              mixer_norm=norm, feed_forward_norm=norm)
 
     layers = (
         layer(0, PartSpec.of("mixer", "attention", window=0, **attn)),
@@ -175,7 +175,7 @@ def plain_toy_logits(w, spec, position, tokens):
         i = step.layer
         p = "toy.layers.%d" % i
         h = plain.rms_norm(x, w[p + ".input_layernorm.weight"], EPS)
-        mixer = spec.layers[i].mixer
+        mixer = spec.layers[i].slot("mixer").part
         if mixer.name == "toy_running_mean":
             mean = torch.cumsum(h, dim=0) / torch.arange(1, T + 1)[:, None]
             d = mean @ w[p + ".self_attn.mix.weight"].T
@@ -198,7 +198,7 @@ def plain_toy_logits(w, spec, position, tokens):
             d = o.reshape(T, HQ * D) @ w[a + ".o_proj.weight"].T
         x = x + d
         h = plain.rms_norm(x, w[p + ".post_attention_layernorm.weight"], EPS)
-        if spec.layers[i].feed_forward.name == "toy_routed":
+        if spec.layers[i].slot("feed_forward").part.name == "toy_routed":
             g = routing_weights(torch.softmax(h @ w[p + ".mlp.router.weight"].T, dim=-1))
             for e in range(EXPERTS):
                 up, down = w[p + ".mlp.experts.%d.up.weight" % e], w[p + ".mlp.experts.%d.down.weight" % e]

@@ -54,9 +54,12 @@ def rope_table(inv_freq, max_positions):
 def qk_norm_rope_store(qkv, num_q_heads, num_kv_heads, head_dim, positions, seq_index,
                        q_weight=None, k_weight=None, eps=0.0, table=None,
                        block_table=None, k_cache=None, v_cache=None,
-                       cu_seqlens_q=None, kv_lens=None, max_q_len=0):
+                       cu_seqlens_q=None, kv_lens=None, max_q_len=0, max_kv_len=0):
     Hq, Hkv, D = num_q_heads, num_kv_heads, head_dim
     T = qkv.shape[0]
+    if table is not None and max_kv_len > table.shape[0]:
+        raise ValueError("the step reaches position %d, the rotation table ends at %d"
+                         % (max_kv_len - 1, table.shape[0] - 1))
     x = qkv.view(T, Hq + 2 * Hkv, D).float()
     q, k, v = x[:, :Hq], x[:, Hq:Hq + Hkv], x[:, Hq + Hkv:]
 

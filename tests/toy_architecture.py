@@ -3,9 +3,13 @@ own configuration class, a function from that configuration to a ModelSpec, and 
 `register_architecture` call. Layers follow a pattern string: `a` is the framework's
 attention (with a window), `b` the same attention without a window and with a position part of
 its own (a rotation over the first half of each head only, by another base), `s` the
-running-mean mixer of test_toy_parts.py, which keeps a state of fixed size per request. Two more keys choose between the framework's RMS norm and a
-mean-subtracting norm with a bias defined here, and between the framework's sequential block
-and a block defined here whose mixer and feed-forward read the same stream. It is no model of anyone's; it shows that the loader, the
+running-mean mixer of test_toy_parts.py, which keeps a state of fixed size per request, `p` a
+mixer defined here that pages one tensor of a width of its own (a float32 vector per token, of
+which it reads the one `LAG` tokens back) and `n` a layer of that mixer alone, without a
+feed-forward. Two more keys choose between the framework's RMS norm and a
+mean-subtracting norm with a bias defined here, and between the framework's sequential block,
+a block defined here whose mixer and feed-forward read the same stream, and one with four norms
+(each part's result is normalised too before it is added). It is no model of anyone's; it shows that the loader, the
 random-weights writer, the cache manager, the step function, the engine and the replay
 program take an architecture they have never heard of.
 
@@ -22,11 +26,13 @@ import plain_qwen3 as plain
 import test_toy_parts  # registers the mixer "toy_running_mean"  # noqa: F401
 from qwen3_from_scratch_amd.config import register_architecture, register_part
 from qwen3_from_scratch_amd.config.model_config import ConfigError
-from qwen3_from_scratch_amd.models import LayerSpec, ModelSpec, RunStep
-from qwen3_from_scratch_amd.parts import Part, PartSpec, TensorShape
+from qwen3_from_scratch_amd.models import LayerSpec, ModelSpec, RunStep, Slot, pre_norm_layer
+from qwen3_from_scratch_amd.parts import CacheNeed, PagedTensor, Part, PartSpec, TensorShape
 
 NAME = "ToyHybridForCausalLM"
 OTHER_BASE = 7.0     # a `b` layer rotates by theta / 7
+LAG = 11             # a `p` or `n` layer multiplies a token's vector with the one of the token 11 back
+MEMORY = 24          # the width of that vector
 KEYS = (("vocab", int), ("width", int), ("inner", int), ("heads", int), ("kv_heads", int), ("head_size", int),
         ("pattern", str), ("window", int), ("eps", float), ("theta", float), ("max_position_embeddings", int),
         ("norm", str), ("arrangement", str))
@@ -85,6 +91,89 @@ class ParallelBlock(Part):
         return x, mixed.float() + self.feed_forward.forward(h2, batch).float()
 
 
+@register_part("block", "toy_sandwich")
+class SandwichBlock(Part):
+    """x = x + norm_2(mixer(norm_1(x))); x = x + norm_4(feed_forward(norm_3(x))): four norms a
+    layer, two of them on what the parts return."""
+
+    def __init__(self, prefix, precision, device):
+        super().__init__(prefix, precision, device)
+
+    def attach(self, mixer, feed_forward, mixer_norm, mixer_out_norm, feed_forward_norm, feed_forward_out_norm):
+        self.mixer, self.feed_forward = mixer, feed_forward
+        self.norms = (mixer_norm, mixer_out_norm, feed_forward_norm, feed_forward_out_norm)
+
+    def forward(self, x, pending, batch, cache, next_norm=None):
+        n1, n2, n3, n4 = self.norms
+        mixed = self.mixer.forward(n1.forward(x, delta=pending), batch, cache)
+        fed = self.feed_forward.forward(n3.forward(x, delta=n2.forward(mixed.float())), batch)
+        return x, n4.forward(fed.float())
+
+
+@register_part("block", "toy_mixer_only")
+class MixerOnlyBlock(Part):
+    """x = x + mixer(norm(x)): a layer without a feed-forward."""
+
+    def __init__(self, prefix, precision, device):
+        super().__init__(prefix, precision, device)
+
+    def attach(self, mixer, mixer_norm):
+        self.mixer, self.mixer_norm = mixer, mixer_norm
+
+    def forward(self, x, pending, batch, cache, next_norm=None):
+        return x, self.mixer.forward(self.mixer_norm.forward(x, delta=pending), batch, cache)
+
+
+@register_part("mixer", "toy_lookback")
+class Lookback(Part):
+    """y_t = W_out (m_t * m_{t - lag}) with m_t = W_in x_t, a vector of `memory` numbers, and
+    m_{t - lag} = 0 before the sequence's start. Every token's m goes to the request's pages: one
+    paged tensor, float32 whatever the engine's precision, a token's numbers side by side; only
+    the last lag + 1 tokens are kept, so pages behind that go back while the request lives."""
+
+    graph_safe = False          # reads lengths and block tables on the host
+
+    def __init__(self, prefix, precision, device, hidden_size, memory, lag):
+        super().__init__(prefix, precision, device)
+        self.hidden_size, self.memory, self.lag = hidden_size, memory, lag
+        self.w_in = self.w_out = None
+
+    def cache_need(self):
+        return CacheNeed(paged=(PagedTensor("memory", (self.memory,), token_axis=0, dtype=torch.float32),),
+                         window=self.lag + 1)
+
+    def tensors(self):
+        return {self._name("in.weight"): (self.memory, self.hidden_size),
+                self._name("out.weight"): (self.hidden_size, self.memory)}
+
+    def load(self, fetch):
+        self.w_in = fetch(self._name("in.weight"), torch.float32)
+        self.w_out = fetch(self._name("out.weight"), torch.float32)
+
+    def forward(self, x, batch, cache):
+        pages = cache.paged["memory"]                      # (pages, page_size, memory)
+        size = pages.shape[1]
+        m = x.float() @ self.w_in.T
+        table = cache.block_table.tolist()
+        out = torch.empty_like(x)
+        at = 0
+        for b, (n, kv) in enumerate(zip(batch.q_lens, batch.kv_lens_host)):
+            for i in range(n):
+                pos = kv - n + i
+                if cache.writes:
+                    pages[table[b][pos // size], pos % size] = m[at + i]
+                back = pos - self.lag
+                if back < 0:
+                    old = torch.zeros_like(m[at + i])
+                else:
+                    page = table[b][back // size]
+                    assert page >= 0, "the page of a position inside the window was given back"
+                    old = pages[page, back % size]
+                out[at + i] = ((m[at + i] * old) @ self.w_out.T).to(x.dtype)
+            at += n
+        return out
+
+
 @dataclasses.dataclass(frozen=True)
 class ToyHybridConfig:
     architecture: str
@@ -108,10 +197,10 @@ class ToyHybridConfig:
         missing = [k for k, _ in KEYS if k not in data]
         if missing:
             raise ConfigError("config.json of %s lacks %s" % (NAME, ", ".join(missing)))
-        if not data["pattern"] or set(data["pattern"]) - set("abs"):
-            raise ConfigError("pattern must be a string of 'a', 'b' and 's'")
-        if data["norm"] not in ("rms", "centred") or data["arrangement"] not in ("sequential", "parallel"):
-            raise ConfigError("norm is rms or centred, arrangement sequential or parallel")
+        if not data["pattern"] or set(data["pattern"]) - set("abspn"):
+            raise ConfigError("pattern must be a string of 'a', 'b', 's', 'p' and 'n'")
+        if data["norm"] not in ("rms", "centred") or data["arrangement"] not in ("sequential", "parallel", "sandwich"):
+            raise ConfigError("norm is rms or centred, arrangement sequential, parallel or sandwich")
         return cls(architecture=data["architectures"][0], **{k: kind(data[k]) for k, kind in KEYS})
 
     def to_dict(self):
@@ -123,7 +212,8 @@ class ToyHybridConfig:
 
 def toy_hybrid_spec(c):
     norm = PartSpec.of("norm", "rms" if c.norm == "rms" else "toy_centred", size=c.width, eps=c.eps)
-    block = PartSpec.of("block", "pre_norm" if c.arrangement == "sequential" else "toy_parallel")
+    block = PartSpec.of("block", {"sequential": "pre_norm", "parallel": "toy_parallel",
+                                  "sandwich": "toy_sandwich"}[c.arrangement])
     attention = PartSpec.of("mixer", "attention", hidden_size=c.width, num_heads=c.heads, num_kv_heads=c.kv_heads,
                             head_dim=c.head_size, qk_norm=False, qk_norm_eps=c.eps, window=c.window)
     everything = attention.with_params(window=0)
@@ -131,10 +221,22 @@ def toy_hybrid_spec(c):
                                 max_positions=c.max_position_embeddings)
     mean = PartSpec.of("mixer", "toy_running_mean", hidden_size=c.width)
     ff = PartSpec.of("feed_forward", "swiglu", hidden_size=c.width, intermediate_size=c.inner)
-    mixers = {"a": attention, "b": everything, "s": mean}
-    layers = tuple(LayerSpec(prefix="hybrid.layers.%d" % i, mixer=mixers[kind], feed_forward=ff,
-                             mixer_norm=norm, feed_forward_norm=norm, block=block,
-                             position=half_rotation if kind == "b" else None) for i, kind in enumerate(c.pattern))
+    lookback = PartSpec.of("mixer", "toy_lookback", hidden_size=c.width, memory=MEMORY, lag=LAG)
+    mixers = {"a": attention, "b": everything, "s": mean, "p": lookback, "n": lookback}
+
+    def layer(i, kind):
+        prefix = "hybrid.layers.%d" % i
+        if kind == "n":                 # a mixer behind its norm and nothing else
+            return LayerSpec(prefix=prefix, block=PartSpec.of("block", "toy_mixer_only"), slots=(
+                Slot("mixer", lookback, "self_attn"), Slot("mixer_norm", norm, "input_layernorm")))
+        usual = pre_norm_layer(prefix, mixer=mixers[kind], feed_forward=ff, mixer_norm=norm, feed_forward_norm=norm,
+                               block=block, position=half_rotation if kind == "b" else None)
+        if c.arrangement != "sandwich":
+            return usual
+        return dataclasses.replace(usual, slots=usual.slots + (
+            Slot("mixer_out_norm", norm, "post_mixer_norm"), Slot("feed_forward_out_norm", norm, "post_mlp_norm")))
+
+    layers = tuple(layer(i, kind) for i, kind in enumerate(c.pattern))
     return ModelSpec(
         hidden_size=c.width, vocab_size=c.vocab,
         embedding=PartSpec.of("embedding", "token", vocab_size=c.vocab, hidden_size=c.width),
@@ -154,6 +256,10 @@ EXAMPLE = dict(architectures=[NAME], vocab=211, width=40, inner=72, heads=6, kv_
 EXAMPLE_PARALLEL = dict(architectures=[NAME], vocab=157, width=56, inner=100, heads=4, kv_heads=4, head_size=32,
                         pattern="sbas", window=0, eps=1e-6, theta=500000.0, max_position_embeddings=300,
                         norm="centred", arrangement="parallel")
+# a block with four norms, a mixer that pages one tensor of its own width, a layer without a feed-forward
+EXAMPLE_SANDWICH = dict(architectures=[NAME], vocab=173, width=48, inner=88, heads=3, kv_heads=1, head_size=16,
+                        pattern="pasnb", window=17, eps=1e-5, theta=20000.0, max_position_embeddings=400,
+                        norm="rms", arrangement="sandwich")
 
 
 def _norm(c, x, w, name):
@@ -175,6 +281,10 @@ def plain_logits(c, w, tokens):
         if kind == "s":
             mean = torch.cumsum(h, dim=0) / torch.arange(1, T + 1)[:, None]
             mixed = mean @ w[p + ".self_attn.mix.weight"].T
+        elif kind in "pn":
+            m = h @ w[p + ".self_attn.in.weight"].T
+            old = torch.cat((torch.zeros(min(LAG, T), m.shape[1]), m[:max(T - LAG, 0)]), dim=0)
+            mixed = (m * old) @ w[p + ".self_attn.out.weight"].T
         else:
             a = p + ".self_attn"
             q = (h @ w[a + ".q_proj.weight"].T).view(T, c.heads, c.head_size)
@@ -191,7 +301,13 @@ def plain_logits(c, w, tokens):
             o = plain.causal_attention(q, k, v, 1.0 / math.sqrt(c.head_size),
                                        (c.window or None) if kind == "a" else None)
             mixed = o.reshape(T, c.heads * c.head_size) @ w[a + ".o_proj.weight"].T
-        if c.arrangement == "parallel":
+        if kind == "n":
+            x = x + mixed
+        elif c.arrangement == "sandwich":
+            x = x + _norm(c, mixed, w, p + ".post_mixer_norm")
+            fed = plain.swiglu_mlp(_norm(c, x, w, p + ".post_attention_layernorm"), w, p + ".mlp")
+            x = x + _norm(c, fed, w, p + ".post_mlp_norm")
+        elif c.arrangement == "parallel":
             x = x + mixed + plain.swiglu_mlp(_norm(c, x, w, p + ".post_attention_layernorm"), w, p + ".mlp")
         else:
             x = x + mixed

@@ -1,0 +1,255 @@
+// A weight-streaming matrix-core product for some tens of rows of x (17 to 96), out[M, N] =
+// x[M, K] . w[N, K]^T in bfloat16 with float32 accumulation, from the tile-ordered copy of the
+// weight that the few-row kernel of gemm.hip reads (w[slab][k / 32][lane][8], one contiguous
+// kilobyte per matrix instruction). The reference has no kernel for this range of its own: its
+// engine sends every projection to the vendor library (src/qwen3_from_scratch/models/self_attn.py:312-342)
+// and the feed-forward to one Triton kernel of 128 x 128 tiles
+// (src/qwen3_from_scratch/kernels/triton/gemm.py:26-274).
+//
+// With 17 to 128 rows a product is still bound by the one pass over the weight, but the rows of x
+// no longer fit a wavefront's registers, and if every slab of 16 weight rows fetches them from the
+// L2 again they pass from the L2 as often as the weight passes from memory (M / 16 times as many
+// bytes). Here a block of WS x 2 wavefronts owns WS slabs and walks K in chunks of 256: the chunk
+// of x (all rows) goes through shared memory once per block, so x leaves the L2 once per WS slabs;
+// each wavefront multiplies its slab's 128 k of the chunk (the weight straight from memory into
+// registers, as the first operand of v_mfma_f32_16x16x32_bf16, x from shared memory as the second)
+// into MT accumulators of 16 x 16, the weight of the next chunk already on its way. The two
+// wavefronts of a slab add up through shared memory in a fixed order. One barrier per chunk.
+//
+// K may be shared out over gridDim.y blocks per slab group (float32 partial products, added by
+// tiles::gemm_tiles_reduce_kernel in a fixed order), which is how a product with few slabs fills
+// the chip; a product with many (the gate/up projection) runs whole, with the epilogues of
+// tiles::store_tile: the division by the rows' root mean square that the norm before it left out,
+// SwiGLU over interleaved (gate, up) rows, bfloat16 or float32 output.
+//
+// Measured on the 8B layer's gate/up product (24,576 x 4,096, 201 MB) with cold caches, this
+// kernel alone: 40 us at 24 to 48 rows, 42 at 64, 50 at 96 (the vendor library's product: 45, 42,
+// 49, 48, 70, without the activation); with the weight loads alone and no arithmetic 42 at 64
+// rows, so it is the stream that takes the time. Blocks of four slabs are some microseconds slower
+// on it, two slabs per wavefront the same; starting every block at another chunk changes nothing.
+// K must be a multiple of 32 (the tile-ordered copy has no other), N of 4 (of 2 with SwiGLU).
+#pragma once
+
+#include "gemm_tiles.h"
+
+namespace stream {
+
+using tiles::f32x4_t;
+using tiles::Frag;
+using tiles::RowScale;
+
+constexpr int WK = 2;            // wavefronts that share a slab's chunk
+constexpr int KC = 128;          // k per wavefront per chunk
+constexpr int KCB = KC * WK;     // k per chunk
+constexpr int STEPS = KC / 32;   // matrix instructions per accumulator per chunk
+constexpr int ROW = KCB * 2 + 16;   // bytes of a row of x in shared memory: 16 more than its data, so that the
+                                    // sixteen rows one operand read touches start in different banks
+constexpr int MOST_ROWS = 96;
+
+constexpr int smem_bytes(int MT, int WS) {
+  const int x_bytes = 2 * MT * 16 * ROW, sums_bytes = WS * WK * MT * 64 * 16;
+  return x_bytes > sums_bytes ? x_bytes : sums_bytes;
+}
+
+template <typename OUT, int EPI, int MT, int WS>
+__global__ __launch_bounds__(WS * WK * 64) void gemm_stream_kernel(const bf16_t* __restrict__ x,
+                                                                   const bf16_t* __restrict__ wt, OUT* __restrict__ out,
+                                                                   int M, int N, int K, int k_per_block,
+                                                                   float* __restrict__ partials, RowScale scale) {
+  constexpr int THREADS = WS * WK * 64;
+  constexpr int ROWS = MT * 16;
+  constexpr int PIECES = ROWS * KCB / 8;                        // 16-byte pieces of a chunk of x
+  constexpr int PER_THREAD = (PIECES + THREADS - 1) / THREADS;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];   // two chunks of x, ROWS x ROW bytes each
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int ws = wave % WS, wk = wave / WS;
+  const int col = lane & 15, grp = lane >> 4;
+  const int slabs = (N + 15) / 16;
+  const int slab = blockIdx.x * WS + ws;
+  const bool slab_ok = slab < slabs;
+  const int kb = blockIdx.y * k_per_block;
+  const int ke = min(K, kb + k_per_block);
+  const int chunks = (ke - kb + KCB - 1) / KCB;
+  const bf16_t* wp = wt + (size_t)(slab_ok ? slab : 0) * (K / 32) * 512 + lane * 8;
+
+  f32x4_t acc[MT][1];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) acc[t][0] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  auto load_w = [&](Frag (&a)[STEPS], int c) {
+    const int k0 = kb + c * KCB + wk * KC;
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+      const int k = k0 + 32 * s;
+      a[s].u = (slab_ok && k < ke) ? *reinterpret_cast<const uint4*>(wp + (size_t)(k / 32) * 512) : make_uint4(0, 0, 0, 0);
+    }
+  };
+  auto load_x = [&](uint4 (&r)[PER_THREAD], int c) {
+    const int k0 = kb + c * KCB;
+#pragma unroll
+    for (int i = 0; i < PER_THREAD; ++i) {
+      const int piece = threadIdx.x + i * THREADS;
+      const int row = piece / (KCB / 8), k = k0 + (piece % (KCB / 8)) * 8;
+      r[i] = (piece < PIECES && row < M && k < ke) ? *reinterpret_cast<const uint4*>(x + (size_t)row * K + k)
+                                                   : make_uint4(0, 0, 0, 0);
+    }
+  };
+  auto store_x = [&](const uint4 (&r)[PER_THREAD], int buffer) {
+#pragma unroll
+    for (int i = 0; i < PER_THREAD; ++i) {
+      const int piece = threadIdx.x + i * THREADS;
+      if (piece < PIECES)
+        *reinterpret_cast<uint4*>(lds + buffer * ROWS * ROW + (piece / (KCB / 8)) * ROW + (piece % (KCB / 8)) * 16) = r[i];
+    }
+  };
+  auto multiply = [&](const Frag (&a)[STEPS], int buffer) {
+    const unsigned char* base = lds + buffer * ROWS * ROW + col * ROW + (wk * KC + 8 * grp) * 2;
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+      Frag b[MT];
+#pragma unroll
+      for (int t = 0; t < MT; ++t) b[t].u = *reinterpret_cast<const uint4*>(base + t * 16 * ROW + s * 64);
+#pragma unroll
+      for (int t = 0; t < MT; ++t) acc[t][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s].v, b[t].v, acc[t][0], 0, 0, 0);
+    }
+  };
+
+  Frag even[STEPS], odd[STEPS];
+  uint4 staged[PER_THREAD];
+  load_w(even, 0);
+  load_x(staged, 0);
+  // the rows' factors while the first loads are on their way
+  float factor[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) factor[t] = (scale.sums && !partials && wk == 0 && 16 * t + col < M) ? scale.of(16 * t + col) : 1.f;
+  store_x(staged, 0);
+  for (int c = 0; c < chunks; c += 2) {
+    // chunk c: its weight in `even`, its x in buffer 0; the next chunk's loads go out before the wait
+    if (c + 1 < chunks) {
+      load_w(odd, c + 1);
+      load_x(staged, c + 1);
+    }
+    __syncthreads();            // buffer 0 is written; nobody still reads buffer 1
+    multiply(even, 0);
+    if (c + 1 >= chunks) break;
+    store_x(staged, 1);
+    if (c + 2 < chunks) {
+      load_w(even, c + 2);
+      load_x(staged, c + 2);
+    }
+    __syncthreads();            // buffer 1 is written; nobody still reads buffer 0
+    multiply(odd, 1);
+    if (c + 2 < chunks) store_x(staged, 0);
+  }
+  // the second wavefront of every slab hands its sums over, and the first adds them to its own
+  __syncthreads();
+  float* sums = reinterpret_cast<float*>(lds);          // [slab of the block][MT][64 lanes][4]
+  if (wk > 0) {
+#pragma unroll
+    for (int t = 0; t < MT; ++t) *reinterpret_cast<f32x4_t*>(sums + ((ws * MT + t) * 64 + lane) * 4) = acc[t][0];
+  }
+  __syncthreads();
+  if (wk > 0 || !slab_ok) return;
+#pragma unroll
+  for (int t = 0; t < MT; ++t) acc[t][0] += *reinterpret_cast<const f32x4_t*>(sums + ((ws * MT + t) * 64 + lane) * 4);
+  if (partials)
+    tiles::store_tile<float, tiles::EPI_PLAIN, MT, 1>(acc, partials + (size_t)blockIdx.y * M * N, M, N, 0, slab * 16, col,
+                                                      grp, factor);
+  else
+    tiles::store_tile<OUT, EPI, MT, 1>(acc, out, M, N, 0, slab * 16, col, grp, factor);
+}
+
+// How a product is laid over the chip: blocks of `ws` slabs (6 or 4), K in `splits` shares.
+struct Plan {
+  int ws = 0, splits = 1;
+};
+
+// By a model of the kernel's time, not a stopwatch (the same for every process): a block streams its
+// share of the weight at what one CU draws from memory (about 21 GB/s), blocks beyond one per CU wait for
+// the next round (with more than two rounds the rounds blur, and the chip's rate is what counts), shares of
+// K cost their float32 partial products written and read once and a second kernel. Blocks of six slabs win
+// a tie. 8B layer at 64 rows: gate/up 6 slabs whole (256 blocks), q/k/v 6 slabs in 4 shares (256 blocks),
+// the vocabulary's product 6 slabs whole (1,583 blocks: 265 us, with blocks of four slabs 270).
+inline Plan plan_for(int M, int N, int K, bool second_kernel_anyway) {
+  const int slabs = (N + 15) / 16, chunks = (K + KCB - 1) / KCB;
+  Plan best;
+  double best_us = 0.0;
+  for (int ws : {6, 4}) {
+    const int blocks_n = (slabs + ws - 1) / ws;
+    for (int splits = 1; splits <= 16 && splits <= chunks; ++splits) {
+      const int per = (chunks + splits - 1) / splits;
+      if ((chunks + per - 1) / per != splits) continue;      // the same shares under another name
+      const long blocks = (long)blocks_n * splits;
+      const double rounds = blocks > 512 ? blocks / 256.0 : (double)((blocks + 255) / 256);
+      double us = 3.0 + rounds * ((double)ws * 16 * per * KCB * 2) / 21000.0;
+      if (splits > 1) us += (second_kernel_anyway ? 0.0 : 1.5) + 2.0 * splits * M * (double)N * 4 / 4.0e6;
+      if (best.ws == 0 || us < 0.98 * best_us) {      // a later candidate has to win by something
+        best.ws = ws;
+        best.splits = splits;
+        best_us = us;
+      }
+    }
+  }
+  return best;
+}
+
+inline bool takes(int M, int N, int K) { return M > 16 && M <= MOST_ROWS && N >= 16 && K >= KCB && K % 32 == 0 && N % 2 == 0; }
+
+template <typename OUT, int EPI, int MT, int WS>
+int launch_shape(const void* x, const void* wt, void* out, int M, int N, int K, int splits, float* partials,
+                 hipStream_t stream, const RowScale& scale, bool keep_partials, int* splits_used) {
+  constexpr int SMEM = smem_bytes(MT, WS);
+  static bool raised[16] = {};   // the dynamic shared-memory limit, once per device
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 16) return Q3_ERR_BAD_ARGUMENT;
+  auto kernel = gemm_stream_kernel<OUT, EPI, MT, WS>;
+  if (!raised[device]) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
+    if (e != hipSuccess) return (int)e;
+    raised[device] = true;
+  }
+  const int slabs = (N + 15) / 16, chunks = (K + KCB - 1) / KCB;
+  if (splits < 1 || splits > chunks || splits > 64) return Q3_ERR_BAD_ARGUMENT;
+  const int per = (chunks + splits - 1) / splits;
+  const int used = (chunks + per - 1) / per;      // no block without a chunk
+  const bool to_partials = used > 1 || keep_partials;
+  if (to_partials && (N % 4 || partials == nullptr)) return Q3_ERR_BAD_ARGUMENT;
+  const int blocks_n = (slabs + WS - 1) / WS;
+  if (blocks_n > 65535 * 32) return Q3_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(kernel, dim3(blocks_n, used), dim3(WS * WK * 64), SMEM, stream, (const bf16_t*)x, (const bf16_t*)wt,
+                     (OUT*)out, M, N, K, per * KCB, to_partials ? partials : nullptr, to_partials ? RowScale() : scale);
+  if (splits_used) *splits_used = used;
+  if (to_partials && !keep_partials) {
+    const size_t quads = (size_t)M * N / 4;
+    hipLaunchKernelGGL((tiles::gemm_tiles_reduce_kernel<OUT, EPI == tiles::EPI_SWIGLU>), dim3((unsigned)((quads + 255) / 256)),
+                       dim3(256), 0, stream, partials, (OUT*)out, quads, N / 4, used, scale);
+  }
+  return q3_launch_status();
+}
+
+// x (M, K) row-major, wt the tile-ordered copy of w (N, K); see tiles::launch for `splits`, `partials`,
+// `scale`, `keep_partials`.
+template <typename OUT, int EPI>
+int launch(const Plan& plan, const void* x, const void* wt, void* out, int M, int N, int K, float* partials,
+           hipStream_t stream, const RowScale& scale = RowScale(), bool keep_partials = false,
+           int* splits_used = nullptr) {
+  if (!takes(M, N, K) || (plan.ws != 6 && plan.ws != 4)) return Q3_ERR_BAD_ARGUMENT;
+  const int mt = (M + 15) / 16;
+#define Q3_STREAM_SHAPE(MT_)                                                                                        \
+  return plan.ws == 6 ? launch_shape<OUT, EPI, MT_, 6>(x, wt, out, M, N, K, plan.splits, partials, stream, scale,   \
+                                                       keep_partials, splits_used)                                  \
+                      : launch_shape<OUT, EPI, MT_, 4>(x, wt, out, M, N, K, plan.splits, partials, stream, scale,   \
+                                                       keep_partials, splits_used)
+  switch (mt) {
+    case 2: Q3_STREAM_SHAPE(2);
+    case 3: Q3_STREAM_SHAPE(3);
+    case 4: Q3_STREAM_SHAPE(4);
+    case 5:
+    case 6: Q3_STREAM_SHAPE(6);
+  }
+#undef Q3_STREAM_SHAPE
+  return Q3_ERR_BAD_ARGUMENT;
+}
+
+}  // namespace stream

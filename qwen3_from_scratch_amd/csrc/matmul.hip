@@ -36,6 +36,7 @@
 
 #include "common.h"
 #include "gemm_tiles.h"
+#include "gemm_stream.h"
 
 #include <hipblaslt/hipblaslt.h>
 
@@ -645,6 +646,60 @@ extern "C" int q3_tiles_residual(const void* x, const void* w, int M, int N, int
     hipLaunchKernelGGL(tiles::tiles_residual_kernel<bf16_t>, grid, dim3(256), 0, stream, d.partials, used, residual,
                        (const bf16_t*)norm_weight, (bf16_t*)values, sums, sums_stride, M, N);
   return q3_launch_status();
+}
+
+// A product of 17 to 96 rows by the weight-streaming kernel of gemm_stream.h, from the tile-ordered copy `wt` of
+// the weight (N, K): out (M, N) in `out_dtype` (`epilogue` 0) or, the weight's rows interleaving gate and up,
+// out (M, N / 2) bfloat16 = silu(gate) * up (`epilogue` 1). With `sums` the rows of x still lack their norm's
+// division, as for q3_tiles_scaled. Returns Q3_DECLINED, and has done nothing, where another kernel is the way:
+// the caller has asked for the library's or the tiled kernel's products alone, the tuner is on (it times those),
+// the size is not the kernel's, or the weight is so small that other kernels serve these rows better.
+constexpr size_t STREAM_LEAST_WEIGHT_BYTES = 24u << 20;
+
+extern "C" int q3_stream_product(const void* x, const void* wt, void* out, int M, int N, int K, int out_dtype,
+                                 int epilogue, const float* sums, int chunks, int sums_stride, float eps, int width,
+                                 void* stream_) {
+  if (!x || !wt || !out || M < 1 || N < 1 || K < 1) return Q3_ERR_BAD_ARGUMENT;
+  const bool swiglu = epilogue == tiles::EPI_SWIGLU;
+  if (!swiglu && epilogue != tiles::EPI_PLAIN) return Q3_ERR_BAD_ARGUMENT;
+  if (swiglu ? out_dtype != Q3_BF16 : (out_dtype != Q3_BF16 && out_dtype != Q3_F32)) return Q3_ERR_BAD_ARGUMENT;
+  if (sums && (chunks < 1 || sums_stride < M || width != K)) return Q3_ERR_BAD_ARGUMENT;
+  hipStream_t stream = (hipStream_t)stream_;
+  std::lock_guard<std::mutex> hold(g_lock);
+  if (g_kernels != KERNELS_BOTH || g_mode != MODE_RULE) return Q3_DECLINED;
+  if (!stream::takes(M, N, K) || (size_t)N * K * 2 < STREAM_LEAST_WEIGHT_BYTES) return Q3_DECLINED;
+  const stream::Plan plan = stream::plan_for(M, N, K, false);
+  if (plan.splits > 1 && (N % 4 || (size_t)plan.splits * M * N * sizeof(float) > PARTIALS_BYTES)) return Q3_DECLINED;
+  int device = 0;
+  HIP_TRY(hipGetDevice(&device));
+  Device& d = g_devices[device];
+  int status = ready_device(d, stream);
+  if (status) return status;
+  tiles::RowScale scale;
+  if (sums) {
+    scale.sums = sums;
+    scale.chunks = chunks;
+    scale.rows = sums_stride;
+    scale.eps = eps;
+    scale.inv_width = 1.f / (float)width;
+  }
+  if (swiglu) return stream::launch<bf16_t, tiles::EPI_SWIGLU>(plan, x, wt, out, M, N, K, d.partials, stream, scale);
+  if (out_dtype == Q3_F32)
+    return stream::launch<float, tiles::EPI_PLAIN>(plan, x, wt, out, M, N, K, d.partials, stream, scale);
+  return stream::launch<bf16_t, tiles::EPI_PLAIN>(plan, x, wt, out, M, N, K, d.partials, stream, scale);
+}
+
+// How q3_stream_product would lay a product over the chip (info[0] slabs per block, info[1] shares of K);
+// 0 is returned for a size it declines under the current settings.
+extern "C" int q3_stream_plan(int M, int N, int K, int* info) {
+  std::lock_guard<std::mutex> hold(g_lock);
+  if (g_kernels != KERNELS_BOTH || g_mode != MODE_RULE) return 0;
+  if (!stream::takes(M, N, K) || (size_t)N * K * 2 < STREAM_LEAST_WEIGHT_BYTES) return 0;
+  const stream::Plan plan = stream::plan_for(M, N, K, false);
+  if (plan.splits > 1 && (N % 4 || (size_t)plan.splits * M * N * sizeof(float) > PARTIALS_BYTES)) return 0;
+  info[0] = plan.ws;
+  info[1] = plan.splits;
+  return 1;
 }
 
 // The hand-written tiled kernel alone (gemm_tiles.h), tile shape `config` (0 .. q3_gemm_tiles_configs() - 1):

@@ -45,6 +45,7 @@ __all__ = [
     "gemm_tiles_configs",
     "gemm_tiles_splits",
     "matmul_plan",
+    "stream_plan",
     "tile_weight",
     "sample",
     "measured_read_rate",
@@ -595,6 +596,43 @@ def _tiles_scaled(x, weight, out, unscaled, swiglu, what):
     return out
 
 
+STREAM_ROWS_MOST = 96
+
+
+def stream_plan(M, N, K):
+    """How the weight-streaming kernel for 17 to 96 rows would serve a product with a tile-ordered
+    weight of (N, K) under the current settings: (slabs of 16 weight rows per block, shares of K),
+    or None where it leaves the product to the other kernels (small weights, `matmul_kernels`
+    other than "both", the tuner on)."""
+    info = (ctypes.c_int * 2)()
+    if not _matmul().q3_stream_plan(int(M), int(N), int(K), info):
+        return None
+    return int(info[0]), int(info[1])
+
+
+def _stream_product(x, weight, tiled, out, swiglu, unscaled, what):
+    """The product by the weight-streaming kernel, if it takes it: True if `out` is written."""
+    M, K = x.shape
+    N = weight.shape[0]
+    if tiled is None or not FEW_ROWS < M <= STREAM_ROWS_MOST or K % 32 or not x.is_contiguous() or not out.is_contiguous():
+        return False
+    _need(tiled.is_cuda and tiled.dtype == torch.bfloat16 and tiled.is_contiguous()
+          and tiled.numel() == (-(-N // 16) * 16) * K, "the tiled copy does not belong to this weight")
+    sums, chunks, stride, eps, width = None, 0, 0, 0.0, 0
+    if unscaled is not None:
+        sums, eps, width = unscaled
+        _check_sums(sums, M)
+        _need(width == K, "the rows' width must be the product's inner size")
+        chunks, stride = sums.shape
+    status = _matmul().q3_stream_product(
+        _ptr(x), _ptr(tiled), _ptr(out), M, N, K, _DT[out.dtype], 1 if swiglu else 0, _ptr(sums), chunks, stride,
+        ctypes.c_float(eps), int(width), _stream())
+    if status == _DECLINED:
+        return False
+    _check(status, what)
+    return True
+
+
 def linear(x, weight, out_dtype=None, out=None, tiled=None, unscaled=None):
     """out = x @ weight^T with float32 accumulation. x (M, K), weight (N, K).
     `tiled` is `tile_weight(weight)`, if the caller keeps one: few rows are then served from it.
@@ -622,6 +660,9 @@ def linear(x, weight, out_dtype=None, out=None, tiled=None, unscaled=None):
         _check(library("gemm").q3_linear_tiled(
             _ptr(x), _ptr(tiled), _ptr(out), M, N, K, _DT[out_dtype], 0, sums, sums_rows, eps, width,
             None, None, 0, None, stride, _stream()), "linear")
+        return out
+    if M and x.dtype == torch.bfloat16 and (unscaled is None or fused_rows_take(weight, M)) \
+            and _stream_product(x, weight, tiled, out, False, unscaled, "linear"):
         return out
     if unscaled is not None and x.dtype == torch.bfloat16 and fused_rows_take(weight, M):
         return _tiles_scaled(x, weight, out, unscaled, False, "linear")
@@ -684,6 +725,11 @@ def linear_swiglu(x, weight, tiled=None, unscaled=None):
             _ptr(x), _ptr(tiled), _ptr(out), M, N, K, 1, 1, sums, sums_rows, eps, width,
             None, None, 0, None, stride, _stream()), "linear_swiglu")
         return out
+    if M and x.dtype == torch.bfloat16 and tiled is not None and FEW_ROWS < M <= STREAM_ROWS_MOST \
+            and (unscaled is None or fused_rows_take(weight, M)):
+        out = torch.empty((M, N // 2), dtype=x.dtype, device=x.device)
+        if _stream_product(x, weight, tiled, out, True, unscaled, "linear_swiglu"):
+            return out
     if unscaled is not None and x.dtype == torch.bfloat16 and fused_rows_take(weight, M):
         out = torch.empty((M, N // 2), dtype=x.dtype, device=x.device)
         return _tiles_scaled(x, weight, out, unscaled, True, "linear_swiglu")

@@ -892,6 +892,63 @@ def test_linear_residual_norm_and_unscaled_rows_beyond_sixteen(M, H, K, N2, norm
         ops.matmul_kernels("both")
 
 
+@pytest.mark.parametrize("M", [17, 32, 33, 50, 64, 80, 96])
+@pytest.mark.parametrize("N,K", [(3400, 4000), (9000, 1440), (24576, 4096), (1540, 12288)])
+def test_weight_streaming_product_for_some_tens_of_rows(M, N, K):
+    """17 to 96 rows against a weight of 24 MB or more, from its tile-ordered copy: plain in bfloat16
+    and float32, with the rows' division by their rms, and with SwiGLU; K that is no multiple of a
+    chunk (256) or of 64, N that is no multiple of 16, few slabs (K shared out, the shares added by
+    a second kernel) and many (one pass, the epilogue in the kernel). Against float64 sums."""
+    ops = _ops()
+    x = _rand((M, K), torch.bfloat16, 61)
+    w = _rand((N, K), torch.bfloat16, 62, scale=0.05)
+    tiled = ops.tile_weight(w)
+    plan = ops.stream_plan(M, N, K)
+    assert plan is not None and plan[0] in (4, 6) and 1 <= plan[1] <= 16
+    if (N, K) == (24576, 4096):
+        assert plan == (6, 1)                                      # whole: 256 blocks of six slabs
+    exact = x.double() @ w.double().T
+    scale = float(exact.abs().max())
+    got32 = ops.linear(x, w, out_dtype=torch.float32, tiled=tiled)
+    assert float((got32.double() - exact).abs().max()) <= 1e-3 * scale
+    got = ops.linear(x, w, tiled=tiled)
+    assert torch.equal(got, ops.linear(x, w, tiled=tiled))         # the same bits every time
+    torch.testing.assert_close(got.float(), got32, rtol=8e-3, atol=4e-3 * scale)
+    # the streaming kernel served these, not the library: its sums are closer to exact than bfloat16 products
+    # of the other kernels are to each other, and the plan says so; without the copy the others serve
+    other = ops.linear(x, w, out_dtype=torch.float32)
+    assert float((other.double() - exact).abs().max()) <= 1e-3 * scale
+    # rows that still lack their norm's division, the sums of squares in chunks as the writer leaves them
+    sums = torch.zeros((-(-K // 1024), ops.sums_stride(M)), dtype=torch.float32, device="cuda")
+    sums[:, :M] = (torch.rand((sums.shape[0], M), device="cuda") + 0.5) * K / sums.shape[0]
+    sums[:, M // 2] *= 900.0                                        # a row whose factor is far from the others'
+    eps = 1e-5
+    factor = torch.rsqrt(sums[:, :M].double().sum(dim=0) / K + eps)[:, None]
+    if K % 64 == 0 and N % 4 == 0:
+        scaled = ops.linear(x, w, out_dtype=torch.float32, tiled=tiled, unscaled=(sums, eps, K))
+        for m in range(M):
+            row = exact[m] * factor[m]
+            assert float((scaled[m].double() - row).abs().max()) <= 2e-3 * float(row.abs().max()), m
+        act = ops.linear_swiglu(x, w, tiled=tiled, unscaled=(sums, eps, K))
+        want = torch_ops.swiglu((exact * factor).float().bfloat16().float())
+        assert act.shape == (M, N // 2)
+        assert float((act.float() - want).abs().max()) <= 2e-2 * max(1.0, float(want.abs().max()))
+    plain_act = ops.linear_swiglu(x, w, tiled=tiled)
+    want = torch_ops.swiglu(exact.float().bfloat16().float())
+    assert float((plain_act.float() - want).abs().max()) <= 2e-2 * max(1.0, float(want.abs().max()))
+    # asked for the other kernels alone, the streaming kernel steps aside
+    try:
+        ops.matmul_kernels("own")
+        assert ops.stream_plan(M, N, K) is None
+        if K % 64 == 0:
+            torch.testing.assert_close(ops.linear(x, w, out_dtype=torch.float32, tiled=tiled), got32, rtol=2e-3,
+                                       atol=1e-3 * scale)
+    finally:
+        ops.matmul_kernels("both")
+    assert ops.stream_plan(16, N, K) is None and ops.stream_plan(97, N, K) is None
+    assert ops.stream_plan(M, 1024, 4096) is None                  # a small weight: the other kernels' rows
+
+
 def test_linear_float32_is_true_float32():
     """Inputs whose products need all 24 bits: a matrix mode of reduced precision
     (bf16 or tf32-like splitting) would be off by far more than float32 rounding."""

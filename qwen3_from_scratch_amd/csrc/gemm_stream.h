@@ -22,6 +22,11 @@
 // tiles::store_tile: the division by the rows' root mean square that the norm before it left out,
 // SwiGLU over interleaved (gate, up) rows, bfloat16 or float32 output.
 //
+// With 9 to 16 rows the few-row kernel of gemm.hip fetches x per slab (or per pair of slabs) and that
+// traffic slows it (gate/up 42.5 us at 12 rows, 44.7 at 16); this kernel takes 40 us at any of them, and
+// serves that product there too. Below nine rows the few-row kernel is as fast or faster, and the products
+// with fewer slabs would need their K shared out and a second kernel, which costs more than it saves.
+//
 // Measured on the 8B layer's gate/up product (24,576 x 4,096, 201 MB) with cold caches, this
 // kernel alone: 40 us at 24 to 48 rows, 42 at 64, 50 at 96 (the vendor library's product: 45, 42,
 // 49, 48, 70, without the activation); with the weight loads alone and no arithmetic 42 at 64
@@ -118,10 +123,31 @@ __global__ __launch_bounds__(WS * WK * 64) void gemm_stream_kernel(const bf16_t*
   uint4 staged[PER_THREAD];
   load_w(even, 0);
   load_x(staged, 0);
-  // the rows' factors while the first loads are on their way
+  // the rows' factors while the first loads are on their way: the partial sums of squares (few chunks of
+  // 1,024 columns from the kernel that adds shares of K, hundreds of slabs from the few-row kernel) are
+  // added by the whole block, thread (g, r) the chunks g, g + G, ... of row r, then the G sums of a row in
+  // their order: a fixed order of additions
   float factor[MT];
 #pragma unroll
-  for (int t = 0; t < MT; ++t) factor[t] = (scale.sums && !partials && wk == 0 && 16 * t + col < M) ? scale.of(16 * t + col) : 1.f;
+  for (int t = 0; t < MT; ++t) factor[t] = 1.f;
+  if (scale.sums && !partials) {
+    __shared__ float part[THREADS];
+    constexpr int G = THREADS / ROWS;
+    const int r = threadIdx.x % ROWS, g = threadIdx.x / ROWS;
+    float sum = 0.f;
+    if (g < G && r < scale.rows)
+      for (int c = g; c < scale.chunks; c += G) sum += scale.sums[(size_t)c * scale.rows + r];
+    part[threadIdx.x] = sum;
+    __syncthreads();
+    if (wk == 0) {
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        float total = 0.f;
+        for (int g2 = 0; g2 < G; ++g2) total += part[g2 * ROWS + 16 * t + col];
+        factor[t] = rsqrtf(total * scale.inv_width + scale.eps);
+      }
+    }
+  }
   store_x(staged, 0);
   for (int c = 0; c < chunks; c += 2) {
     // chunk c: its weight in `even`, its x in buffer 0; the next chunk's loads go out before the wait
@@ -193,7 +219,7 @@ inline Plan plan_for(int M, int N, int K, bool second_kernel_anyway) {
   return best;
 }
 
-inline bool takes(int M, int N, int K) { return M > 16 && M <= MOST_ROWS && N >= 16 && K >= KCB && K % 32 == 0 && N % 2 == 0; }
+inline bool takes(int M, int N, int K) { return M > 8 && M <= MOST_ROWS && N >= 16 && K >= KCB && K % 32 == 0 && N % 2 == 0; }
 
 template <typename OUT, int EPI, int MT, int WS>
 int launch_shape(const void* x, const void* wt, void* out, int M, int N, int K, int splits, float* partials,
@@ -242,6 +268,7 @@ int launch(const Plan& plan, const void* x, const void* wt, void* out, int M, in
                       : launch_shape<OUT, EPI, MT_, 4>(x, wt, out, M, N, K, plan.splits, partials, stream, scale,   \
                                                        keep_partials, splits_used)
   switch (mt) {
+    case 1: Q3_STREAM_SHAPE(1);
     case 2: Q3_STREAM_SHAPE(2);
     case 3: Q3_STREAM_SHAPE(3);
     case 4: Q3_STREAM_SHAPE(4);

@@ -648,13 +648,29 @@ extern "C" int q3_tiles_residual(const void* x, const void* w, int M, int N, int
   return q3_launch_status();
 }
 
-// A product of 17 to 96 rows by the weight-streaming kernel of gemm_stream.h, from the tile-ordered copy `wt` of
+// A product of 17 to 96 rows (and a gate/up product of 9 to 16) by the weight-streaming kernel of gemm_stream.h, from the tile-ordered copy `wt` of
 // the weight (N, K): out (M, N) in `out_dtype` (`epilogue` 0) or, the weight's rows interleaving gate and up,
 // out (M, N / 2) bfloat16 = silu(gate) * up (`epilogue` 1). With `sums` the rows of x still lack their norm's
 // division, as for q3_tiles_scaled. Returns Q3_DECLINED, and has done nothing, where another kernel is the way:
 // the caller has asked for the library's or the tiled kernel's products alone, the tuner is on (it times those),
 // the size is not the kernel's, or the weight is so small that other kernels serve these rows better.
 constexpr size_t STREAM_LEAST_WEIGHT_BYTES = 24u << 20;
+
+// Whether the streaming kernel is the way for this product under the current settings, and how (the lock is held).
+// Up to 16 rows only a gate/up product that runs whole and gives at least three CUs in four a block is taken:
+// everything else there is the few-row kernel's.
+static bool stream_plan_locked(int M, int N, int K, bool swiglu, stream::Plan& plan) {
+  if (g_kernels != KERNELS_BOTH || g_mode != MODE_RULE) return false;
+  if (!stream::takes(M, N, K) || (size_t)N * K * 2 < STREAM_LEAST_WEIGHT_BYTES) return false;
+  if (M <= 16) {
+    if (!swiglu || ((N + 15) / 16 + 5) / 6 < 192) return false;
+    plan.ws = 6;
+    plan.splits = 1;
+    return true;
+  }
+  plan = stream::plan_for(M, N, K, false);
+  return plan.splits == 1 || (N % 4 == 0 && (size_t)plan.splits * M * N * sizeof(float) <= PARTIALS_BYTES);
+}
 
 extern "C" int q3_stream_product(const void* x, const void* wt, void* out, int M, int N, int K, int out_dtype,
                                  int epilogue, const float* sums, int chunks, int sums_stride, float eps, int width,
@@ -666,10 +682,8 @@ extern "C" int q3_stream_product(const void* x, const void* wt, void* out, int M
   if (sums && (chunks < 1 || sums_stride < M || width != K)) return Q3_ERR_BAD_ARGUMENT;
   hipStream_t stream = (hipStream_t)stream_;
   std::lock_guard<std::mutex> hold(g_lock);
-  if (g_kernels != KERNELS_BOTH || g_mode != MODE_RULE) return Q3_DECLINED;
-  if (!stream::takes(M, N, K) || (size_t)N * K * 2 < STREAM_LEAST_WEIGHT_BYTES) return Q3_DECLINED;
-  const stream::Plan plan = stream::plan_for(M, N, K, false);
-  if (plan.splits > 1 && (N % 4 || (size_t)plan.splits * M * N * sizeof(float) > PARTIALS_BYTES)) return Q3_DECLINED;
+  stream::Plan plan;
+  if (!stream_plan_locked(M, N, K, swiglu, plan)) return Q3_DECLINED;
   int device = 0;
   HIP_TRY(hipGetDevice(&device));
   Device& d = g_devices[device];
@@ -691,12 +705,10 @@ extern "C" int q3_stream_product(const void* x, const void* wt, void* out, int M
 
 // How q3_stream_product would lay a product over the chip (info[0] slabs per block, info[1] shares of K);
 // 0 is returned for a size it declines under the current settings.
-extern "C" int q3_stream_plan(int M, int N, int K, int* info) {
+extern "C" int q3_stream_plan(int M, int N, int K, int swiglu, int* info) {
   std::lock_guard<std::mutex> hold(g_lock);
-  if (g_kernels != KERNELS_BOTH || g_mode != MODE_RULE) return 0;
-  if (!stream::takes(M, N, K) || (size_t)N * K * 2 < STREAM_LEAST_WEIGHT_BYTES) return 0;
-  const stream::Plan plan = stream::plan_for(M, N, K, false);
-  if (plan.splits > 1 && (N % 4 || (size_t)plan.splits * M * N * sizeof(float) > PARTIALS_BYTES)) return 0;
+  stream::Plan plan;
+  if (!stream_plan_locked(M, N, K, swiglu != 0, plan)) return 0;
   info[0] = plan.ws;
   info[1] = plan.splits;
   return 1;

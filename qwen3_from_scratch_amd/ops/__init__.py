@@ -599,13 +599,16 @@ def _tiles_scaled(x, weight, out, unscaled, swiglu, what):
 STREAM_ROWS_MOST = 96
 
 
-def stream_plan(M, N, K):
-    """How the weight-streaming kernel for 17 to 96 rows would serve a product with a tile-ordered
-    weight of (N, K) under the current settings: (slabs of 16 weight rows per block, shares of K),
-    or None where it leaves the product to the other kernels (small weights, `matmul_kernels`
-    other than "both", the tuner on)."""
+STREAM_ROWS_LEAST = 9      # of a gate/up product that runs whole; every other product from 17 rows
+
+
+def stream_plan(M, N, K, swiglu=False):
+    """How the weight-streaming kernel for 17 to 96 rows (9 to 96 of a gate/up product with the
+    activation) would serve a product with a tile-ordered weight of (N, K) under the current
+    settings: (slabs of 16 weight rows per block, shares of K), or None where it leaves the
+    product to the other kernels (small weights, `matmul_kernels` other than "both", the tuner on)."""
     info = (ctypes.c_int * 2)()
-    if not _matmul().q3_stream_plan(int(M), int(N), int(K), info):
+    if not _matmul().q3_stream_plan(int(M), int(N), int(K), 1 if swiglu else 0, info):
         return None
     return int(info[0]), int(info[1])
 
@@ -614,7 +617,8 @@ def _stream_product(x, weight, tiled, out, swiglu, unscaled, what):
     """The product by the weight-streaming kernel, if it takes it: True if `out` is written."""
     M, K = x.shape
     N = weight.shape[0]
-    if tiled is None or not FEW_ROWS < M <= STREAM_ROWS_MOST or K % 32 or not x.is_contiguous() or not out.is_contiguous():
+    least = STREAM_ROWS_LEAST if swiglu else FEW_ROWS + 1
+    if tiled is None or not least <= M <= STREAM_ROWS_MOST or K % 32 or not x.is_contiguous() or not out.is_contiguous():
         return False
     _need(tiled.is_cuda and tiled.dtype == torch.bfloat16 and tiled.is_contiguous()
           and tiled.numel() == (-(-N // 16) * 16) * K, "the tiled copy does not belong to this weight")
@@ -718,6 +722,13 @@ def linear_swiglu(x, weight, tiled=None, unscaled=None):
     _need(x.dtype in _DT and weight.dtype == x.dtype, "x and weight must share bfloat16 or float32")
     M, K = x.shape
     N = weight.shape[0]
+    if x.dtype == torch.bfloat16 and tiled is not None and STREAM_ROWS_LEAST <= M <= FEW_ROWS and N % 4 == 0:
+        # a whole gate/up product of 9 to 16 rows: the streaming kernel, where it takes the size
+        if unscaled is not None:
+            _need(unscaled[0].dim() == 2 and unscaled[0].shape[1] == sums_stride(M), "row sums (P, M rounded up to 16)")
+        out = torch.empty((M, N // 2), dtype=x.dtype, device=x.device)
+        if _stream_product(x, weight, tiled, out, True, unscaled, "linear_swiglu"):
+            return out
     if M and x.dtype == torch.bfloat16 and _tiled_ok(tiled, weight, M):
         out = torch.empty((M, N // 2), dtype=x.dtype, device=x.device)
         sums, sums_rows, eps, width, stride = _row_sums_args(unscaled, M, K)

@@ -949,6 +949,40 @@ def test_weight_streaming_product_for_some_tens_of_rows(M, N, K):
     assert ops.stream_plan(M, 1024, 4096) is None                  # a small weight: the other kernels' rows
 
 
+@pytest.mark.parametrize("M", [9, 12, 16])
+@pytest.mark.parametrize("I,K,chunks", [(12288, 4096, 256), (9300, 2080, 130), (12288, 4096, 4)])
+def test_gate_up_of_nine_to_sixteen_rows_by_the_streaming_kernel(M, I, K, chunks):
+    """A whole gate/up product of 9 to 16 rows goes to the weight-streaming kernel, with the
+    rows' sums of squares as the few-row kernel leaves them (a partial sum per slab of 16 columns:
+    hundreds of them) or in a few chunks; the same product from the few-row kernel agrees."""
+    ops = _ops()
+    N = 2 * I
+    x = _rand((M, K), torch.bfloat16, 71)
+    w = _rand((N, K), torch.bfloat16, 72, scale=0.05)
+    tiled = ops.tile_weight(w)
+    assert ops.stream_plan(M, N, K, swiglu=True) is not None and ops.stream_plan(M, N, K) is None
+    assert ops.stream_plan(8, N, K, swiglu=True) is None and ops.stream_plan(M, 12000, 2080, swiglu=True) is None
+    sums = torch.zeros((chunks, 16), dtype=torch.float32, device="cuda")
+    sums[:, :M] = (torch.rand((chunks, M), device="cuda") + 0.5) * K / chunks
+    sums[:, M // 2] *= 400.0
+    sums[:, M:] = float("nan")                                      # rows that are not there: never read into a result
+    eps = 1e-6
+    factor = torch.rsqrt(sums[:, :M].double().sum(dim=0) / K + eps)[:, None]
+    exact = x.double() @ w.double().T
+    for unscaled, truth in ((None, exact), ((sums, eps, K), exact * factor)):
+        got = ops.linear_swiglu(x, w, tiled=tiled, unscaled=unscaled)
+        want = torch_ops.swiglu(truth.float().bfloat16().float())
+        assert got.shape == (M, I)
+        assert float((got.float() - want).abs().max()) <= 2e-2 * max(1.0, float(want.abs().max()))
+        assert torch.equal(got, ops.linear_swiglu(x, w, tiled=tiled, unscaled=unscaled))
+        try:
+            ops.matmul_kernels("own")                               # the few-row kernel serves it then
+            other = ops.linear_swiglu(x, w, tiled=tiled, unscaled=unscaled)
+        finally:
+            ops.matmul_kernels("both")
+        torch.testing.assert_close(got.float(), other.float(), rtol=2e-2, atol=2e-2 * max(1.0, float(want.abs().max())))
+
+
 def test_linear_float32_is_true_float32():
     """Inputs whose products need all 24 bits: a matrix mode of reduced precision
     (bf16 or tf32-like splitting) would be off by far more than float32 rounding."""

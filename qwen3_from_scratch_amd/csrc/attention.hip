@@ -1000,9 +1000,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   constexpr int KB4 = TILE / 16;  // 16-key blocks per tile
   __shared__ __attribute__((aligned(16))) unsigned char smem[STAGES * SM::STAGE];
   __shared__ int sh_pages[PREFILL_PAGES];  // the block-table entries of the tiles in hand
-  // and where each entry's (page, this key head) begins in either cache, in elements: worked out
-  // once per entry, so that a tile's loads find their addresses with a few additions
-  __shared__ long long sh_base[PREFILL_PAGES];
+  // and the address at which each entry's (page, this key head) begins in either cache: worked out
+  // once per entry, so that a tile's load finds its address with one read of this table and one
+  // addition of a number the thread keeps for the whole kernel
+  __shared__ long long sh_kaddr[PREFILL_PAGES], sh_vaddr[PREFILL_PAGES];
   const int b = blockIdx.z, g_kv = blockIdx.x;
   const int G = Hq / Hkv;
   const int q0 = cu_q[b];
@@ -1109,9 +1110,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     v_h[j] = q & 1;
   }
   const size_t page_elems = (size_t)page * D;  // elements of one (page, head) in either cache
-  int v_in[V_TURNS];                           // a value piece's place in its page, but for the key's
+  // What a thread keeps per load of a whole tile: where in the address tables its piece's page stands,
+  // counted from the tile's first page, and the piece's byte offset within (page, head). With pages of
+  // fewer keys than a tile the tile begins a page and both are fixed; with larger pages the tile lies
+  // in one page, at an offset that is the same for all threads and is added per tile.
+  const bool small_pages = page < TILE;
+  unsigned k_slot[K_TURNS], k_at[K_TURNS], v_slot[V_TURNS], v_at[V_TURNS];
 #pragma unroll
-  for (int j = 0; j < V_TURNS; ++j) v_in[j] = v_d[j] * page + 8 * v_h[j];
+  for (int j = 0; j < K_TURNS; ++j) {
+    k_slot[j] = small_pages ? 8u * (unsigned)(k_row[j] >> page_shift) : 0u;
+    k_at[j] = 2u * (unsigned)((small_pages ? k_row[j] & (page - 1) : k_row[j]) * D + k_off[j]);
+  }
+#pragma unroll
+  for (int j = 0; j < V_TURNS; ++j) {
+    const int key = 16 * v_kb[j] + 8 * v_h[j];   // the first of the piece's eight keys, from the tile's first
+    v_slot[j] = small_pages ? 8u * (unsigned)(key >> page_shift) : 0u;
+    v_at[j] = 2u * (unsigned)(v_d[j] * page + (small_pages ? key & (page - 1) : key));
+  }
   // A load of 16 bytes per lane that writes shared memory directly: lane L's bytes land at
   // `lds` + 16 L (`lds` the same in all lanes). It is written as assembly on purpose: for the
   // compiler's own form of this instruction the compiler makes every later read of shared
@@ -1131,24 +1146,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // this wavefront's kilobyte of each turn
     const unsigned ks = __builtin_amdgcn_readfirstlane(smem_lds + stage * SM::STAGE + 1024 * wave);
     const unsigned vs = ks + SM::K_BYTES;
+    const unsigned first = 8u * (unsigned)((key0 >> page_shift) - page_base);   // the tile's first page in the tables
+    const unsigned within = small_pages ? 0u : (unsigned)(key0 & (page - 1));   // the tile's first key in its page
+    const unsigned k_in = 2u * within * D, v_in = 2u * within;
+    const char* k_table = reinterpret_cast<const char*>(sh_kaddr) + first;
+    const char* v_table = reinterpret_cast<const char*>(sh_vaddr) + first;
     long long base[K_TURNS + V_TURNS];
-    int key[K_TURNS + V_TURNS];
 #pragma unroll
-    for (int j = 0; j < K_TURNS; ++j) key[j] = key0 + k_row[j];
+    for (int j = 0; j < K_TURNS; ++j) base[j] = *reinterpret_cast<const long long*>(k_table + k_slot[j]);
 #pragma unroll
-    for (int j = 0; j < V_TURNS; ++j) key[K_TURNS + j] = key0 + 16 * v_kb[j];
+    for (int j = 0; j < V_TURNS; ++j) base[K_TURNS + j] = *reinterpret_cast<const long long*>(v_table + v_slot[j]);
 #pragma unroll
-    for (int j = 0; j < K_TURNS + V_TURNS; ++j) base[j] = sh_base[(key[j] >> page_shift) - page_base];
+    for (int j = 0; j < K_TURNS; ++j)
+      load_to_lds(reinterpret_cast<const char*>(base[j]) + (k_at[j] + k_in), ks + 4096 * j);
 #pragma unroll
-    for (int j = 0; j < K_TURNS; ++j) {
-      const int in = (key[j] & (page - 1)) * D + k_off[j];
-      load_to_lds(k_cache + (base[j] + in), ks + 4096 * j);
-    }
-#pragma unroll
-    for (int j = 0; j < V_TURNS; ++j) {
-      const int in = v_in[j] + (key[K_TURNS + j] & (page - 1));
-      load_to_lds(v_cache + (base[K_TURNS + j] + in), vs + 4096 * j);
-    }
+    for (int j = 0; j < V_TURNS; ++j)
+      load_to_lds(reinterpret_cast<const char*>(base[K_TURNS + j]) + (v_at[j] + v_in), vs + 4096 * j);
   };
   auto copy_checked = [&](int t, int stage) {
     const int key0 = t * TILE;
@@ -1225,7 +1238,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       for (int i = tid; page_base + i <= last_page; i += 256) {
         const int pg = bt_row[page_base + i];
         sh_pages[i] = pg;
-        sh_base[i] = (long long)(min(max(pg, 0), num_pages - 1) * Hkv + g_kv) * (long long)page_elems;
+        const long long at = 2 * (long long)(min(max(pg, 0), num_pages - 1) * Hkv + g_kv) * (long long)page_elems;
+        sh_kaddr[i] = reinterpret_cast<long long>(k_cache) + at;
+        sh_vaddr[i] = reinterpret_cast<long long>(v_cache) + at;
       }
     }
     __syncthreads();

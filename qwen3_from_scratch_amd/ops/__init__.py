@@ -447,8 +447,21 @@ def _splits(B, Hkv, max_kv_len):
     until the chip is full, two blocks a compute unit and no more (the blocks beyond 512 run when
     the others have ended: 24 requests of 8 key heads over 768 keys take 27 us in two parts and 31
     in three, 12 requests over 2,000 keys 30 us in five parts and 35 in six); beyond 32 parts the
-    merge costs more than the split gains."""
-    return max(1, min(max_kv_len // 64, 512 // (B * Hkv), 32))
+    merge costs more than the split gains. Two corrections to that, both measured with 8 key heads
+    of 128: with 8,192 keys or more a block's work dwarfs its start and what counts is that the
+    blocks come in even rounds, so at least eight parts are taken up to 384 (sequence, key head)
+    pairs and four beyond (33 sequences over 8,200 keys: 257 us whole, 199 in eight parts; 40: 272
+    and 232; 24: 156 in two parts, 143 in eight; 48: 295 whole, 274 in four; over 32,000 keys 955
+    and 713, 1,022 and 832, 557 and 511, 1,110 and 1,018); and 257 to 320 pairs over fewer keys are
+    split in three (33 sequences over 2,100 keys: 78 us whole, 70 in three; 40: 85 and 78; from 48
+    sequences on one part is the fastest there)."""
+    pairs = B * Hkv
+    splits = max(1, min(max_kv_len // 64, 512 // pairs, 32))
+    if max_kv_len >= 8192 and pairs < 512:
+        splits = max(splits, 8 if pairs <= 384 else 4)
+    elif 256 < pairs <= 320 and max_kv_len >= 1024:
+        splits = 3
+    return splits
 
 
 def decode_attention_takes(num_q_heads, num_kv_heads, head_dim, page_size, dtype, rotary_dim=0):

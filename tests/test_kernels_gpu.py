@@ -736,11 +736,19 @@ def test_linear_from_the_tiled_copy(M, N, K):
     for out_dtype in (torch.bfloat16, torch.float32):
         assert torch.equal(ops.linear(x, w, out_dtype=out_dtype, tiled=tiled), ops.linear(x, w, out_dtype=out_dtype))
     if N % 2 == 0:
-        assert torch.equal(ops.linear_swiglu(x, w, tiled=tiled), ops.linear_swiglu(x, w))
+        act, want = ops.linear_swiglu(x, w, tiled=tiled), ops.linear_swiglu(x, w)
+        if ops.stream_plan(M, N, K, swiglu=True) is None:
+            assert torch.equal(act, want)
+        else:       # a whole gate/up product of 9 to 16 rows is the streaming kernel's: another order of the sums
+            torch.testing.assert_close(act.float(), want.float(), rtol=2e-2, atol=2e-2 * float(want.float().abs().max()))
     assert ops.tile_weight(_rand((8, 72), torch.bfloat16, 1)) is None       # K not a multiple of 32
     assert ops.tile_weight(w.float()) is None
-    many = _rand((40, K), torch.bfloat16, 25)                                 # many rows ignore the copy
-    assert torch.equal(ops.linear(many, w, tiled=tiled), ops.linear(many, w))
+    many = _rand((40, K), torch.bfloat16, 25)
+    got, plain = ops.linear(many, w, tiled=tiled), ops.linear(many, w)
+    if ops.stream_plan(40, N, K) is None:                                      # many rows of a small weight ignore the copy
+        assert torch.equal(got, plain)
+    else:                                                                      # a large one is streamed from it: other sums' order
+        torch.testing.assert_close(got.float(), plain.float(), rtol=2e-2, atol=2e-2 * float(plain.float().abs().max()))
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -910,7 +910,17 @@ __global__ __launch_bounds__(256) void attn_decode_reduce_kernel(
 #define PREFILL_PAGES 512
 // (measured for one 2,048-token prompt at head size 128: 64-key tiles in two stages 94 us, 32-key
 // tiles in four stages, which have three tiles on their way, 116 us; three stages of 64 keys
-// leave room for one block a CU only, 184 us)
+// leave room for one block a CU only, 184 us. With the address tables in shared memory, which took
+// some hundred vector instructions per tile out of the copies: 78 us, and 682 for 8,192 tokens.
+// The same kernel rewritten around v_mfma_f32_32x32x16_bf16 (a wavefront's 32 rows one operand, the
+// two lanes of a row exchanging runs of four probabilities by v_permlane32_swap so that each holds
+// eight consecutive keys, values as D rows of 64 keys in shared memory) was correct and took 71 us
+// and 690, 9,100 for 32,768 tokens; with blocks of 256 rows, eight wavefronts and three stages,
+// which halve the tiles' traffic from the L2 to the CUs, 90, 698 and 8,960. So neither the matrix
+// instruction's rate nor that traffic is what bounds it: per wavefront and tile the matrix pipe is
+// busy about 1,050 to 1,800 cycles, the vector unit about 1,200, and a wavefront takes 6,400 with
+// two wavefronts a SIMD, the phases of a block's four wavefronts tied together by the barrier of
+// every tile. The rewrite was not kept: its gain is within what boxes differ by from 4,096 tokens on.)
 #define PF_TILE 64    // keys per tile
 #define PF_STAGES 2  // tiles in shared memory: one being worked on, the others on their way
 template <int D, int TILE>

@@ -16,23 +16,30 @@
 // into MT accumulators of 16 x 16, the weight of the next chunk already on its way. The two
 // wavefronts of a slab add up through shared memory in a fixed order. One barrier per chunk.
 //
-// K may be shared out over gridDim.y blocks per slab group (float32 partial products, added by
-// tiles::gemm_tiles_reduce_kernel in a fixed order), which is how a product with few slabs fills
-// the chip; a product with many (the gate/up projection) runs whole, with the epilogues of
-// tiles::store_tile: the division by the rows' root mean square that the norm before it left out,
-// SwiGLU over interleaved (gate, up) rows, bfloat16 or float32 output.
+// The product runs whole (no shares of K, no second kernel), with the epilogues of tiles::store_tile:
+// the division by the rows' root mean square that the norm before it left out, SwiGLU over interleaved
+// (gate, up) rows, bfloat16 or float32 output. It is taken where its blocks fill the chip in one round
+// (see slabs_per_block): a block holds a CU alone, all blocks take the same time, and what a second, partly
+// filled round costs is more than the kernel saves.
 //
 // With 9 to 16 rows the few-row kernel of gemm.hip fetches x per slab (or per pair of slabs) and that
 // traffic slows it (gate/up 42.5 us at 12 rows, 44.7 at 16); this kernel takes 40 us at any of them, and
 // serves that product there too. Below nine rows the few-row kernel is as fast or faster, and the products
 // with fewer slabs would need their K shared out and a second kernel, which costs more than it saves.
 //
-// Measured on the 8B layer's gate/up product (24,576 x 4,096, 201 MB) with cold caches, this
-// kernel alone: 40 us at 24 to 48 rows, 42 at 64, 50 at 96 (the vendor library's product: 45, 42,
-// 49, 48, 70, without the activation); with the weight loads alone and no arithmetic 42 at 64
-// rows, so it is the stream that takes the time. Blocks of four slabs are some microseconds slower
-// on it, two slabs per wavefront the same; starting every block at another chunk changes nothing.
-// K must be a multiple of 32 (the tile-ordered copy has no other), N of 4 (of 2 with SwiGLU).
+// Measured with cold caches, weights in turn, against the other route for these rows (for a layer's products
+// the tiled kernel of gemm_tiles.h with K shared out and its adding kernel, for the vocabulary's what the
+// table of sizes names), microseconds at 24 / 48 / 64 / 96 rows:
+//   8B gate/up   24,576 x 4,096, 256 blocks of six slabs     41.1 / 42.1 / 44.0 / 53.0   against 46.3 / 53.7 / 52.8 / 61.1
+//   14B gate/up  34,816 x 5,120, 544 blocks of four          80.3 / 86.0 / 94.2 / 122.7  against 69.2 / 76.6 / 77.4 / 97.1
+//   32B gate/up  51,200 x 5,120, 534 blocks of six          113.6 / 121.0 / 130.0 / 160.5 against 101.2 / 108.9 / 111.3 / 144.5
+//   vocabulary   151,936 x 4,096, 1,583 blocks of six       234.6 / 253.1 / 270.9 / 319.3 against 230.2 / 240.3 / 247.6 / 270.6
+//   q/k/v with K in two to five shares and a second kernel: equal on the 8B layer, a tenth slower on the others.
+// So it wins where one round of blocks covers the product and loses beyond; shares of K never paid, and the
+// kernel has none. With the weight loads alone and no arithmetic the 8B gate/up product takes 42 us at 64 rows,
+// so it is the stream that takes the time. Two slabs per wavefront: the same; starting every block at another
+// chunk changes nothing.
+// K must be a multiple of 32 (the tile-ordered copy has no other), N of 2.
 #pragma once
 
 #include "gemm_tiles.h"
@@ -59,8 +66,7 @@ constexpr int smem_bytes(int MT, int WS) {
 template <typename OUT, int EPI, int MT, int WS>
 __global__ __launch_bounds__(WS * WK * 64) void gemm_stream_kernel(const bf16_t* __restrict__ x,
                                                                    const bf16_t* __restrict__ wt, OUT* __restrict__ out,
-                                                                   int M, int N, int K, int k_per_block,
-                                                                   float* __restrict__ partials, RowScale scale) {
+                                                                   int M, int N, int K, RowScale scale) {
   constexpr int THREADS = WS * WK * 64;
   constexpr int ROWS = MT * 16;
   constexpr int PIECES = ROWS * KCB / 8;                        // 16-byte pieces of a chunk of x
@@ -72,9 +78,7 @@ __global__ __launch_bounds__(WS * WK * 64) void gemm_stream_kernel(const bf16_t*
   const int slabs = (N + 15) / 16;
   const int slab = blockIdx.x * WS + ws;
   const bool slab_ok = slab < slabs;
-  const int kb = blockIdx.y * k_per_block;
-  const int ke = min(K, kb + k_per_block);
-  const int chunks = (ke - kb + KCB - 1) / KCB;
+  const int chunks = (K + KCB - 1) / KCB;
   const bf16_t* wp = wt + (size_t)(slab_ok ? slab : 0) * (K / 32) * 512 + lane * 8;
 
   f32x4_t acc[MT][1];
@@ -82,20 +86,20 @@ __global__ __launch_bounds__(WS * WK * 64) void gemm_stream_kernel(const bf16_t*
   for (int t = 0; t < MT; ++t) acc[t][0] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
   auto load_w = [&](Frag (&a)[STEPS], int c) {
-    const int k0 = kb + c * KCB + wk * KC;
+    const int k0 = c * KCB + wk * KC;
 #pragma unroll
     for (int s = 0; s < STEPS; ++s) {
       const int k = k0 + 32 * s;
-      a[s].u = (slab_ok && k < ke) ? *reinterpret_cast<const uint4*>(wp + (size_t)(k / 32) * 512) : make_uint4(0, 0, 0, 0);
+      a[s].u = (slab_ok && k < K) ? *reinterpret_cast<const uint4*>(wp + (size_t)(k / 32) * 512) : make_uint4(0, 0, 0, 0);
     }
   };
   auto load_x = [&](uint4 (&r)[PER_THREAD], int c) {
-    const int k0 = kb + c * KCB;
+    const int k0 = c * KCB;
 #pragma unroll
     for (int i = 0; i < PER_THREAD; ++i) {
       const int piece = threadIdx.x + i * THREADS;
       const int row = piece / (KCB / 8), k = k0 + (piece % (KCB / 8)) * 8;
-      r[i] = (piece < PIECES && row < M && k < ke) ? *reinterpret_cast<const uint4*>(x + (size_t)row * K + k)
+      r[i] = (piece < PIECES && row < M && k < K) ? *reinterpret_cast<const uint4*>(x + (size_t)row * K + k)
                                                    : make_uint4(0, 0, 0, 0);
     }
   };
@@ -124,13 +128,13 @@ __global__ __launch_bounds__(WS * WK * 64) void gemm_stream_kernel(const bf16_t*
   load_w(even, 0);
   load_x(staged, 0);
   // the rows' factors while the first loads are on their way: the partial sums of squares (few chunks of
-  // 1,024 columns from the kernel that adds shares of K, hundreds of slabs from the few-row kernel) are
+  // 1,024 columns from the kernel that adds the tiled kernel's shares of K, hundreds of slabs from the few-row kernel) are
   // added by the whole block, thread (g, r) the chunks g, g + G, ... of row r, then the G sums of a row in
   // their order: a fixed order of additions
   float factor[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) factor[t] = 1.f;
-  if (scale.sums && !partials) {
+  if (scale.sums) {
     __shared__ float part[THREADS];
     constexpr int G = THREADS / ROWS;
     const int r = threadIdx.x % ROWS, g = threadIdx.x / ROWS;
@@ -178,52 +182,26 @@ __global__ __launch_bounds__(WS * WK * 64) void gemm_stream_kernel(const bf16_t*
   if (wk > 0 || !slab_ok) return;
 #pragma unroll
   for (int t = 0; t < MT; ++t) acc[t][0] += *reinterpret_cast<const f32x4_t*>(sums + ((ws * MT + t) * 64 + lane) * 4);
-  if (partials)
-    tiles::store_tile<float, tiles::EPI_PLAIN, MT, 1>(acc, partials + (size_t)blockIdx.y * M * N, M, N, 0, slab * 16, col,
-                                                      grp, factor);
-  else
-    tiles::store_tile<OUT, EPI, MT, 1>(acc, out, M, N, 0, slab * 16, col, grp, factor);
+  tiles::store_tile<OUT, EPI, MT, 1>(acc, out, M, N, 0, slab * 16, col, grp, factor);
 }
 
-// How a product is laid over the chip: blocks of `ws` slabs (6 or 4), K in `splits` shares.
-struct Plan {
-  int ws = 0, splits = 1;
-};
-
-// By a model of the kernel's time, not a stopwatch (the same for every process): a block streams its
-// share of the weight at what one CU draws from memory (about 21 GB/s), blocks beyond one per CU wait for
-// the next round (with more than two rounds the rounds blur, and the chip's rate is what counts), shares of
-// K cost their float32 partial products written and read once and a second kernel. Blocks of six slabs win
-// a tie. 8B layer at 64 rows: gate/up 6 slabs whole (256 blocks), q/k/v 6 slabs in 4 shares (256 blocks),
-// the vocabulary's product 6 slabs whole (1,583 blocks: 265 us, with blocks of four slabs 270).
-inline Plan plan_for(int M, int N, int K, bool second_kernel_anyway) {
-  const int slabs = (N + 15) / 16, chunks = (K + KCB - 1) / KCB;
-  Plan best;
-  double best_us = 0.0;
+// How many slabs a block takes (6 or 4) so that the blocks fill the chip's `cus` CUs in one round, at least
+// three CUs in four busy; 0 where neither does. Up to 16 rows blocks of six only (measured: blocks of four
+// are some microseconds slower there).
+inline int slabs_per_block(int M, int N, int cus) {
+  const int slabs = (N + 15) / 16;
   for (int ws : {6, 4}) {
-    const int blocks_n = (slabs + ws - 1) / ws;
-    for (int splits = 1; splits <= 16 && splits <= chunks; ++splits) {
-      const int per = (chunks + splits - 1) / splits;
-      if ((chunks + per - 1) / per != splits) continue;      // the same shares under another name
-      const long blocks = (long)blocks_n * splits;
-      const double rounds = blocks > 512 ? blocks / 256.0 : (double)((blocks + 255) / 256);
-      double us = 3.0 + rounds * ((double)ws * 16 * per * KCB * 2) / 21000.0;
-      if (splits > 1) us += (second_kernel_anyway ? 0.0 : 1.5) + 2.0 * splits * M * (double)N * 4 / 4.0e6;
-      if (best.ws == 0 || us < 0.98 * best_us) {      // a later candidate has to win by something
-        best.ws = ws;
-        best.splits = splits;
-        best_us = us;
-      }
-    }
+    const int blocks = (slabs + ws - 1) / ws;
+    if (blocks <= cus && 4 * blocks >= 3 * cus) return ws;
+    if (M <= 16) break;
   }
-  return best;
+  return 0;
 }
 
 inline bool takes(int M, int N, int K) { return M > 8 && M <= MOST_ROWS && N >= 16 && K >= KCB && K % 32 == 0 && N % 2 == 0; }
 
 template <typename OUT, int EPI, int MT, int WS>
-int launch_shape(const void* x, const void* wt, void* out, int M, int N, int K, int splits, float* partials,
-                 hipStream_t stream, const RowScale& scale, bool keep_partials, int* splits_used) {
+int launch_shape(const void* x, const void* wt, void* out, int M, int N, int K, hipStream_t stream, const RowScale& scale) {
   constexpr int SMEM = smem_bytes(MT, WS);
   static bool raised[16] = {};   // the dynamic shared-memory limit, once per device
   int device = 0;
@@ -235,38 +213,21 @@ int launch_shape(const void* x, const void* wt, void* out, int M, int N, int K, 
     if (e != hipSuccess) return (int)e;
     raised[device] = true;
   }
-  const int slabs = (N + 15) / 16, chunks = (K + KCB - 1) / KCB;
-  if (splits < 1 || splits > chunks || splits > 64) return Q3_ERR_BAD_ARGUMENT;
-  const int per = (chunks + splits - 1) / splits;
-  const int used = (chunks + per - 1) / per;      // no block without a chunk
-  const bool to_partials = used > 1 || keep_partials;
-  if (to_partials && (N % 4 || partials == nullptr)) return Q3_ERR_BAD_ARGUMENT;
-  const int blocks_n = (slabs + WS - 1) / WS;
-  if (blocks_n > 65535 * 32) return Q3_ERR_UNSUPPORTED;
-  hipLaunchKernelGGL(kernel, dim3(blocks_n, used), dim3(WS * WK * 64), SMEM, stream, (const bf16_t*)x, (const bf16_t*)wt,
-                     (OUT*)out, M, N, K, per * KCB, to_partials ? partials : nullptr, to_partials ? RowScale() : scale);
-  if (splits_used) *splits_used = used;
-  if (to_partials && !keep_partials) {
-    const size_t quads = (size_t)M * N / 4;
-    hipLaunchKernelGGL((tiles::gemm_tiles_reduce_kernel<OUT, EPI == tiles::EPI_SWIGLU>), dim3((unsigned)((quads + 255) / 256)),
-                       dim3(256), 0, stream, partials, (OUT*)out, quads, N / 4, used, scale);
-  }
+  const int blocks = ((N + 15) / 16 + WS - 1) / WS;
+  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(WS * WK * 64), SMEM, stream, (const bf16_t*)x, (const bf16_t*)wt,
+                     (OUT*)out, M, N, K, scale);
   return q3_launch_status();
 }
 
-// x (M, K) row-major, wt the tile-ordered copy of w (N, K); see tiles::launch for `splits`, `partials`,
-// `scale`, `keep_partials`.
+// x (M, K) row-major, wt the tile-ordered copy of w (N, K), `ws` slabs per block; `scale` as for tiles::launch.
 template <typename OUT, int EPI>
-int launch(const Plan& plan, const void* x, const void* wt, void* out, int M, int N, int K, float* partials,
-           hipStream_t stream, const RowScale& scale = RowScale(), bool keep_partials = false,
-           int* splits_used = nullptr) {
-  if (!takes(M, N, K) || (plan.ws != 6 && plan.ws != 4)) return Q3_ERR_BAD_ARGUMENT;
+int launch(int ws, const void* x, const void* wt, void* out, int M, int N, int K, hipStream_t stream,
+           const RowScale& scale = RowScale()) {
+  if (!takes(M, N, K) || (ws != 6 && ws != 4)) return Q3_ERR_BAD_ARGUMENT;
   const int mt = (M + 15) / 16;
-#define Q3_STREAM_SHAPE(MT_)                                                                                        \
-  return plan.ws == 6 ? launch_shape<OUT, EPI, MT_, 6>(x, wt, out, M, N, K, plan.splits, partials, stream, scale,   \
-                                                       keep_partials, splits_used)                                  \
-                      : launch_shape<OUT, EPI, MT_, 4>(x, wt, out, M, N, K, plan.splits, partials, stream, scale,   \
-                                                       keep_partials, splits_used)
+#define Q3_STREAM_SHAPE(MT_)                                                                   \
+  return ws == 6 ? launch_shape<OUT, EPI, MT_, 6>(x, wt, out, M, N, K, stream, scale)          \
+                 : launch_shape<OUT, EPI, MT_, 4>(x, wt, out, M, N, K, stream, scale)
   switch (mt) {
     case 1: Q3_STREAM_SHAPE(1);
     case 2: Q3_STREAM_SHAPE(2);

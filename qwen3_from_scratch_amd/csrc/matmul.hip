@@ -653,23 +653,31 @@ extern "C" int q3_tiles_residual(const void* x, const void* w, int M, int N, int
 // out (M, N / 2) bfloat16 = silu(gate) * up (`epilogue` 1). With `sums` the rows of x still lack their norm's
 // division, as for q3_tiles_scaled. Returns Q3_DECLINED, and has done nothing, where another kernel is the way:
 // the caller has asked for the library's or the tiled kernel's products alone, the tuner is on (it times those),
-// the size is not the kernel's, or the weight is so small that other kernels serve these rows better.
+// the size is not the kernel's, the weight is so small that other kernels serve these rows better, or its slabs
+// do not fill the chip in one round of blocks.
 constexpr size_t STREAM_LEAST_WEIGHT_BYTES = 24u << 20;
 
-// Whether the streaming kernel is the way for this product under the current settings, and how (the lock is held).
-// Up to 16 rows only a gate/up product that runs whole and gives at least three CUs in four a block is taken:
-// everything else there is the few-row kernel's.
-static bool stream_plan_locked(int M, int N, int K, bool swiglu, stream::Plan& plan) {
-  if (g_kernels != KERNELS_BOTH || g_mode != MODE_RULE) return false;
-  if (!stream::takes(M, N, K) || (size_t)N * K * 2 < STREAM_LEAST_WEIGHT_BYTES) return false;
-  if (M <= 16) {
-    if (!swiglu || ((N + 15) / 16 + 5) / 6 < 192) return false;
-    plan.ws = 6;
-    plan.splits = 1;
-    return true;
+// The CUs of the current device (256 where it cannot be asked).
+static int cu_count() {
+  static int cached[16] = {};
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 16) return 256;
+  if (!cached[device]) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || n < 1) n = 256;
+    cached[device] = n;
   }
-  plan = stream::plan_for(M, N, K, false);
-  return plan.splits == 1 || (N % 4 == 0 && (size_t)plan.splits * M * N * sizeof(float) <= PARTIALS_BYTES);
+  return cached[device];
+}
+
+// Whether the streaming kernel is the way for this product under the current settings, and with how many slabs
+// per block (the lock is held): a weight of 24 MB or more whose blocks fill the chip in one round. Up to 16
+// rows only a gate/up product is taken: everything else there is the few-row kernel's.
+static int stream_plan_locked(int M, int N, int K, bool swiglu) {
+  if (g_kernels != KERNELS_BOTH || g_mode != MODE_RULE) return 0;
+  if (!stream::takes(M, N, K) || (size_t)N * K * 2 < STREAM_LEAST_WEIGHT_BYTES) return 0;
+  if (M <= 16 && !swiglu) return 0;
+  return stream::slabs_per_block(M, N, cu_count());
 }
 
 extern "C" int q3_stream_product(const void* x, const void* wt, void* out, int M, int N, int K, int out_dtype,
@@ -682,13 +690,8 @@ extern "C" int q3_stream_product(const void* x, const void* wt, void* out, int M
   if (sums && (chunks < 1 || sums_stride < M || width != K)) return Q3_ERR_BAD_ARGUMENT;
   hipStream_t stream = (hipStream_t)stream_;
   std::lock_guard<std::mutex> hold(g_lock);
-  stream::Plan plan;
-  if (!stream_plan_locked(M, N, K, swiglu, plan)) return Q3_DECLINED;
-  int device = 0;
-  HIP_TRY(hipGetDevice(&device));
-  Device& d = g_devices[device];
-  int status = ready_device(d, stream);
-  if (status) return status;
+  const int ws = stream_plan_locked(M, N, K, swiglu);
+  if (!ws) return Q3_DECLINED;
   tiles::RowScale scale;
   if (sums) {
     scale.sums = sums;
@@ -697,21 +700,16 @@ extern "C" int q3_stream_product(const void* x, const void* wt, void* out, int M
     scale.eps = eps;
     scale.inv_width = 1.f / (float)width;
   }
-  if (swiglu) return stream::launch<bf16_t, tiles::EPI_SWIGLU>(plan, x, wt, out, M, N, K, d.partials, stream, scale);
-  if (out_dtype == Q3_F32)
-    return stream::launch<float, tiles::EPI_PLAIN>(plan, x, wt, out, M, N, K, d.partials, stream, scale);
-  return stream::launch<bf16_t, tiles::EPI_PLAIN>(plan, x, wt, out, M, N, K, d.partials, stream, scale);
+  if (swiglu) return stream::launch<bf16_t, tiles::EPI_SWIGLU>(ws, x, wt, out, M, N, K, stream, scale);
+  if (out_dtype == Q3_F32) return stream::launch<float, tiles::EPI_PLAIN>(ws, x, wt, out, M, N, K, stream, scale);
+  return stream::launch<bf16_t, tiles::EPI_PLAIN>(ws, x, wt, out, M, N, K, stream, scale);
 }
 
-// How q3_stream_product would lay a product over the chip (info[0] slabs per block, info[1] shares of K);
-// 0 is returned for a size it declines under the current settings.
-extern "C" int q3_stream_plan(int M, int N, int K, int swiglu, int* info) {
+// How q3_stream_product would lay a product over the chip: the slabs per block, or 0 for a size it declines
+// under the current settings.
+extern "C" int q3_stream_plan(int M, int N, int K, int swiglu) {
   std::lock_guard<std::mutex> hold(g_lock);
-  stream::Plan plan;
-  if (!stream_plan_locked(M, N, K, swiglu != 0, plan)) return 0;
-  info[0] = plan.ws;
-  info[1] = plan.splits;
-  return 1;
+  return stream_plan_locked(M, N, K, swiglu != 0);
 }
 
 // The hand-written tiled kernel alone (gemm_tiles.h), tile shape `config` (0 .. q3_gemm_tiles_configs() - 1):

@@ -618,12 +618,11 @@ STREAM_ROWS_LEAST = 9      # of a gate/up product that runs whole; every other p
 def stream_plan(M, N, K, swiglu=False):
     """How the weight-streaming kernel for 17 to 96 rows (9 to 96 of a gate/up product with the
     activation) would serve a product with a tile-ordered weight of (N, K) under the current
-    settings: (slabs of 16 weight rows per block, shares of K), or None where it leaves the
-    product to the other kernels (small weights, `matmul_kernels` other than "both", the tuner on)."""
-    info = (ctypes.c_int * 2)()
-    if not _matmul().q3_stream_plan(int(M), int(N), int(K), 1 if swiglu else 0, info):
-        return None
-    return int(info[0]), int(info[1])
+    settings: the slabs of 16 weight rows per block (6 or 4), or None where it leaves the product
+    to the other kernels (small weights, slabs that do not fill the chip in one round of blocks,
+    `matmul_kernels` other than "both", the tuner on)."""
+    ws = _matmul().q3_stream_plan(int(M), int(N), int(K), 1 if swiglu else 0)
+    return int(ws) if ws else None
 
 
 def _stream_product(x, weight, tiled, out, swiglu, unscaled, what):

@@ -901,20 +901,18 @@ def test_linear_residual_norm_and_unscaled_rows_beyond_sixteen(M, H, K, N2, norm
 
 
 @pytest.mark.parametrize("M", [17, 32, 33, 50, 64, 80, 96])
-@pytest.mark.parametrize("N,K", [(3400, 4000), (9000, 1440), (24576, 4096), (1540, 12288)])
+@pytest.mark.parametrize("N,K", [(24576, 4096), (20002, 1440), (16384, 1024), (12288, 4000)])
 def test_weight_streaming_product_for_some_tens_of_rows(M, N, K):
-    """17 to 96 rows against a weight of 24 MB or more, from its tile-ordered copy: plain in bfloat16
-    and float32, with the rows' division by their rms, and with SwiGLU; K that is no multiple of a
-    chunk (256) or of 64, N that is no multiple of 16, few slabs (K shared out, the shares added by
-    a second kernel) and many (one pass, the epilogue in the kernel). Against float64 sums."""
+    """17 to 96 rows against a weight of 24 MB or more whose slabs fill the chip in one round of blocks,
+    from its tile-ordered copy: plain in bfloat16 and float32, with the rows' division by their rms, and
+    with SwiGLU; K that is no multiple of a chunk (256) or of 64, N that is no multiple of 16, blocks of
+    six slabs and of four. Against float64 sums."""
     ops = _ops()
     x = _rand((M, K), torch.bfloat16, 61)
     w = _rand((N, K), torch.bfloat16, 62, scale=0.05)
     tiled = ops.tile_weight(w)
     plan = ops.stream_plan(M, N, K)
-    assert plan is not None and plan[0] in (4, 6) and 1 <= plan[1] <= 16
-    if (N, K) == (24576, 4096):
-        assert plan == (6, 1)                                      # whole: 256 blocks of six slabs
+    assert plan == {24576: 6, 20002: 6, 16384: 4, 12288: 4}[N]     # 256, 209, 256 and 192 blocks
     exact = x.double() @ w.double().T
     scale = float(exact.abs().max())
     got32 = ops.linear(x, w, out_dtype=torch.float32, tiled=tiled)
@@ -955,6 +953,9 @@ def test_weight_streaming_product_for_some_tens_of_rows(M, N, K):
         ops.matmul_kernels("both")
     assert ops.stream_plan(16, N, K) is None and ops.stream_plan(97, N, K) is None
     assert ops.stream_plan(M, 1024, 4096) is None                  # a small weight: the other kernels' rows
+    # slabs that would leave CUs idle (36 blocks) or need a second round (544, 1,583): the other kernels'
+    assert ops.stream_plan(M, 3400, 4000) is None and ops.stream_plan(M, 34816, 5120) is None
+    assert ops.stream_plan(M, 151936, 4096) is None
 
 
 @pytest.mark.parametrize("M", [9, 12, 16])
@@ -968,8 +969,9 @@ def test_gate_up_of_nine_to_sixteen_rows_by_the_streaming_kernel(M, I, K, chunks
     x = _rand((M, K), torch.bfloat16, 71)
     w = _rand((N, K), torch.bfloat16, 72, scale=0.05)
     tiled = ops.tile_weight(w)
-    assert ops.stream_plan(M, N, K, swiglu=True) is not None and ops.stream_plan(M, N, K) is None
+    assert ops.stream_plan(M, N, K, swiglu=True) == 6 and ops.stream_plan(M, N, K) is None
     assert ops.stream_plan(8, N, K, swiglu=True) is None and ops.stream_plan(M, 12000, 2080, swiglu=True) is None
+    assert ops.stream_plan(M, 34816, 5120, swiglu=True) is None      # 363 blocks: more than one round
     sums = torch.zeros((chunks, 16), dtype=torch.float32, device="cuda")
     sums[:, :M] = (torch.rand((chunks, M), device="cuda") + 0.5) * K / chunks
     sums[:, M // 2] *= 400.0

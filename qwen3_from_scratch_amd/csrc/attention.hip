@@ -917,10 +917,12 @@ __global__ __launch_bounds__(256) void attn_decode_reduce_kernel(
 // eight consecutive keys, values as D rows of 64 keys in shared memory) was correct and took 71 us
 // and 690, 9,100 for 32,768 tokens; with blocks of 256 rows, eight wavefronts and three stages,
 // which halve the tiles' traffic from the L2 to the CUs, 90, 698 and 8,960. So neither the matrix
-// instruction's rate nor that traffic is what bounds it: per wavefront and tile the matrix pipe is
-// busy about 1,050 to 1,800 cycles, the vector unit about 1,200, and a wavefront takes 6,400 with
-// two wavefronts a SIMD, the phases of a block's four wavefronts tied together by the barrier of
-// every tile. The rewrite was not kept: its gain is within what boxes differ by from 4,096 tokens on.)
+// instruction's form nor that traffic is what bounds it. Time stamps around the phases of one wavefront
+// (the kernel runs at 1.77 GHz): per tile the copy's issue 580 cycles, the first product 870, the softmax
+// 1,360, the second product 880, waits 160, about 4,600 with the loop around them, in which the SIMD serves
+// two wavefronts; the 64 matrix instructions of a tile take 1,024 cycles of the matrix pipe and its 265
+// other vector instructions about 1,200 of the vector unit: each works about half the time, and they
+// overlap only in part. The rewrite was not kept: its gain is within what boxes differ by from 4,096 tokens on.)
 #define PF_TILE 64    // keys per tile
 #define PF_STAGES 2  // tiles in shared memory: one being worked on, the others on their way
 template <int D, int TILE>

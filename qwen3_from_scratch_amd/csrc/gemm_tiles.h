@@ -23,7 +23,7 @@
 // of the cycles, no bank conflicts), the vendor library's best kernel 279. So it is the copies'
 // passage itself, not their latency, that takes the time from the operand reads. The other
 // matrix instruction, v_mfma_f32_32x32x16_bf16, runs at 2.4 PFLOP/s from registers where
-// this kernel's 16 x 16 x 32 runs at 1.4 (one wavefront a SIMD: 2.1 against 0.8), but in this
+// this kernel's 16 x 16 x 32 runs at 2.2 (one wavefront a SIMD: 2.25 against 1.8), and in this
 // kernel it changed nothing (256 x 256 tiles 417 us beside the library's 312 on a box where the
 // 16 x 16 x 32 form took about 375; no bank conflicts, the matrix pipes busy 39 % of the time):
 // the time goes to the wait for each step's copies with only two stages in flight, not to

@@ -960,14 +960,14 @@ __device__ __forceinline__ void softmax_tile(const f32x4_t (&s)[KB4], bool full,
 #pragma unroll
   for (int j = 0; j < N; ++j) v[j] = s[j >> 2][j & 3];
   if (!full) {
-    // (the row's position goes through an empty piece of assembly so that the comparisons'
-    // operands are worked out here, where they are needed, and not before the branch for
+    // (the row's position and the lane's first key go through an empty piece of assembly so that the
+    // comparisons' operands are worked out here, where they are needed, and not before the branch for
     // every tile)
-    int pos = row_pos;
-    asm volatile("" : "+v"(pos));
+    int pos = row_pos, first_key = key0 + 4 * grp;
+    asm volatile("" : "+v"(pos), "+v"(first_key));
 #pragma unroll
     for (int j = 0; j < N; ++j) {
-      const int key = key0 + 16 * (j >> 2) + 4 * grp + (j & 3);
+      const int key = first_key + 16 * (j >> 2) + (j & 3);
       bool seen = key <= pos;
       if (window > 0 && pos - key >= window) seen = false;
       if (!seen) v[j] = -INFINITY;
@@ -975,12 +975,22 @@ __device__ __forceinline__ void softmax_tile(const f32x4_t (&s)[KB4], bool full,
   }
   // the scores are matrix results or minus infinity, never NaN: the three-operand maximum as
   // it is (the compiler's own first makes every operand a quiet NaN, one instruction each)
+  // (one statement for a tile of 64 keys: after every statement of assembly the compiler leaves a wait state)
   float mx;
-  asm("v_max_f32 %0, %1, %2" : "=v"(mx) : "v"(v[0]), "v"(v[1]));
+  if constexpr (N == 16) {
+    asm("v_max_f32 %0, %1, %2\n\tv_max3_f32 %0, %0, %3, %4\n\tv_max3_f32 %0, %0, %5, %6\n\tv_max3_f32 %0, %0, %7, %8\n\t"
+        "v_max3_f32 %0, %0, %9, %10\n\tv_max3_f32 %0, %0, %11, %12\n\tv_max3_f32 %0, %0, %13, %14\n\t"
+        "v_max3_f32 %0, %0, %15, %16"
+        : "=&v"(mx)
+        : "v"(v[0]), "v"(v[1]), "v"(v[2]), "v"(v[3]), "v"(v[4]), "v"(v[5]), "v"(v[6]), "v"(v[7]), "v"(v[8]), "v"(v[9]),
+          "v"(v[10]), "v"(v[11]), "v"(v[12]), "v"(v[13]), "v"(v[14]), "v"(v[15]));
+  } else {
+    asm("v_max_f32 %0, %1, %2" : "=v"(mx) : "v"(v[0]), "v"(v[1]));
 #pragma unroll
-  for (int j = 2; j < N; j += 2) asm("v_max3_f32 %0, %1, %2, %3" : "=v"(mx) : "v"(mx), "v"(v[j]), "v"(v[j + 1]));
-  mx = quad_rows_max(mx);
-  const float m_new = fmaxf(m_run, mx * scale_log2);
+    for (int j = 2; j < N; j += 2) asm("v_max3_f32 %0, %1, %2, %3" : "=v"(mx) : "v"(mx), "v"(v[j]), "v"(v[j + 1]));
+  }
+  mx = quad_rows_max_of_numbers(mx);
+  const float m_new = max_of_numbers(m_run, mx * scale_log2);
   // a row that has seen no key yet has minus infinity here and in all its scores: its terms are
   // exp2(-inf - 0) = 0
   const float m_use = m_new > -INFINITY ? m_new : 0.f;
@@ -1068,6 +1078,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     pos_max = max(pos_max, __shfl_xor(pos_max, off, 64));
     pos_min = min(pos_min, __shfl_xor(pos_min, off, 64));
   }
+  // the same in all lanes: kept as scalars, so that what is decided by them per tile is a scalar branch
+  pos_max = __builtin_amdgcn_readfirstlane(pos_max);
+  pos_min = __builtin_amdgcn_readfirstlane(pos_min);
   f32x4_t acc[2][D / 16];
 #pragma unroll
   for (int qb = 0; qb < 2; ++qb)

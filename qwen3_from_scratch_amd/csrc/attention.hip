@@ -1324,8 +1324,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
           for (int half = 0; half < KB4 / 2; ++half)
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
+            for (int kb = 0; kb < 2; ++kb) {
+              // (an empty statement of assembly after each read keeps it a ds_read_b64 of its own: joined by the
+              // compiler into one ds_read2st64_b64, two addresses a multiple of 512 bytes apart fall into the
+              // same banks, and shared memory takes sixteen cycles per kilobyte, half of them counted as bank
+              // conflicts, where two ds_read_b64 take two cycles each; measured with the read pattern alone.
+              // These reads were four fifths of the kernel's shared-memory time, and shared memory was its
+              // busiest unit.)
               to[half].h[kb] = *reinterpret_cast<const uint2*>(vs + (2 * nb + kb) * SM::VPR * 256 + v_read[half]);
+              asm volatile("" ::: "memory");
+            }
         };
         read_values(0, vt[0]);
         read_values(1, vt[1]);
@@ -1340,12 +1348,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                   __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt[nb & 3][half].v, p[qb][half].v, acc[qb][nb], 0, 0, 0);
         }
         // the order the compiler is to keep (left to itself it reads each operand right before
-        // its use, into the same registers, and waits for it every time): four reads ahead
-        __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+        // its use, into the same registers, and waits for it every time): four operands (two reads each) ahead
+        __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
 #pragma unroll
         for (int i = 0; i < (D / 16) * (KB4 / 2) - 4; ++i) {
           __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
         }
         __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
       }

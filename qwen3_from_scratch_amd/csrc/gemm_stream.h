@@ -54,8 +54,10 @@ constexpr int WK = 2;            // wavefronts that share a slab's chunk
 constexpr int KC = 128;          // k per wavefront per chunk
 constexpr int KCB = KC * WK;     // k per chunk
 constexpr int STEPS = KC / 32;   // matrix instructions per accumulator per chunk
-constexpr int ROW = KCB * 2 + 16;   // bytes of a row of x in shared memory: 16 more than its data, so that the
-                                    // sixteen rows one operand read touches start in different banks
+constexpr int ROW = KCB * 2 + 32;   // bytes of a row of x in shared memory: 32 more than its data. With 16 more the
+                                    // operand reads (16 bytes a lane, sixteen rows a group of lanes) took eight cycles of
+                                    // shared memory each, four of them counted as bank conflicts; with 32 more four and none
+                                    // (measured with the read pattern alone)
 constexpr int MOST_ROWS = 96;
 
 constexpr int smem_bytes(int MT, int WS) {

@@ -30,7 +30,7 @@
 // Measured with cold caches, weights in turn, against the other route for these rows (for a layer's products
 // the tiled kernel of gemm_tiles.h with K shared out and its adding kernel, for the vocabulary's what the
 // table of sizes names), microseconds at 24 / 48 / 64 / 96 rows:
-//   8B gate/up   24,576 x 4,096, 256 blocks of six slabs     41.1 / 42.1 / 44.0 / 53.0   against 46.3 / 53.7 / 52.8 / 61.1
+//   8B gate/up   24,576 x 4,096, 256 blocks of six slabs     40.7 / 41.0 / 41.6 / 47.9   against 46.3 / 53.7 / 52.8 / 61.1
 //   14B gate/up  34,816 x 5,120, 544 blocks of four          80.3 / 86.0 / 94.2 / 122.7  against 69.2 / 76.6 / 77.4 / 97.1
 //   32B gate/up  51,200 x 5,120, 534 blocks of six          113.6 / 121.0 / 130.0 / 160.5 against 101.2 / 108.9 / 111.3 / 144.5
 //   vocabulary   151,936 x 4,096, 1,583 blocks of six       234.6 / 253.1 / 270.9 / 319.3 against 230.2 / 240.3 / 247.6 / 270.6

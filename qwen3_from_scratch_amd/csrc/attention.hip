@@ -1181,12 +1181,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int j = 0; j < K_TURNS; ++j) base[j] = *reinterpret_cast<const long long*>(k_table + k_slot[j]);
 #pragma unroll
     for (int j = 0; j < V_TURNS; ++j) base[K_TURNS + j] = *reinterpret_cast<const long long*>(v_table + v_slot[j]);
+    if (small_pages) {   // a tile begins a page: nothing to add to the thread's own offsets
 #pragma unroll
-    for (int j = 0; j < K_TURNS; ++j)
-      load_to_lds(reinterpret_cast<const char*>(base[j]) + (k_at[j] + k_in), ks + 4096 * j);
+      for (int j = 0; j < K_TURNS; ++j) load_to_lds(reinterpret_cast<const char*>(base[j]) + k_at[j], ks + 4096 * j);
 #pragma unroll
-    for (int j = 0; j < V_TURNS; ++j)
-      load_to_lds(reinterpret_cast<const char*>(base[K_TURNS + j]) + (v_at[j] + v_in), vs + 4096 * j);
+      for (int j = 0; j < V_TURNS; ++j)
+        load_to_lds(reinterpret_cast<const char*>(base[K_TURNS + j]) + v_at[j], vs + 4096 * j);
+    } else {
+#pragma unroll
+      for (int j = 0; j < K_TURNS; ++j)
+        load_to_lds(reinterpret_cast<const char*>(base[j]) + (k_at[j] + k_in), ks + 4096 * j);
+#pragma unroll
+      for (int j = 0; j < V_TURNS; ++j)
+        load_to_lds(reinterpret_cast<const char*>(base[K_TURNS + j]) + (v_at[j] + v_in), vs + 4096 * j);
+    }
   };
   auto copy_checked = [&](int t, int stage) {
     const int key0 = t * TILE;
